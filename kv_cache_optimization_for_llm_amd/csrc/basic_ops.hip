@@ -1,0 +1,189 @@
+// Embedding gather, RMSNorm (optionally fused with the residual add before it and with a row
+// gather), SwiGLU activation and dtype casts.  One workgroup handles one row; all arithmetic
+// is fp32 whatever the storage type is.
+//
+// Formulas follow the reference's kernels: rmsNormKernel (base/src/kernels.cu:10-36),
+// residualKernel (:38-43), siluKernel (:45-52), embeddingGatherKernel (:279-287) and
+// gatherRowsKernel (:472-480).
+#include "common.h"
+#include <stdarg.h>
+#include <stdio.h>
+
+static thread_local char g_error[512] = "";
+
+extern "C" const char *kva_last_error() { return g_error; }
+
+void kva_set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+// ---------------------------------------------------------------------------------------
+template <typename TW, typename TO>
+__global__ void embed_gather_kernel(TO *__restrict__ out, const TW *__restrict__ table,
+                                    const int *__restrict__ ids, int width) {
+    const int row = blockIdx.x;
+    const TW *src = table + (size_t)ids[row] * width;
+    TO *dst = out + (size_t)row * width;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = from_float<TO>(to_float(src[i]));
+}
+
+extern "C" int kva_embed_gather(void *out, const void *table, const int *ids, int rows, int width,
+                                int table_dtype, int out_dtype, hipStream_t stream) {
+    KVA_REQUIRE(rows >= 0 && width > 0, "embed_gather: bad sizes rows=%d width=%d", rows, width);
+    if (rows == 0) return KVA_OK;
+    dim3 grid(rows), block(256);
+#define LAUNCH(TW, TO)                                                                    \
+    hipLaunchKernelGGL((embed_gather_kernel<TW, TO>), grid, block, 0, stream, (TO *)out, \
+                       (const TW *)table, ids, width)
+    if (table_dtype == KVA_F32 && out_dtype == KVA_F32) LAUNCH(float, float);
+    else if (table_dtype == KVA_BF16 && out_dtype == KVA_BF16) LAUNCH(bf16_t, bf16_t);
+    else if (table_dtype == KVA_F32 && out_dtype == KVA_BF16) LAUNCH(float, bf16_t);
+    else if (table_dtype == KVA_BF16 && out_dtype == KVA_F32) LAUNCH(bf16_t, float);
+    else KVA_REQUIRE(false, "embed_gather: unsupported dtypes %d -> %d", table_dtype, out_dtype);
+#undef LAUNCH
+    KVA_CHECK_LAUNCH("embed_gather");
+    return KVA_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// y = (x / sqrt(mean(x^2) + eps)) * w.  The sum of squares is fp32, the sqrt runs in double
+// as the reference's does.  With `delta`, the norm is taken of s = round(hidden + delta) (fp32
+// add, rounded to the storage type), which is what a separate residual kernel followed by a norm
+// kernel would see; s is written back to hidden unless rows are gathered.  With `row_idx`,
+// output row i is the norm of input row row_idx[i] and hidden is left untouched (a row may be
+// named twice).
+template <typename T, typename TW>
+__global__ void rmsnorm_kernel(T *__restrict__ out, T *__restrict__ hidden,
+                               const T *__restrict__ delta, const TW *__restrict__ weight,
+                               const int *__restrict__ row_idx, int width, float eps) {
+    __shared__ float scratch[16];
+    const int orow = blockIdx.x;
+    const int irow = row_idx ? row_idx[orow] : orow;
+    T *x = hidden + (size_t)irow * width;
+    const T *dl = delta ? delta + (size_t)irow * width : nullptr;
+    const bool write_back = dl && !row_idx;
+    T *y = out + (size_t)orow * width;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        float v = to_float(x[i]);
+        if (dl) {
+            const T r = from_float<T>(v + to_float(dl[i]));
+            if (write_back) x[i] = r;
+            v = to_float(r);
+        }
+        ss += v * v;
+    }
+    const float total = block_sum(ss, scratch, blockDim.x / KVA_WAVE);
+    const float r = (float)sqrt((double)total / (double)width + (double)eps);
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        float v = to_float(x[i]);
+        if (dl && !write_back) v = to_float(from_float<T>(v + to_float(dl[i])));
+        y[i] = from_float<T>((v / r) * to_float(weight[i]));
+    }
+}
+
+extern "C" int kva_rmsnorm(void *out, void *hidden, const void *delta, const void *weight,
+                           const int *row_idx, int out_rows, int width, float eps, int dtype,
+                           int weight_dtype, hipStream_t stream) {
+    KVA_REQUIRE(out_rows >= 0 && width > 0, "rmsnorm: bad sizes rows=%d width=%d", out_rows, width);
+    if (out_rows == 0) return KVA_OK;
+    dim3 grid(out_rows), block(width >= 2048 ? 512 : 256);
+#define LAUNCH(T, TW)                                                                      \
+    hipLaunchKernelGGL((rmsnorm_kernel<T, TW>), grid, block, 0, stream, (T *)out, (T *)hidden, \
+                       (const T *)delta, (const TW *)weight, row_idx, width, eps)
+    if (dtype == KVA_F32 && weight_dtype == KVA_F32) LAUNCH(float, float);
+    else if (dtype == KVA_BF16 && weight_dtype == KVA_BF16) LAUNCH(bf16_t, bf16_t);
+    else if (dtype == KVA_BF16 && weight_dtype == KVA_F32) LAUNCH(bf16_t, float);
+    else if (dtype == KVA_F32 && weight_dtype == KVA_BF16) LAUNCH(float, bf16_t);
+    else KVA_REQUIRE(false, "rmsnorm: unsupported dtypes %d / %d", dtype, weight_dtype);
+#undef LAUNCH
+    KVA_CHECK_LAUNCH("rmsnorm");
+    return KVA_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// hidden <- hidden + delta, fp32 add, rounded to the storage type.
+template <typename T>
+__global__ void residual_add_kernel(T *__restrict__ hidden, const T *__restrict__ delta, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) hidden[i] = from_float<T>(to_float(hidden[i]) + to_float(delta[i]));
+}
+
+extern "C" int kva_residual_add(void *hidden, const void *delta, long long n, int dtype,
+                                hipStream_t stream) {
+    KVA_REQUIRE(n >= 0, "residual_add: bad size");
+    if (n == 0) return KVA_OK;
+    int blocks = (int)((n + 255) / 256);
+    if (blocks > 8192) blocks = 8192;
+    if (dtype == KVA_F32)
+        hipLaunchKernelGGL(residual_add_kernel<float>, dim3(blocks), dim3(256), 0, stream,
+                           (float *)hidden, (const float *)delta, (size_t)n);
+    else if (dtype == KVA_BF16)
+        hipLaunchKernelGGL(residual_add_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream,
+                           (bf16_t *)hidden, (const bf16_t *)delta, (size_t)n);
+    else KVA_REQUIRE(false, "residual_add: unsupported dtype %d", dtype);
+    KVA_CHECK_LAUNCH("residual_add");
+    return KVA_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// out[t, i] = silu(gu[t, i]) * gu[t, inter + i]; silu(g) = g / (1 + exp(-g)) in fp32.
+template <typename T>
+__global__ void silu_mul_kernel(T *__restrict__ out, const T *__restrict__ gate_up, int inter) {
+    const int row = blockIdx.y;
+    const T *g = gate_up + (size_t)row * 2 * inter;
+    const T *u = g + inter;
+    T *o = out + (size_t)row * inter;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < inter; i += gridDim.x * blockDim.x) {
+        const float gv = to_float(g[i]);
+        o[i] = from_float<T>(gv * (1.f / (1.f + expf(-gv))) * to_float(u[i]));
+    }
+}
+
+extern "C" int kva_silu_mul(void *out, const void *gate_up, int rows, int inter, int dtype,
+                            hipStream_t stream) {
+    KVA_REQUIRE(rows >= 0 && inter > 0, "silu_mul: bad sizes");
+    KVA_REQUIRE(rows <= 65535, "silu_mul: at most 65535 rows per call, got %d", rows);
+    if (rows == 0) return KVA_OK;
+    int bx = (inter + 255) / 256;
+    if (bx > 64) bx = 64;
+    dim3 grid(bx, rows), block(256);
+    if (dtype == KVA_F32)
+        hipLaunchKernelGGL(silu_mul_kernel<float>, grid, block, 0, stream, (float *)out,
+                           (const float *)gate_up, inter);
+    else if (dtype == KVA_BF16)
+        hipLaunchKernelGGL(silu_mul_kernel<bf16_t>, grid, block, 0, stream, (bf16_t *)out,
+                           (const bf16_t *)gate_up, inter);
+    else KVA_REQUIRE(false, "silu_mul: unsupported dtype %d", dtype);
+    KVA_CHECK_LAUNCH("silu_mul");
+    return KVA_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+template <typename TI, typename TO>
+__global__ void cast_kernel(TO *__restrict__ out, const TI *__restrict__ in, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) out[i] = from_float<TO>(to_float(in[i]));
+}
+
+extern "C" int kva_cast(void *out, const void *in, long long n, int in_dtype, int out_dtype,
+                        hipStream_t stream) {
+    KVA_REQUIRE(n >= 0, "cast: bad size");
+    if (n == 0) return KVA_OK;
+    int blocks = (int)((n + 255) / 256);
+    if (blocks > 8192) blocks = 8192;
+    if (in_dtype == KVA_BF16 && out_dtype == KVA_F32)
+        hipLaunchKernelGGL((cast_kernel<bf16_t, float>), dim3(blocks), dim3(256), 0, stream,
+                           (float *)out, (const bf16_t *)in, (size_t)n);
+    else if (in_dtype == KVA_F32 && out_dtype == KVA_BF16)
+        hipLaunchKernelGGL((cast_kernel<float, bf16_t>), dim3(blocks), dim3(256), 0, stream,
+                           (bf16_t *)out, (const float *)in, (size_t)n);
+    else KVA_REQUIRE(false, "cast: unsupported dtypes %d -> %d", in_dtype, out_dtype);
+    KVA_CHECK_LAUNCH("cast");
+    return KVA_OK;
+}

@@ -1,0 +1,94 @@
+// Shared device helpers for the gfx950 kernels: bf16 storage type, 64-lane wavefront
+// reductions, vector loads and the launch-error convention of the extern "C" entry points.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define KVA_WAVE 64
+
+// Every entry point returns 0 on success or a negative code; the Python side turns the
+// code into an exception with kva_last_error().
+#define KVA_OK 0
+#define KVA_ERR_ARG (-1)
+#define KVA_ERR_LAUNCH (-2)
+
+extern "C" const char *kva_last_error();
+void kva_set_error(const char *fmt, ...);
+
+#define KVA_REQUIRE(cond, ...)                                                             \
+    do {                                                                                   \
+        if (!(cond)) {                                                                     \
+            kva_set_error(__VA_ARGS__);                                                    \
+            return KVA_ERR_ARG;                                                            \
+        }                                                                                  \
+    } while (0)
+
+#define KVA_CHECK_LAUNCH(name)                                                             \
+    do {                                                                                   \
+        hipError_t e_ = hipGetLastError();                                                 \
+        if (e_ != hipSuccess) {                                                            \
+            kva_set_error("%s: launch failed: %s", name, hipGetErrorString(e_));           \
+            return KVA_ERR_LAUNCH;                                                         \
+        }                                                                                  \
+    } while (0)
+
+// ---- bfloat16 as a storage type -------------------------------------------------------
+// All arithmetic is done in float; bf16 is only ever loaded from and stored to memory.
+struct bf16_t {
+    uint16_t bits;
+};
+
+__host__ __device__ inline float bf16_bits_to_float(uint16_t b) {
+    union { uint32_t u; float f; } c;
+    c.u = ((uint32_t)b) << 16;
+    return c.f;
+}
+
+// round to nearest, ties to even; NaN stays NaN
+__host__ __device__ inline uint16_t float_to_bf16_bits(float f) {
+    union { uint32_t u; float f; } c;
+    c.f = f;
+    uint32_t u = c.u;
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+__host__ __device__ inline float to_float(float v) { return v; }
+__host__ __device__ inline float to_float(bf16_t v) { return bf16_bits_to_float(v.bits); }
+
+template <typename T> __host__ __device__ inline T from_float(float f);
+template <> __host__ __device__ inline float from_float<float>(float f) { return f; }
+template <> __host__ __device__ inline bf16_t from_float<bf16_t>(float f) {
+    bf16_t r;
+    r.bits = float_to_bf16_bits(f);
+    return r;
+}
+
+// ---- wavefront (64 lanes) reductions ---------------------------------------------------
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+    for (int off = KVA_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, KVA_WAVE);
+    return v;
+}
+
+__device__ inline float wave_max(float v) {
+#pragma unroll
+    for (int off = KVA_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, KVA_WAVE));
+    return v;
+}
+
+// Sum over a whole workgroup of `nwaves` wavefronts; `scratch` holds at least nwaves floats.
+// Every thread gets the result.  The order of the additions is fixed.
+__device__ inline float block_sum(float v, float *scratch, int nwaves) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x % KVA_WAVE, wave = threadIdx.x / KVA_WAVE;
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float total = 0.f;
+    for (int w = 0; w < nwaves; ++w) total += scratch[w];
+    return total;
+}
+
+enum KvaDtype { KVA_F32 = 0, KVA_BF16 = 1 };

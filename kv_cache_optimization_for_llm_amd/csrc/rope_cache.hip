@@ -1,0 +1,112 @@
+// Rotary position encoding of Q and K fused with the write of K and V into the paged cache.
+//
+// The reference does this in three launches per layer: ropePackedKernel on Q, on K
+// (base/src/kernels.cu:289-319) and scatterKVPackedKernel
+// (paged_attention/src/kernels.cu:335-363).  Pairing is rotate-half: inside a head, element j
+// pairs with j + rot/2 and both use angle index j:
+//     out[j]         = x[j] * cos - x[j + rot/2] * sin
+//     out[j + rot/2] = x[j] * sin + x[j + rot/2] * cos
+// cos and sin come from fp32 tables [max_positions, rot/2] built once on the host.
+// K is rotated BEFORE it is cached, V is cached as it is.
+//
+// Cache layout (both K and V): [num_pages, num_kv_heads, page_size, head_dim]; slot s of the
+// slot mapping is page s / page_size, row s % page_size.  A negative slot skips the write.
+#include "common.h"
+
+template <typename T>
+__global__ void rope_kv_write_kernel(T *__restrict__ qkv, T *__restrict__ k_cache,
+                                     T *__restrict__ v_cache, const float *__restrict__ cos_table,
+                                     const float *__restrict__ sin_table,
+                                     const int *__restrict__ positions,
+                                     const int *__restrict__ slot_mapping, int num_q_heads,
+                                     int num_kv_heads, int head_dim, int rot_dim, int page_size,
+                                     int write_cache) {
+    const int t = blockIdx.x;
+    const int row_width = (num_q_heads + 2 * num_kv_heads) * head_dim;
+    T *row = qkv + (size_t)t * row_width;
+    const int pos = positions[t];
+    const int half = rot_dim / 2;
+    const float *cs = cos_table ? cos_table + (size_t)pos * half : nullptr;
+    const float *sn = sin_table ? sin_table + (size_t)pos * half : nullptr;
+
+    int slot = -1;
+    if (write_cache) slot = slot_mapping[t];
+    const int page = slot >= 0 ? slot / page_size : 0;
+    const int off = slot >= 0 ? slot % page_size : 0;
+
+    // work item = (head among q and k heads, pair index in [0, head_dim/2)); pairs beyond the
+    // rotated part (partial rotary) pass two plain elements through
+    const int pairs_per_head = head_dim / 2;
+    const int qk_heads = num_q_heads + num_kv_heads;
+    for (int w = threadIdx.x; w < qk_heads * pairs_per_head; w += blockDim.x) {
+        const int head = w / pairs_per_head;
+        const int p = w % pairs_per_head;
+        T *h = row + (size_t)head * head_dim;
+        int i1, i2;
+        float o1, o2;
+        if (p < half) {
+            i1 = p;
+            i2 = p + half;
+            const float x1 = to_float(h[i1]), x2 = to_float(h[i2]);
+            if (cs) {
+                const float c = cs[p], s = sn[p];
+                o1 = x1 * c - x2 * s;
+                o2 = x1 * s + x2 * c;
+            } else {
+                o1 = x1;
+                o2 = x2;
+            }
+        } else {
+            i1 = rot_dim + 2 * (p - half);
+            i2 = i1 + 1;
+            o1 = to_float(h[i1]);
+            o2 = to_float(h[i2]);
+        }
+        const T r1 = from_float<T>(o1), r2 = from_float<T>(o2);
+        if (head < num_q_heads) {
+            h[i1] = r1;
+            h[i2] = r2;
+        } else if (slot >= 0) {
+            const int kvh = head - num_q_heads;
+            T *dst = k_cache + (((size_t)page * num_kv_heads + kvh) * page_size + off) * head_dim;
+            dst[i1] = r1;
+            dst[i2] = r2;
+        }
+    }
+    if (slot >= 0) {
+        const T *v = row + (size_t)(num_q_heads + num_kv_heads) * head_dim;
+        for (int w = threadIdx.x; w < num_kv_heads * head_dim; w += blockDim.x) {
+            const int kvh = w / head_dim, j = w % head_dim;
+            v_cache[(((size_t)page * num_kv_heads + kvh) * page_size + off) * head_dim + j] = v[w];
+        }
+    }
+}
+
+extern "C" int kva_rope_kv_write(void *qkv, void *k_cache, void *v_cache, const float *cos_table,
+                                 const float *sin_table, const int *positions,
+                                 const int *slot_mapping, int tokens, int num_q_heads,
+                                 int num_kv_heads, int head_dim, int rot_dim, int page_size,
+                                 int write_cache, int dtype, hipStream_t stream) {
+    KVA_REQUIRE(tokens >= 0 && num_q_heads > 0 && num_kv_heads > 0, "rope_kv_write: bad sizes");
+    KVA_REQUIRE(head_dim > 0 && head_dim % 2 == 0, "rope_kv_write: head_dim %d must be even", head_dim);
+    KVA_REQUIRE(rot_dim >= 0 && rot_dim <= head_dim && rot_dim % 2 == 0,
+                "rope_kv_write: rotary dim %d must be even and at most head_dim %d", rot_dim, head_dim);
+    KVA_REQUIRE((cos_table == nullptr) == (sin_table == nullptr), "rope_kv_write: one table missing");
+    KVA_REQUIRE(!write_cache || (k_cache && v_cache && slot_mapping && page_size > 0),
+                "rope_kv_write: cache write asked for without cache, slots or page size");
+    if (tokens == 0) return KVA_OK;
+    dim3 grid(tokens), block(256);
+    if (dtype == KVA_F32)
+        hipLaunchKernelGGL(rope_kv_write_kernel<float>, grid, block, 0, stream, (float *)qkv,
+                           (float *)k_cache, (float *)v_cache, cos_table, sin_table, positions,
+                           slot_mapping, num_q_heads, num_kv_heads, head_dim, rot_dim, page_size,
+                           write_cache);
+    else if (dtype == KVA_BF16)
+        hipLaunchKernelGGL(rope_kv_write_kernel<bf16_t>, grid, block, 0, stream, (bf16_t *)qkv,
+                           (bf16_t *)k_cache, (bf16_t *)v_cache, cos_table, sin_table, positions,
+                           slot_mapping, num_q_heads, num_kv_heads, head_dim, rot_dim, page_size,
+                           write_cache);
+    else KVA_REQUIRE(false, "rope_kv_write: unsupported dtype %d", dtype);
+    KVA_CHECK_LAUNCH("rope_kv_write");
+    return KVA_OK;
+}

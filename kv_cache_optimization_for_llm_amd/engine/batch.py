@@ -1,0 +1,107 @@
+"""One step's batch: a flat run of tokens from several requests, with the index arrays the
+kernels need.
+
+An entry is (request, its next tokens, the places among them whose logits are wanted).  Entries
+may be portions of prompts of any length beside single decoded tokens.  The reference builds
+comparable arrays for its prefill pass (``base/src/engine.cu:574-633``: token_positions,
+token_slot_ids, last_token_rows) and its decode pass (``:1013-1029``); here one layout serves
+both.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Sequence
+
+import numpy as np
+import torch
+
+
+@dataclass
+class StepEntry:
+    request_id: object
+    tokens: Sequence[int]
+    want: Sequence[int] = ()        # indices into ``tokens`` whose logits are returned
+
+
+@dataclass
+class StepBatch:
+    num_tokens: int
+    num_entries: int
+    num_logit_rows: int
+    # device int32 arrays
+    token_ids: torch.Tensor          # [T]
+    positions: torch.Tensor          # [T] absolute position inside the own request
+    tok_seat: torch.Tensor           # [T] seat (block-table row, state row) of the token's request
+    logit_rows: torch.Tensor         # [R] rows whose logits are wanted, in entry order
+    slot_mapping: List[torch.Tensor]  # per cache group: [T] cache slot to write
+    entry_seat: torch.Tensor         # [E]
+    entry_q_start: torch.Tensor      # [E + 1] first row of each entry (last = T)
+    entry_start_pos: torch.Tensor    # [E] position of the entry's first token
+    # host copies of the same
+    h_positions: np.ndarray = field(repr=False, default=None)
+    h_tok_seat: np.ndarray = field(repr=False, default=None)
+    h_entry_seat: np.ndarray = field(repr=False, default=None)
+    h_entry_q_start: np.ndarray = field(repr=False, default=None)
+    h_entry_start_pos: np.ndarray = field(repr=False, default=None)
+    max_q_len: int = 0
+    max_context: int = 0
+
+
+def _align(n: int, a: int = 4) -> int:
+    return (n + a - 1) // a * a
+
+
+def build_batch(seats: Sequence[int], starts: Sequence[int], token_lists: Sequence[Sequence[int]],
+                wants: Sequence[Sequence[int]], slot_maps: Sequence[Sequence[np.ndarray]],
+                device) -> StepBatch:
+    """Packs the index arrays into one pinned staging buffer and uploads it with one copy.
+
+    ``slot_maps[g][e]`` is the slot array of entry ``e`` in cache group ``g``."""
+    E = len(seats)
+    lens = [len(t) for t in token_lists]
+    T = int(sum(lens))
+    q_start = np.zeros(E + 1, dtype=np.int32)
+    np.cumsum(lens, out=q_start[1:])
+    token_ids = np.concatenate([np.asarray(t, dtype=np.int32) for t in token_lists]) if T else np.zeros(0, np.int32)
+    positions = np.concatenate([np.arange(s, s + n, dtype=np.int32) for s, n in zip(starts, lens)]) \
+        if T else np.zeros(0, np.int32)
+    tok_seat = np.repeat(np.asarray(seats, dtype=np.int32), lens)
+    rows: List[int] = []
+    for e, w in enumerate(wants):
+        for i in w:
+            if not 0 <= i < lens[e]:
+                raise ValueError(f"entry {e}: wanted place {i} is outside its {lens[e]} tokens")
+            rows.append(int(q_start[e]) + int(i))
+    logit_rows = np.asarray(rows, dtype=np.int32)
+    G = len(slot_maps)
+    segs: Dict[str, np.ndarray] = {
+        "token_ids": token_ids, "positions": positions, "tok_seat": tok_seat,
+        "logit_rows": logit_rows, "entry_seat": np.asarray(seats, dtype=np.int32),
+        "entry_q_start": q_start, "entry_start_pos": np.asarray(starts, dtype=np.int32),
+    }
+    for g in range(G):
+        segs[f"slots{g}"] = np.concatenate(slot_maps[g]).astype(np.int32) if T else np.zeros(0, np.int32)
+    offsets, total = {}, 0
+    for name, arr in segs.items():
+        offsets[name] = total
+        total += _align(max(1, arr.shape[0]))
+    staging = torch.empty(total, dtype=torch.int32, pin_memory=True)
+    st_np = staging.numpy()
+    for name, arr in segs.items():
+        st_np[offsets[name]:offsets[name] + arr.shape[0]] = arr
+    dev = staging.to(device, non_blocking=True)
+
+    def view(name):
+        return dev[offsets[name]:offsets[name] + segs[name].shape[0]]
+
+    return StepBatch(
+        num_tokens=T, num_entries=E, num_logit_rows=len(rows),
+        token_ids=view("token_ids"), positions=view("positions"), tok_seat=view("tok_seat"),
+        logit_rows=view("logit_rows"), slot_mapping=[view(f"slots{g}") for g in range(G)],
+        entry_seat=view("entry_seat"), entry_q_start=view("entry_q_start"),
+        entry_start_pos=view("entry_start_pos"),
+        h_positions=positions, h_tok_seat=tok_seat, h_entry_seat=segs["entry_seat"],
+        h_entry_q_start=q_start, h_entry_start_pos=segs["entry_start_pos"],
+        max_q_len=max(lens) if lens else 0,
+        max_context=max((s + n for s, n in zip(starts, lens)), default=0),
+    )

@@ -1,0 +1,167 @@
+"""The engine: a model folder, a cache and ONE step function.
+
+``Engine.step(entries)`` takes a batch of (request, its next tokens, wanted places) - portions
+of prompts of any length beside single decoded tokens - runs exactly those tokens through the
+model against the cache that earlier steps left, and returns the logits at the wanted places.
+The reference has two separate passes for this (``prefillBatch`` ``base/src/engine.cu:550-979``,
+which cannot continue a partly cached prompt, and ``decodeStep`` ``:982-1311``).
+"""
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager
+from ..config.model_config import read_config_json
+from ..models.builder import Model, spec_for_config
+from ..ops.library import KernelLibraryError, hip_lib
+from ..weights.loader import load_tensors
+from .batch import StepBatch, StepEntry, build_batch
+
+_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32,
+           "bf16": torch.bfloat16, "fp32": torch.float32}
+
+
+class CacheExhausted(RuntimeError):
+    """A step needs more pages (or a longer reservation) than the cache can give."""
+
+
+class EngineError(RuntimeError):
+    pass
+
+
+@dataclass
+class EngineOptions:
+    dtype: str = "bfloat16"             # "bfloat16": serving kernels; "float32": true 32-bit everywhere
+    cache_mode: str = "paged"           # "paged" | "contiguous"
+    page_size: int = 16                 # tokens per page (reference: BLOCK_SIZE, paged config.h:181)
+    cache_tokens: Optional[int] = None  # pool size in tokens (default: max_seqs * max_seq_len)
+    max_seqs: int = 8                   # seats (reference: MAX_SEQUENCES)
+    max_seq_len: Optional[int] = None   # longest request (default: max_position_embeddings)
+    device: str = "cuda:0"
+
+
+def require_gpu(device: str = "cuda:0") -> torch.device:
+    if not torch.cuda.is_available():
+        raise KernelLibraryError(
+            "no GPU is visible to torch; this engine runs on the GPU only (hand-written HIP "
+            "kernels for gfx950) and has no CPU path")
+    hip_lib()
+    return torch.device(device)
+
+
+class Engine:
+    def __init__(self, model_dir: str, options: Optional[EngineOptions] = None):
+        self.options = options = options or EngineOptions()
+        if options.dtype not in _DTYPES:
+            raise EngineError(f"dtype {options.dtype!r} is not one of bfloat16, float32")
+        self.dtype = _DTYPES[options.dtype]
+        self.device = require_gpu(options.device)
+        if self.dtype == torch.float32:
+            # the 32-bit path never uses a reduced-precision matrix mode
+            torch.backends.cuda.matmul.allow_tf32 = False
+            torch.backends.cudnn.allow_tf32 = False
+        self.model_dir = model_dir
+        self.config_dict = read_config_json(model_dir)
+        self.config, self.spec = spec_for_config(self.config_dict)
+        self.model = Model(self.spec, self.dtype, self.device)
+        tensors = load_tensors(model_dir, self.model.tensor_specs(), self.dtype, self.device,
+                               self.spec.ignorable_tensors)
+        self.model.load(tensors)
+        del tensors
+        self.vocab_size = self.spec.vocab_size
+        max_seq_len = options.max_seq_len or self.spec.max_positions
+        max_seq_len = min(max_seq_len, self.spec.max_positions)
+        cache_tokens = options.cache_tokens or options.max_seqs * max_seq_len
+        num_pages = (cache_tokens + options.page_size - 1) // options.page_size
+        groups, states = self.model.cache_requirements()
+        self.cache = CacheManager(groups, states, page_size=options.page_size, num_pages=num_pages,
+                                  max_seqs=options.max_seqs, max_seq_len=max_seq_len,
+                                  mode=options.cache_mode, device=self.device, dtype=self.dtype)
+        self.max_seq_len = max_seq_len
+        self._seat_of: Dict[object, int] = {}
+        self.steps_run = 0
+
+    # ------------------------------------------------------------------ requests
+    def has_request(self, request_id) -> bool:
+        return request_id in self._seat_of
+
+    def seat_of(self, request_id) -> int:
+        return self._seat_of[request_id]
+
+    def add_request(self, request_id, reserve_tokens: Optional[int] = None) -> Optional[int]:
+        """Gives the request a seat (and, in contiguous mode, its reservation).  ``None`` when
+        there is no seat or no room for the reservation."""
+        if request_id in self._seat_of:
+            raise EngineError(f"request {request_id!r} is live already")
+        if self.cache.mode == "contiguous" and reserve_tokens is None:
+            reserve_tokens = self.max_seq_len       # the reference's 'max' policy
+        seat = self.cache.admit(request_id, reserve_tokens)
+        if seat is not None:
+            self._seat_of[request_id] = seat
+        return seat
+
+    def release(self, request_id) -> None:
+        """The request is finished: its pages, reservation and seat are given back."""
+        seat = self._seat_of.pop(request_id)
+        self.cache.free(seat)
+
+    def length(self, request_id) -> int:
+        return self.cache.length(self._seat_of[request_id])
+
+    # ------------------------------------------------------------------ the step
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Runs one batch; returns fp32 logits ``[wanted places, vocab]`` on the device, in the
+        order of the entries and of each entry's ``want``."""
+        batch = self.prepare(entries)
+        logits = self.model.forward(batch, self.cache)
+        self.finish(entries)
+        return logits
+
+    def prepare(self, entries: Sequence[StepEntry]) -> StepBatch:
+        if not entries:
+            raise EngineError("a step needs at least one entry")
+        seen = set()
+        seats, starts, toks, wants = [], [], [], []
+        for e in entries:
+            if e.request_id in seen:
+                raise EngineError(f"request {e.request_id!r} appears twice in one step")
+            seen.add(e.request_id)
+            if len(e.tokens) == 0:
+                raise EngineError(f"request {e.request_id!r}: an entry needs at least one token")
+            arr = np.asarray(e.tokens, dtype=np.int64)
+            if arr.min() < 0 or arr.max() >= self.vocab_size:
+                raise EngineError(f"request {e.request_id!r}: token id outside [0, {self.vocab_size})")
+            if e.request_id not in self._seat_of:
+                if self.add_request(e.request_id) is None:
+                    raise CacheExhausted(f"no seat (or reservation) for request {e.request_id!r}")
+            seat = self._seat_of[e.request_id]
+            start = self.cache.length(seat)
+            seats.append(seat)
+            starts.append(start)
+            toks.append(arr)
+            wants.append(list(e.want))
+        # map pages for every entry, or for none
+        grown = []
+        for e, seat, start, arr in zip(entries, seats, starts, toks):
+            if not self.cache.grow(seat, start + len(arr)):
+                need = self.cache.pages_needed(seat, start + len(arr))
+                raise CacheExhausted(
+                    f"request {e.request_id!r} needs {need} more pages for positions "
+                    f"{start}..{start + len(arr) - 1} (capacity {self.cache.capacity_tokens(seat)} "
+                    f"tokens, free pages {[g.free_pages() for g in self.cache.groups]})")
+            grown.append(seat)
+        slot_maps = [[self.cache.slot_mapping(seat, start, len(arr), g.index)
+                      for seat, start, arr in zip(seats, starts, toks)] for g in self.cache.groups]
+        self.cache.flush_tables()
+        return build_batch(seats, starts, toks, wants, slot_maps, self.device)
+
+    def finish(self, entries: Sequence[StepEntry]) -> None:
+        for e in entries:
+            seat = self._seat_of[e.request_id]
+            self.cache.commit(seat, self.cache.length(seat) + len(e.tokens))
+        self.steps_run += 1

@@ -1,0 +1,149 @@
+"""Turns a ModelSpec into objects: parts from the registries, tensors from a checkpoint, and the
+forward pass over a step's batch."""
+from __future__ import annotations
+
+from typing import Any, Dict, List, Mapping, Optional, Tuple
+
+import torch
+
+from .. import parts as _parts  # noqa: F401  (registers the built-in part kinds)
+from . import llama as _llama   # noqa: F401  (registers LlamaForCausalLM)
+from ..config.registry import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, architecture_for)
+from ..models.spec import LayerCall, ModelSpec, TensorSpec
+from ..ops import kernels as K
+from ..parts.base import Block, KVCacheSpec, KVView, MixerContext, StateSpec
+from ..parts.linear import Linear
+
+
+def spec_for_config(config_dict: Mapping[str, Any]) -> Tuple[Any, ModelSpec]:
+    arch = architecture_for(config_dict)
+    config = arch.parse_config(config_dict)
+    return config, arch.build_spec(config)
+
+
+def build_blocks(spec: ModelSpec) -> List[Block]:
+    blocks = []
+    for ls in spec.layers:
+        mixer = MIXERS.get(ls.mixer.kind)(**ls.mixer.params)
+        ffn = FEED_FORWARDS.get(ls.feed_forward.kind)(**ls.feed_forward.params)
+        n1 = NORMS.get(ls.mixer_norm.kind)(**ls.mixer_norm.params)
+        n2 = NORMS.get(ls.ffn_norm.kind)(**ls.ffn_norm.params)
+        blocks.append(BLOCKS.get(ls.block.kind)(mixer, ffn, n1, n2, **ls.block.params))
+    return blocks
+
+
+def model_tensor_specs(spec: ModelSpec, blocks: List[Block], final_norm) -> Dict[str, TensorSpec]:
+    out: Dict[str, TensorSpec] = {spec.embedding_name: TensorSpec((spec.vocab_size, spec.hidden_size))}
+    for b in blocks:
+        for part in b.parts():
+            for name, ts in part.tensor_specs().items():
+                if name in out and out[name] != ts:
+                    raise ValueError(f"tensor {name!r} is declared twice with different specs")
+                out[name] = ts
+    out.update(final_norm.tensor_specs())
+    if spec.head_name is not None:
+        out[spec.head_name] = TensorSpec((spec.vocab_size, spec.hidden_size))
+    return out
+
+
+def tensor_specs_for_config(config_dict: Mapping[str, Any]) -> Dict[str, TensorSpec]:
+    """Names, shapes and init rules of every tensor a model folder for this config holds."""
+    _, spec = spec_for_config(config_dict)
+    blocks = build_blocks(spec)
+    final_norm = NORMS.get(spec.final_norm.kind)(**spec.final_norm.params)
+    return model_tensor_specs(spec, blocks, final_norm)
+
+
+def resolve_order(spec: ModelSpec) -> List[Tuple[LayerCall, int]]:
+    """(call, cache slot id) per entry of the run order; ``cache=None`` gets a private slot."""
+    used = {c.cache for c in spec.order if c.cache is not None}
+    nxt = (max(used) + 1) if used else 0
+    out = []
+    for call in spec.order:
+        if not 0 <= call.layer < len(spec.layers):
+            raise ValueError(f"run order names layer {call.layer}, the model has {len(spec.layers)}")
+        slot = call.cache
+        if slot is None:
+            slot, nxt = nxt, nxt + 1
+        out.append((call, slot))
+    return out
+
+
+class Model:
+    """Parts built from a ModelSpec, holding their tensors, run over a StepBatch."""
+
+    def __init__(self, spec: ModelSpec, dtype: torch.dtype, device):
+        self.spec, self.dtype, self.device = spec, dtype, torch.device(device)
+        self.blocks = build_blocks(spec)
+        self.final_norm = NORMS.get(spec.final_norm.kind)(**spec.final_norm.params)
+        self.calls = resolve_order(spec)
+        self.embedding: Optional[torch.Tensor] = None
+        self.head: Optional[Linear] = None
+
+    # ---- what the cache manager has to provide
+    def cache_requirements(self):
+        """(groups, states): groups = [(KVCacheSpec, [cache slot ids])] for slots that need paged
+        K/V, states = {cache slot id: StateSpec}."""
+        slot_spec: Dict[int, KVCacheSpec] = {}
+        slot_writer: Dict[int, bool] = {}
+        states: Dict[int, StateSpec] = {}
+        for call, slot in self.calls:
+            mixer = self.blocks[call.layer].mixer
+            kv = mixer.kv_cache_spec()
+            if kv is not None:
+                if slot in slot_spec and slot_spec[slot] != kv:
+                    raise ValueError(f"cache slot {slot} is shared by mixers with different needs")
+                slot_spec[slot] = kv
+                slot_writer[slot] = slot_writer.get(slot, False) or call.writes_cache
+            st = mixer.state_spec()
+            if st is not None:
+                if slot in states and states[slot] != st:
+                    raise ValueError(f"state slot {slot} is shared by mixers with different state")
+                states[slot] = st
+        for slot, has_writer in slot_writer.items():
+            if not has_writer:
+                raise ValueError(f"cache slot {slot} is read but no layer call writes it")
+        groups: Dict[KVCacheSpec, List[int]] = {}
+        for slot in sorted(slot_spec):
+            groups.setdefault(slot_spec[slot], []).append(slot)
+        return list(groups.items()), states
+
+    # ---- weights
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return model_tensor_specs(self.spec, self.blocks, self.final_norm)
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.embedding = tensors[self.spec.embedding_name]
+        for b in self.blocks:
+            for part in b.parts():
+                part.load(tensors)
+        self.final_norm.load(tensors)
+        head = tensors[self.spec.head_name] if self.spec.head_name is not None else self.embedding
+        self.head = Linear(head)
+
+    # ---- forward
+    def forward(self, batch, cache) -> torch.Tensor:
+        """Runs the batch's tokens through every layer call and returns fp32 logits
+        ``[len(batch.logit_rows), vocab]``."""
+        T = batch.num_tokens
+        hidden = torch.empty((T, self.spec.hidden_size), dtype=self.dtype, device=self.device)
+        K.embed_gather(self.embedding, batch.token_ids, hidden)
+        delta = None
+        for call, slot in self.calls:
+            block = self.blocks[call.layer]
+            ctx = MixerContext(batch=batch)
+            group = cache.group_of(slot)
+            if group is not None:
+                _, k, v = cache.kv_arrays(slot)
+                ctx.kv = KVView(k, v, group.table_dev, batch.slot_mapping[group.index],
+                                group.page_size, writes=call.writes_cache)
+            if slot in cache.state:
+                ctx.state = cache.state[slot]
+            hidden, delta = block.forward(hidden, delta, ctx)
+        R = batch.num_logit_rows
+        logits = torch.empty((R, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+        if R == 0:
+            return logits
+        x = self.final_norm.forward(hidden, delta=delta, row_idx=batch.logit_rows)
+        self.head(x, out=logits)
+        return logits

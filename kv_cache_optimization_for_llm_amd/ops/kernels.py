@@ -1,0 +1,221 @@
+"""Tensor-level entry points of the HIP kernels.
+
+Each function checks on the host that shapes, dtypes, devices and layouts are what the kernel
+and its grid assume, then launches on torch's current HIP stream.  There is no other code path:
+a tensor that is not on the GPU, or a missing kernel library, is an error.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .library import KernelError, check, hip_lib
+
+F32, BF16 = 0, 1
+_DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dt]
+    except KeyError:
+        raise KernelError(f"unsupported dtype {dt}; kernels take float32 and bfloat16") from None
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t: torch.Tensor, name: str, dtype: Optional[torch.dtype] = None, contiguous: bool = True):
+    if not isinstance(t, torch.Tensor):
+        raise KernelError(f"{name}: expected a tensor, got {type(t).__name__}")
+    if not t.is_cuda:
+        raise KernelError(f"{name}: tensor is on {t.device}; the kernels run on the GPU only")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name}: dtype {t.dtype}, expected {dtype}")
+    if contiguous and not t.is_contiguous():
+        raise KernelError(f"{name}: tensor must be contiguous")
+    return t.data_ptr()
+
+
+def _opt(t: Optional[torch.Tensor], name: str, dtype: Optional[torch.dtype] = None):
+    return None if t is None else _dev(t, name, dtype)
+
+
+# --------------------------------------------------------------------------------------
+def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, :] = table[ids[t], :], converted to out's dtype."""
+    rows, width = out.shape
+    if table.dim() != 2 or table.shape[1] != width or ids.shape != (rows,):
+        raise KernelError(f"embed_gather: shapes table {tuple(table.shape)} ids {tuple(ids.shape)} "
+                          f"out {tuple(out.shape)} do not fit")
+    check(hip_lib().kva_embed_gather(_dev(out, "out"), _dev(table, "table"),
+                                     _dev(ids, "ids", torch.int32), rows, width,
+                                     dtype_code(table.dtype), dtype_code(out.dtype), _stream()),
+          "embed_gather")
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+            delta: Optional[torch.Tensor] = None, row_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = rmsnorm(x) * weight.  With ``delta``: x += delta first (in place, fp32 add).  With
+    ``row_idx``: out[i] = rmsnorm(x[row_idx[i]])."""
+    width = x.shape[-1]
+    out_rows = out.shape[0]
+    if x.dim() != 2 or out.dim() != 2 or out.shape[1] != width or weight.shape != (width,):
+        raise KernelError(f"rmsnorm: shapes x {tuple(x.shape)} weight {tuple(weight.shape)} out "
+                          f"{tuple(out.shape)} do not fit")
+    if out.dtype != x.dtype:
+        raise KernelError("rmsnorm: out must have x's dtype")
+    if row_idx is None:
+        if out_rows != x.shape[0]:
+            raise KernelError("rmsnorm: out needs as many rows as x")
+    elif row_idx.shape != (out_rows,):
+        raise KernelError("rmsnorm: one row index per output row")
+    if delta is not None and (delta.shape != x.shape or delta.dtype != x.dtype):
+        raise KernelError("rmsnorm: delta must match x")
+    check(hip_lib().kva_rmsnorm(_dev(out, "out"), _dev(x, "x"), _opt(delta, "delta"),
+                                _dev(weight, "weight"), _opt(row_idx, "row_idx", torch.int32),
+                                out_rows, width, float(eps), dtype_code(x.dtype),
+                                dtype_code(weight.dtype), _stream()), "rmsnorm")
+    return out
+
+
+def residual_add(hidden: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+    if hidden.shape != delta.shape or hidden.dtype != delta.dtype:
+        raise KernelError("residual_add: operands must match")
+    check(hip_lib().kva_residual_add(_dev(hidden, "hidden"), _dev(delta, "delta"), hidden.numel(),
+                                     dtype_code(hidden.dtype), _stream()), "residual_add")
+    return hidden
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]."""
+    rows, inter = out.shape
+    if gate_up.shape != (rows, 2 * inter) or gate_up.dtype != out.dtype:
+        raise KernelError(f"silu_mul: gate_up {tuple(gate_up.shape)} does not fit out {tuple(out.shape)}")
+    check(hip_lib().kva_silu_mul(_dev(out, "out"), _dev(gate_up, "gate_up"), rows, inter,
+                                 dtype_code(out.dtype), _stream()), "silu_mul")
+    return out
+
+
+def cast(src: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    if src.shape != out.shape:
+        raise KernelError("cast: shapes differ")
+    if src.dtype == out.dtype:
+        raise KernelError("cast: same dtype on both sides")
+    check(hip_lib().kva_cast(_dev(out, "out"), _dev(src, "src"), src.numel(), dtype_code(src.dtype),
+                             dtype_code(out.dtype), _stream()), "cast")
+    return out
+
+
+def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int, num_kv_heads: int,
+                  head_dim: int, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+                  k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                  slot_mapping: Optional[torch.Tensor], page_size: int) -> None:
+    """Rotates the Q and K heads of ``qkv`` [T, (nq + 2 nkv) d] by the tokens' positions; Q in
+    place, rotated K and plain V into the cache [pages, nkv, page_size, d] at ``slot_mapping``."""
+    tokens = qkv.shape[0]
+    if qkv.dim() != 2 or qkv.shape[1] != (num_q_heads + 2 * num_kv_heads) * head_dim:
+        raise KernelError(f"rope_kv_write: qkv {tuple(qkv.shape)} is not [T, (nq + 2 nkv) * d]")
+    if positions.shape != (tokens,):
+        raise KernelError("rope_kv_write: one position per token")
+    rot = 0
+    if cos is not None:
+        if sin is None or cos.shape != sin.shape or cos.dim() != 2:
+            raise KernelError("rope_kv_write: cos and sin tables must be [positions, rot/2]")
+        rot = 2 * cos.shape[1]
+    write = k_cache is not None
+    if write:
+        if v_cache is None or slot_mapping is None or k_cache.shape != v_cache.shape:
+            raise KernelError("rope_kv_write: K and V cache and a slot mapping are all needed")
+        if k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (num_kv_heads, page_size, head_dim):
+            raise KernelError(f"rope_kv_write: cache {tuple(k_cache.shape)} is not "
+                              f"[pages, {num_kv_heads}, {page_size}, {head_dim}]")
+        if k_cache.dtype != qkv.dtype or slot_mapping.shape != (tokens,):
+            raise KernelError("rope_kv_write: cache dtype or slot mapping shape does not fit")
+    check(hip_lib().kva_rope_kv_write(
+        _dev(qkv, "qkv"), _opt(k_cache, "k_cache"), _opt(v_cache, "v_cache"),
+        _opt(cos, "cos", torch.float32), _opt(sin, "sin", torch.float32),
+        _dev(positions, "positions", torch.int32), _opt(slot_mapping, "slot_mapping", torch.int32),
+        tokens, num_q_heads, num_kv_heads, head_dim, rot, page_size, 1 if write else 0,
+        dtype_code(qkv.dtype), _stream()), "rope_kv_write")
+
+
+def attention_rowwise(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cache: torch.Tensor,
+                      v_cache: torch.Tensor, block_table: torch.Tensor, tok_seat: torch.Tensor,
+                      tok_pos: torch.Tensor, num_q_heads: int, num_kv_heads: int, head_dim: int,
+                      scale: float, window: int = 0) -> torch.Tensor:
+    """Causal GQA attention of every token over its request's cached keys; ``q`` is a view whose
+    rows are ``q_row_stride`` elements apart (the Q part of a fused QKV buffer)."""
+    tokens = out.shape[0]
+    if out.shape != (tokens, num_q_heads * head_dim):
+        raise KernelError("attention: out must be [T, nq * d]")
+    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or k_cache.shape[1] != num_kv_heads \
+            or k_cache.shape[3] != head_dim:
+        raise KernelError(f"attention: cache {tuple(k_cache.shape)} is not [pages, nkv, page, d]")
+    if block_table.dim() != 2 or tok_seat.shape != (tokens,) or tok_pos.shape != (tokens,):
+        raise KernelError("attention: block table [seats, blocks], one seat and position per token")
+    if q.dtype != out.dtype or k_cache.dtype != out.dtype:
+        raise KernelError("attention: q, cache and out must share a dtype")
+    if q.data_ptr() % 16 or q_row_stride < num_q_heads * head_dim:
+        raise KernelError("attention: q view is misaligned or its stride is too small")
+    page_size = k_cache.shape[2]
+    check(hip_lib().kva_attention_rowwise(
+        _dev(out, "out"), _dev(q, "q", contiguous=False), q_row_stride, _dev(k_cache, "k_cache"),
+        _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32), block_table.shape[1],
+        _dev(tok_seat, "tok_seat", torch.int32), _dev(tok_pos, "tok_pos", torch.int32), tokens,
+        num_q_heads, num_kv_heads, head_dim, page_size, float(scale), int(window),
+        dtype_code(out.dtype), _stream()), "attention_rowwise")
+    return out
+
+
+def gemm_nt_f32(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[M, N] = a[M, K] @ w[N, K]^T in true fp32."""
+    m, k = a.shape
+    n = w.shape[0]
+    if w.shape != (n, k) or out.shape != (m, n):
+        raise KernelError(f"gemm_f32: a {tuple(a.shape)} w {tuple(w.shape)} out {tuple(out.shape)} do not fit")
+    check(hip_lib().kva_gemm_nt_f32(_dev(out, "out", torch.float32), _dev(a, "a", torch.float32),
+                                    _dev(w, "w", torch.float32), m, n, k, k, k, n, _stream()),
+          "gemm_nt_f32")
+    return out
+
+
+def sample(logits: torch.Tensor, out_tokens: torch.Tensor, *, chunks: int = 128,
+           inv_temperature: Optional[torch.Tensor] = None, seed: int = 0,
+           rng_key: Optional[torch.Tensor] = None, rng_step: Optional[torch.Tensor] = None,
+           penalty_mask: Optional[torch.Tensor] = None, row_seat: Optional[torch.Tensor] = None,
+           penalty: float = 1.0) -> torch.Tensor:
+    """Greedy (rows whose inv_temperature is 0 or absent) or temperature sampling per row."""
+    rows, vocab = logits.shape
+    if out_tokens.shape != (rows,):
+        raise KernelError("sample: one output token per row")
+    any_sampled = inv_temperature is not None
+    if any_sampled and (rng_key is None or rng_step is None or inv_temperature.shape != (rows,)
+                        or rng_key.shape != (rows,) or rng_step.shape != (rows,)):
+        raise KernelError("sample: inv_temperature, rng_key and rng_step are needed per row")
+    if penalty_mask is not None:
+        if row_seat is None or row_seat.shape != (rows,) or penalty_mask.dim() != 2 \
+                or penalty_mask.shape[1] != vocab:
+            raise KernelError("sample: penalty mask [seats, vocab] needs a seat per row")
+    lib = hip_lib()
+    ws = torch.empty(lib.kva_sample_workspace_bytes(rows, chunks) // 4, dtype=torch.float32,
+                     device=logits.device)
+    check(lib.kva_sample(
+        _dev(out_tokens, "out_tokens", torch.int32), _dev(logits, "logits", torch.float32), rows, vocab,
+        chunks, _opt(penalty_mask, "penalty_mask", torch.uint8), _opt(row_seat, "row_seat", torch.int32),
+        float(penalty), _opt(inv_temperature, "inv_temperature", torch.float32), int(seed) & 0xFFFFFFFF,
+        _opt(rng_key, "rng_key", torch.int32), _opt(rng_step, "rng_step", torch.int32),
+        1 if any_sampled else 0, _dev(ws, "workspace"), _stream()), "sample")
+    return out_tokens
+
+
+def mark_tokens(mask: torch.Tensor, seats: torch.Tensor, tokens: torch.Tensor) -> None:
+    n = seats.shape[0]
+    if tokens.shape != (n,) or mask.dim() != 2:
+        raise KernelError("mark_tokens: one seat per token, mask [seats, vocab]")
+    check(hip_lib().kva_mark_tokens(_dev(mask, "mask", torch.uint8), _dev(seats, "seats", torch.int32),
+                                    _dev(tokens, "tokens", torch.int32), n, mask.shape[1], _stream()),
+          "mark_tokens")

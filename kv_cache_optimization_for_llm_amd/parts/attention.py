@@ -1,0 +1,66 @@
+"""Grouped-query causal attention over the paged cache (the Llama mixer).
+
+Per token (reference order, ``base/src/engine.cu:652-762``): Q, K, V projections without bias
+-> position encoding of Q and K -> K and V written to the cache -> scores ``q.k * scale`` over
+the request's keys up to the token's own position (optionally only the last ``window``),
+softmax in fp32 -> ``P V`` -> output projection.  ``kv_head = q_head // (num_heads / num_kv_heads)``.
+
+The three projection matrices are joined at load time into one ``[nq*d + 2*nkv*d, hidden]``
+matrix, so the step runs one product instead of three.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..config.registry import MIXERS, POSITION_ENCODINGS
+from ..models.spec import PartSpec, TensorSpec
+from ..ops import attention as attn_ops
+from .base import KVCacheSpec, Mixer, MixerContext
+from .linear import Linear
+
+
+@MIXERS.register("gqa_attention")
+class GQAAttention(Mixer):
+    def __init__(self, prefix: str, *, hidden_size: int, num_heads: int, num_kv_heads: int,
+                 head_dim: int, scale: float, position: PartSpec, window: int = 0):
+        super().__init__(prefix)
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads is not a multiple of {num_kv_heads} kv heads")
+        self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
+        self.head_dim, self.scale, self.window = head_dim, float(scale), int(window)
+        self.position = POSITION_ENCODINGS.get(position.kind)(**position.params)
+        self.qkv: Optional[Linear] = None
+        self.o: Optional[Linear] = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        p, d = self.prefix, self.head_dim
+        return {
+            p + "q_proj.weight": TensorSpec((self.num_heads * d, self.hidden_size)),
+            p + "k_proj.weight": TensorSpec((self.num_kv_heads * d, self.hidden_size)),
+            p + "v_proj.weight": TensorSpec((self.num_kv_heads * d, self.hidden_size)),
+            p + "o_proj.weight": TensorSpec((self.hidden_size, self.num_heads * d)),
+        }
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        p = self.prefix
+        q, k, v = (tensors[p + n + "_proj.weight"] for n in "qkv")
+        if not (q.dtype == k.dtype == v.dtype):
+            raise ValueError(f"{p}: q/k/v projection weights are stored in different dtypes")
+        self.qkv = Linear(torch.cat([q, k, v], dim=0))
+        self.o = Linear(tensors[p + "o_proj.weight"])
+
+    def kv_cache_spec(self) -> KVCacheSpec:
+        return KVCacheSpec(self.num_kv_heads, self.head_dim,
+                           kind="window" if self.window > 0 else "full", window=self.window)
+
+    def forward(self, x: torch.Tensor, ctx: MixerContext) -> torch.Tensor:
+        batch, kv = ctx.batch, ctx.kv
+        qkv = self.qkv(x)
+        self.position.apply_and_cache(qkv, batch.positions, self.num_heads, self.num_kv_heads,
+                                      self.head_dim, kv)
+        out = torch.empty((x.shape[0], self.num_heads * self.head_dim), dtype=x.dtype, device=x.device)
+        attn_ops.paged_attention(qkv, out, kv, batch, self.num_heads, self.num_kv_heads,
+                                 self.head_dim, self.scale, self.window)
+        return self.o(out)

@@ -1,0 +1,65 @@
+"""Random-weights mode: writes a model folder (``config.json`` + ``model.safetensors``) from a
+configuration and a seed.
+
+Matrices are N(0, 0.02), norm weights 1 + U(-0.1, 0.1).  Each tensor's generator is seeded from
+(seed, tensor name), so a tensor's values do not depend on which other tensors exist or on the
+order they are made in.  Values are drawn in fp32 and stored in the configuration's
+``torch_dtype`` (or the dtype asked for).
+"""
+from __future__ import annotations
+
+import hashlib
+import os
+from typing import Any, Dict, Mapping, Optional
+
+import torch
+
+from ..config.model_config import write_config_json
+from ..models.spec import TensorSpec
+
+_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+def _generator(seed: int, name: str) -> torch.Generator:
+    digest = hashlib.sha256(f"{seed}:{name}".encode()).digest()
+    g = torch.Generator(device="cpu")
+    g.manual_seed(int.from_bytes(digest[:8], "little") & ((1 << 63) - 1))
+    return g
+
+
+def random_tensor(name: str, spec: TensorSpec, seed: int, dtype: torch.dtype) -> torch.Tensor:
+    g = _generator(seed, name)
+    if spec.role == "table":
+        return torch.zeros(spec.shape, dtype=torch.int32)
+    if spec.init == "normal":
+        t = torch.randn(spec.shape, generator=g, dtype=torch.float32) * 0.02
+    elif spec.init == "norm":
+        t = 1.0 + (torch.rand(spec.shape, generator=g, dtype=torch.float32) * 0.2 - 0.1)
+    elif spec.init == "zeros":
+        t = torch.zeros(spec.shape, dtype=torch.float32)
+    else:
+        raise ValueError(f"tensor {name!r}: unknown init rule {spec.init!r}")
+    return t.to(dtype)
+
+
+def random_state_dict(specs: Mapping[str, TensorSpec], seed: int, dtype: torch.dtype) -> Dict[str, torch.Tensor]:
+    return {name: random_tensor(name, spec, seed, dtype) for name, spec in specs.items()}
+
+
+def write_random_model(model_dir: str, config_dict: Mapping[str, Any], seed: int,
+                       dtype: Optional[str] = None) -> str:
+    """Creates ``model_dir`` with ``config.json`` and a seeded ``model.safetensors``."""
+    from safetensors.torch import save_file
+    from ..models.builder import tensor_specs_for_config
+
+    cfg = dict(config_dict)
+    dtype_name = dtype or cfg.get("torch_dtype", "bfloat16")
+    if dtype_name not in _DTYPES:
+        raise ValueError(f"dtype {dtype_name!r} is not one of {sorted(_DTYPES)}")
+    cfg["torch_dtype"] = dtype_name
+    specs = tensor_specs_for_config(cfg)
+    os.makedirs(model_dir, exist_ok=True)
+    write_config_json(model_dir, cfg)
+    state = random_state_dict(specs, seed, _DTYPES[dtype_name])
+    save_file(state, os.path.join(model_dir, "model.safetensors"), metadata={"format": "pt"})
+    return model_dir
