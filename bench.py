@@ -1,0 +1,177 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine on one MI355X, Llama-3.2-1B shape, random bf16 weights.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line.  ``value`` is decoded tokens per second of the default run: a batch of 8
+requests, each holding a context of 8,192 tokens, one decode step (model forward over the paged
+cache + greedy sampling + token ids back on the host) per "step".  The same line carries the
+2,048-token prefill, the decode roofline (bytes the step has to read / time / HBM peak) and the
+batch-1 and batch-64 points.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+HBM_PEAK_GBS = 8000.0
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "fp32": 157.3}
+
+# BASELINE.json configs[2]: Llama 3.2 1B shape
+CONFIG_1B = dict(
+    architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=128256, hidden_size=2048,
+    intermediate_size=8192, num_hidden_layers=16, num_attention_heads=32, num_key_value_heads=8,
+    head_dim=64, rms_norm_eps=1e-5, rope_theta=500000.0, max_position_embeddings=8192,
+    rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+    tie_word_embeddings=True, hidden_act="silu", torch_dtype="bfloat16",
+)
+CONTEXT = 8192
+PAGE = 16
+PREFILL_TOKENS = 2048
+
+
+def weight_bytes(cfg, elem=2):
+    H, I, V, L = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"], cfg["num_hidden_layers"]
+    q, kv = cfg["num_attention_heads"] * cfg["head_dim"], cfg["num_key_value_heads"] * cfg["head_dim"]
+    per_layer = (q + 2 * kv) * H + H * q + 3 * I * H + 2 * H
+    head = V * H if cfg["tie_word_embeddings"] else V * H      # the output matrix is read once either way
+    return (L * per_layer + H + head) * elem
+
+
+def kv_bytes_per_token(cfg, elem=2):
+    return 2 * cfg["num_key_value_heads"] * cfg["head_dim"] * cfg["num_hidden_layers"] * elem
+
+
+def prefill_flops(cfg, T):
+    H, I, V, L = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"], cfg["num_hidden_layers"]
+    q, kv = cfg["num_attention_heads"] * cfg["head_dim"], cfg["num_key_value_heads"] * cfg["head_dim"]
+    linear = 2 * T * L * ((q + 2 * kv) * H + H * q + 3 * I * H)
+    attn = L * 4 * cfg["num_attention_heads"] * cfg["head_dim"] * T * (T + 1) / 2
+    return linear + attn + 2 * V * H
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=CONTEXT)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the 16 of the configuration")
+    ap.add_argument("--skip-points", action="store_true", help="only the default decode run and the prefill")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")
+        return 2
+
+    import torch
+    from kv_cache_optimization_for_llm_amd.engine.batch import StepEntry
+    from kv_cache_optimization_for_llm_amd.engine.engine import Engine, EngineOptions
+    from kv_cache_optimization_for_llm_amd.sampling.sampler import SampleRow, Sampler
+
+    cfg = dict(CONFIG_1B)
+    full_layers = cfg["num_hidden_layers"]
+    if args.layers:
+        cfg["num_hidden_layers"] = args.layers
+    max_batch = 64 if not args.skip_points else args.batch
+    ctx = args.context
+    # room for max_batch requests at the context, one more page each for the tokens decoded
+    pool = max_batch * (ctx + 2 * PAGE)
+    engine = Engine(None, EngineOptions(dtype="bfloat16", page_size=PAGE, cache_tokens=pool,
+                                        max_seqs=max_batch, max_seq_len=cfg["max_position_embeddings"]),
+                    config_dict=cfg, random_seed=0)
+    dev = engine.device
+    for g in engine.cache.groups:       # random keys and values stand for the context
+        g.k.normal_(0.0, 1.0)
+        g.v.normal_(0.0, 1.0)
+    sampler = Sampler(engine.vocab_size, max_batch, dev)
+    gen = torch.Generator().manual_seed(0)
+
+    def decode_run(batch, steps, warmup, context):
+        """Times ``steps`` decode steps of ``batch`` requests whose contexts END at ``context``."""
+        ids = [f"d{batch}_{i}" for i in range(batch)]
+        first = context - (steps + warmup)
+        for rid in ids:
+            engine.preload_context(rid, first)
+        toks = [int(t) for t in torch.randint(0, engine.vocab_size, (batch,), generator=gen)]
+        rows = [SampleRow(engine.seat_of(r)) for r in ids]
+
+        def one():
+            nonlocal toks
+            logits = engine.step([StepEntry(r, [t], [0]) for r, t in zip(ids, toks)])
+            toks = [int(t) for t in sampler.sample(logits, rows)]
+        for _ in range(warmup):
+            one()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            one()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        for rid in ids:
+            engine.release(rid)
+        return dt
+
+    dt = decode_run(args.batch, args.steps, args.warmup, ctx)
+    ms_per_step = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+    mean_ctx = ctx - args.steps / 2
+    step_bytes = weight_bytes(cfg) + args.batch * mean_ctx * kv_bytes_per_token(cfg)
+    achieved = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # prefill of 2,048 tokens: one request, one step, logits at the last place
+    prompt = [int(t) for t in torch.randint(0, engine.vocab_size, (PREFILL_TOKENS,), generator=gen)]
+    pre_ms = []
+    for i in range(3):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step([StepEntry(f"p{i}", prompt, [PREFILL_TOKENS - 1])])
+        torch.cuda.synchronize()
+        pre_ms.append((time.perf_counter() - t0) * 1e3)
+        engine.release(f"p{i}")
+    p_ms = min(pre_ms[1:])
+    flops = prefill_flops(cfg, PREFILL_TOKENS)
+    prefill = {"value": round(PREFILL_TOKENS / (p_ms * 1e-3), 1), "tokens": PREFILL_TOKENS,
+               "ms": round(p_ms, 3), "frac": round(flops / (p_ms * 1e-3) / (PEAK_TFLOPS["bf16"] * 1e12), 4)}
+
+    points = {}
+    if not args.skip_points:
+        for b in (1, 64):
+            k = max(16, args.steps // 2)
+            d = decode_run(b, k, 8, ctx)
+            points[f"decode_b{b}"] = round(b * k / d, 1)
+        # the workload BASELINE.json words: 512-token prompts, 256 generated tokens
+        for b in (1, 8, 64):
+            d = decode_run(b, 256, 8, 512 + 256 + 8)
+            points[f"decode_b{b}_p512_g256"] = round(b * 256 / d, 1)
+
+    out = {
+        "metric": "decode tok/s at batch 8 (context 8192), Llama-3.2-1B shape", "value": round(value, 1),
+        "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic: random weights N(0,0.02), seeded uniform token ids, random cache contents for the context",
+        "config": {"model": "llama-3.2-1b-shape", "global_batch": args.batch, "seq_len": ctx,
+                   "parallelism": "single-gpu", "layers": cfg["num_hidden_layers"], "layers_full": full_layers,
+                   "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
+                   "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
+                   "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
+                   "page_size": PAGE, "prefill_tokens": PREFILL_TOKENS, "tied_embeddings": True,
+                   "rope": "llama3 factor 32", "sampling": "greedy on device"},
+        "prefill": prefill,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

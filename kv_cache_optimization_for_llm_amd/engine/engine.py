@@ -20,6 +20,7 @@ from ..config.model_config import read_config_json
 from ..models.builder import Model, spec_for_config
 from ..ops.library import KernelLibraryError, hip_lib
 from ..weights.loader import load_tensors
+from ..weights.random_init import random_tensors_on_device
 from .batch import StepBatch, StepEntry, build_batch
 
 _DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32,
@@ -55,7 +56,12 @@ def require_gpu(device: str = "cuda:0") -> torch.device:
 
 
 class Engine:
-    def __init__(self, model_dir: str, options: Optional[EngineOptions] = None):
+    """``Engine(model_dir)`` loads a model folder.  ``Engine(None, config_dict=..., random_seed=...)``
+    builds the same model with random weights made on the device (for measurements; the values
+    differ from the folder the random-weights mode writes for the same seed)."""
+
+    def __init__(self, model_dir: Optional[str], options: Optional[EngineOptions] = None, *,
+                 config_dict: Optional[dict] = None, random_seed: Optional[int] = None):
         self.options = options = options or EngineOptions()
         if options.dtype not in _DTYPES:
             raise EngineError(f"dtype {options.dtype!r} is not one of bfloat16, float32")
@@ -66,11 +72,17 @@ class Engine:
             torch.backends.cuda.matmul.allow_tf32 = False
             torch.backends.cudnn.allow_tf32 = False
         self.model_dir = model_dir
-        self.config_dict = read_config_json(model_dir)
+        if model_dir is None and (config_dict is None or random_seed is None):
+            raise EngineError("without a model folder, config_dict and random_seed are needed")
+        self.config_dict = read_config_json(model_dir) if model_dir is not None else dict(config_dict)
         self.config, self.spec = spec_for_config(self.config_dict)
         self.model = Model(self.spec, self.dtype, self.device)
-        tensors = load_tensors(model_dir, self.model.tensor_specs(), self.dtype, self.device,
-                               self.spec.ignorable_tensors)
+        if model_dir is not None:
+            tensors = load_tensors(model_dir, self.model.tensor_specs(), self.dtype, self.device,
+                                   self.spec.ignorable_tensors)
+        else:
+            tensors = random_tensors_on_device(self.model.tensor_specs(), random_seed, self.dtype,
+                                               self.device)
         self.model.load(tensors)
         del tensors
         self.vocab_size = self.spec.vocab_size
@@ -113,6 +125,17 @@ class Engine:
     def length(self, request_id) -> int:
         return self.cache.length(self._seat_of[request_id])
 
+    def preload_context(self, request_id, num_tokens: int) -> None:
+        """For measurements: the request is taken to hold ``num_tokens`` tokens already; pages are
+        mapped for them and whatever the cache arrays contain there stands for their keys and
+        values.  Nothing is computed."""
+        if request_id not in self._seat_of and self.add_request(request_id) is None:
+            raise CacheExhausted(f"no seat for request {request_id!r}")
+        seat = self._seat_of[request_id]
+        if not self.cache.grow(seat, num_tokens):
+            raise CacheExhausted(f"no pages for {num_tokens} tokens of request {request_id!r}")
+        self.cache.commit(seat, num_tokens)
+
     # ------------------------------------------------------------------ the step
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Runs one batch; returns fp32 logits ``[wanted places, vocab]`` on the device, in the
@@ -120,6 +143,18 @@ class Engine:
         batch = self.prepare(entries)
         logits = self.model.forward(batch, self.cache)
         self.finish(entries)
+        return logits
+
+    def step_planned(self, entries: Sequence[StepEntry], seats: Sequence[int],
+                     starts: Sequence[int]) -> torch.Tensor:
+        """The step for a scheduler that owns the seats itself: entry ``i`` belongs to
+        ``seats[i]`` and starts at position ``starts[i]``; lengths are committed by the caller."""
+        for e, seat, start in zip(entries, seats, starts):
+            if self._seat_of.get(e.request_id) != seat or self.cache.length(seat) != start:
+                raise EngineError(f"plan does not fit the cache: request {e.request_id!r}")
+        batch = self.prepare(entries)
+        logits = self.model.forward(batch, self.cache)
+        self.steps_run += 1
         return logits
 
     def prepare(self, entries: Sequence[StepEntry]) -> StepBatch:

@@ -1,0 +1,127 @@
+"""Scheduler + step function + sampler in one loop; the Python entry point ``LLM.generate``."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, Iterable, List, Optional, Sequence
+
+from ..sampling.sampler import SampleRow, Sampler
+from .batch import StepEntry
+from .engine import Engine, EngineOptions
+from .scheduler import Event, Request, Scheduler, StepPlan
+
+
+@dataclass
+class ServeOptions:
+    """Options of the serving loop; names follow the reference's environment variables
+    (``base/src/main.cu:52-105``) and limits (``base/src/config.h:80-136``)."""
+
+    temperature: float = 0.0            # TEMPERATURE: <= 0 is greedy
+    sampling_seed: int = 0              # SAMPLING_SEED
+    ignore_eos: bool = False            # IGNORE_EOS
+    repetition_penalty: float = 1.0     # REPETITION_PENALTY (the reference fixes 1.15)
+    max_batch_tokens: int = 3072        # MAX_BATCH_TOKENS: a step's token budget
+    chunk_size: Optional[int] = None    # most prompt tokens of one request per step
+    reserve_policy: str = "max"         # ORCA_POLICY: max | pow2 | oracle (contiguous mode)
+
+
+class Runner:
+    """Drives requests to completion, one batch per call to :meth:`step`."""
+
+    def __init__(self, engine: Engine, options: Optional[ServeOptions] = None):
+        self.engine = engine
+        self.options = options = options or ServeOptions()
+        self.scheduler = Scheduler(
+            engine.cache, max_batch_tokens=options.max_batch_tokens, chunk_size=options.chunk_size,
+            eos_token_ids=engine.spec.eos_token_ids, ignore_eos=options.ignore_eos,
+            reserve_policy=options.reserve_policy)
+        self.sampler = Sampler(engine.vocab_size, engine.cache.max_seqs, engine.device,
+                               seed=options.sampling_seed, repetition_penalty=options.repetition_penalty)
+        self.scheduler.on_admit = self._on_admit
+        self.scheduler.on_release = self._on_release
+        self._next_id = 0
+
+    # the scheduler owns seats; the engine only needs to know which request sits where
+    def _on_admit(self, seq) -> None:
+        self.engine._seat_of[("sched", seq.request.id, seq.request.seq_index, seq.request.arrival)] = seq.seat
+        emitted = seq.prompt[len(seq.prompt) - seq.request.resumed_tokens:] if seq.request.resumed_tokens else ()
+        self.sampler.reset_seat(seq.seat, emitted)
+
+    def _on_release(self, seq) -> None:
+        self.engine._seat_of.pop(("sched", seq.request.id, seq.request.seq_index, seq.request.arrival), None)
+
+    def submit(self, tokens: Sequence[int], max_new_tokens: int, *, request_id: Optional[int] = None,
+               n_seqs: int = 1, temperature: Optional[float] = None) -> int:
+        """Queues ``n_seqs`` copies of a request (reference wire format:
+        ``<id> <max_tokens> <n_seqs> <tok> ...``, ``base/src/request_queue.cpp:11-61``)."""
+        if request_id is None:
+            request_id = self._next_id
+        self._next_id = max(self._next_id, request_id + 1)
+        t = self.options.temperature if temperature is None else temperature
+        for i in range(n_seqs):
+            self.scheduler.add(Request(request_id, [int(x) for x in tokens], int(max_new_tokens),
+                                       seq_index=i, temperature=float(t)))
+        return request_id
+
+    def idle(self) -> bool:
+        return self.scheduler.idle()
+
+    def step(self) -> List[Event]:
+        plan = self.scheduler.plan()
+        events = list(plan.events)
+        if not plan.entries:
+            return events
+        entries, rows = [], []
+        for e in plan.entries:
+            rid = ("sched", e.seq.request.id, e.seq.request.seq_index, e.seq.request.arrival)
+            entries.append(StepEntry(rid, e.tokens, [len(e.tokens) - 1] if e.sample else []))
+            if e.sample:
+                req = e.seq.request
+                emitted_before = req.resumed_tokens + len(e.seq.generated)
+                rows.append(SampleRow(e.seq.seat, req.temperature, req.id * 8 + req.seq_index,
+                                      e.start + len(e.tokens), apply_penalty=emitted_before > 0))
+        logits = self.engine.step_planned(entries, [e.seq.seat for e in plan.entries],
+                                          [e.start for e in plan.entries])
+        sampled = self.sampler.sample(logits, rows)
+        events.extend(self.scheduler.complete(plan, sampled))
+        return events
+
+    def run_until_idle(self) -> Iterable[Event]:
+        while not self.idle():
+            for ev in self.step():
+                yield ev
+
+
+class LLM:
+    """Python entry point: ``LLM(model_dir).generate(prompts, max_new_tokens=...)``."""
+
+    def __init__(self, model_dir: str, engine_options: Optional[EngineOptions] = None,
+                 serve_options: Optional[ServeOptions] = None):
+        self.engine = Engine(model_dir, engine_options)
+        self.serve_options = serve_options or ServeOptions()
+
+    def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: int = 16, *,
+                 temperature: Optional[float] = None, seed: Optional[int] = None,
+                 ignore_eos: Optional[bool] = None, repetition_penalty: Optional[float] = None,
+                 return_reasons: bool = False):
+        """Generates for every prompt (token ids in, token ids out), batched continuously."""
+        opts = ServeOptions(**vars(self.serve_options))
+        if temperature is not None:
+            opts.temperature = temperature
+        if seed is not None:
+            opts.sampling_seed = seed
+        if ignore_eos is not None:
+            opts.ignore_eos = ignore_eos
+        if repetition_penalty is not None:
+            opts.repetition_penalty = repetition_penalty
+        runner = Runner(self.engine, opts)
+        ids = [runner.submit(p, max_new_tokens) for p in prompts]
+        out: Dict[int, List[int]] = {i: [] for i in ids}
+        reasons: Dict[int, str] = {}
+        for ev in runner.run_until_idle():
+            if ev.kind == "token":
+                out[ev.request_id].append(ev.token)
+            elif ev.kind in ("done", "rejected"):
+                reasons[ev.request_id] = ev.reason
+        self.last_runner = runner
+        results = [out[i] for i in ids]
+        return (results, [reasons.get(i) for i in ids]) if return_reasons else results

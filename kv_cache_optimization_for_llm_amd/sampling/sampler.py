@@ -1,0 +1,106 @@
+"""Greedy and temperature sampling over a step's logits, on the device.
+
+Options and their meaning follow the reference (``base/src/main.cu:57-84``,
+``base/src/kernels.cu:489-835``, ``python/sampling_reference.py``):
+
+* ``temperature`` <= 0: greedy, the maximum logit, ties to the lowest token id;
+* ``temperature`` > 0: inverse-CDF sampling of ``softmax(logits / temperature)`` with the
+  counter-based uniform ``counter_uniform(seed, key, step)``; ``key = request_id * 8 +
+  seq_index`` as in the reference, ``step`` = the absolute position the sampled token will take,
+  so a draw is a pure function of (seed, request, position) - the intent the reference states at
+  ``base/src/kernels.cuh:158-160`` - and a recomputed request draws the same tokens again;
+* ``repetition_penalty`` (reference: fixed 1.15, ``base/src/config.h:83``): logits of tokens the
+  request has already emitted are divided (if positive) or multiplied (if negative) by it, from
+  the second generated token on.  The emitted-token mask lives in the request's seat, one byte
+  per vocabulary entry.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..ops import kernels as K
+
+
+def counter_uniform(seed: int, key: int, step: int) -> float:
+    """Host mirror of the device function (splitmix64 finaliser, top 24 bits)."""
+    M = (1 << 64) - 1
+    z = (((key & 0xFFFFFFFF) << 32) ^ (step & 0xFFFFFFFF)) & M
+    z ^= ((seed & 0xFFFFFFFF) * 0x9E3779B97F4A7C15) & M
+    z = (z + 0x9E3779B97F4A7C15) & M
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & M
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & M
+    z ^= z >> 31
+    return (z >> 40) * (1.0 / 16777216.0)
+
+
+@dataclass
+class SampleRow:
+    seat: int
+    temperature: float = 0.0
+    rng_key: int = 0
+    rng_step: int = 0
+    apply_penalty: bool = False
+
+
+def _as_i32(values: Sequence[int]) -> np.ndarray:
+    return (np.asarray(values, dtype=np.int64) & 0xFFFFFFFF).astype(np.uint32).view(np.int32)
+
+
+class Sampler:
+    def __init__(self, vocab_size: int, max_seqs: int, device, *, seed: int = 0,
+                 repetition_penalty: float = 1.0, chunks: int = 128):
+        if repetition_penalty <= 0:
+            raise ValueError("repetition_penalty must be positive")
+        self.vocab_size, self.device, self.seed = vocab_size, device, int(seed)
+        self.penalty = float(repetition_penalty)
+        self.chunks = max(1, min(chunks, (vocab_size + 255) // 256))
+        self.mask: Optional[torch.Tensor] = None
+        if self.penalty != 1.0:
+            self.mask = torch.zeros((max_seqs, vocab_size), dtype=torch.uint8, device=device)
+
+    def reset_seat(self, seat: int, emitted: Sequence[int] = ()) -> None:
+        """A request takes the seat: clear its mask and mark what it has emitted before (a
+        recomputed request arrives with its earlier output)."""
+        if self.mask is None:
+            return
+        self.mask[seat].zero_()
+        if len(emitted):
+            self.mark([seat] * len(emitted), emitted)
+
+    def mark(self, seats: Sequence[int], tokens: Sequence[int]) -> None:
+        if self.mask is None or not len(seats):
+            return
+        s = torch.from_numpy(np.asarray(seats, dtype=np.int32)).to(self.device)
+        t = torch.from_numpy(np.asarray(tokens, dtype=np.int32)).to(self.device)
+        K.mark_tokens(self.mask, s, t)
+
+    def sample(self, logits: torch.Tensor, rows: Sequence[SampleRow]) -> np.ndarray:
+        """One token per logits row; returns host int32."""
+        n = len(rows)
+        if logits.shape != (n, self.vocab_size):
+            raise ValueError(f"logits {tuple(logits.shape)} do not fit {n} rows of {self.vocab_size}")
+        out = torch.empty(n, dtype=torch.int32, device=self.device)
+        if n == 0:
+            return np.zeros(0, dtype=np.int32)
+        any_sampled = any(r.temperature > 0 for r in rows)
+        inv_t = key = step = seat_t = None
+        if any_sampled:
+            inv_t = torch.tensor([1.0 / r.temperature if r.temperature > 0 else 0.0 for r in rows],
+                                 dtype=torch.float32).to(self.device)
+            key = torch.from_numpy(_as_i32([r.rng_key for r in rows])).to(self.device)
+            step = torch.from_numpy(_as_i32([r.rng_step for r in rows])).to(self.device)
+        use_mask = self.mask is not None and any(r.apply_penalty for r in rows)
+        if use_mask:
+            seat_t = torch.tensor([r.seat if r.apply_penalty else -1 for r in rows],
+                                  dtype=torch.int32).to(self.device)
+        K.sample(logits, out, chunks=self.chunks, inv_temperature=inv_t, seed=self.seed, rng_key=key,
+                 rng_step=step, penalty_mask=self.mask if use_mask else None, row_seat=seat_t,
+                 penalty=self.penalty)
+        tokens = out.cpu().numpy()
+        if self.mask is not None:
+            self.mark([r.seat for r in rows], tokens)
+        return tokens
