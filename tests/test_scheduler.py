@@ -1,0 +1,197 @@
+"""The scheduler's decisions, on the CPU, with a made-up token source instead of a model."""
+import pytest
+
+from kv_cache_optimization_for_llm_amd.cache.manager import CacheManager
+from kv_cache_optimization_for_llm_amd.engine.scheduler import (Request, Scheduler, reservation_tokens)
+from kv_cache_optimization_for_llm_amd.parts.base import KVCacheSpec
+
+SPEC = KVCacheSpec(2, 16)
+EOS = 7
+
+
+def cache(pages=64, seqs=8, mode="paged", page=16, max_len=512):
+    return CacheManager([(SPEC, [0, 1])], {}, page_size=page, num_pages=pages, max_seqs=seqs,
+                        max_seq_len=max_len, mode=mode)
+
+
+def fake_token(request_id, position):
+    """What 'the model' samples for the token that will sit at ``position``: a pure function, as
+    greedy decoding of a fixed model is."""
+    t = (request_id * 31 + position * 17) % 97 + 8
+    return t
+
+
+def run(s, max_steps=10000, on_plan=None):
+    """Runs to idle; returns ({(id, seq): tokens}, {(id, seq): reason}, all events, plans)."""
+    out, reasons, events, plans = {}, {}, [], []
+    for _ in range(max_steps):
+        if s.idle():
+            break
+        plan = s.plan()
+        s.cache.check()
+        plans.append(plan)
+        if on_plan:
+            on_plan(plan)
+        evs = list(plan.events)
+        for e in plan.entries:
+            assert s.cache.grow(e.seq.seat, e.start + len(e.tokens)), "the plan promised pages it cannot get"
+        sampled = [fake_token(e.seq.request.id, e.start + len(e.tokens)) for e in plan.entries if e.sample]
+        evs += s.complete(plan, sampled)
+        s.cache.check()
+        for ev in evs:
+            key = (ev.request_id, ev.seq_index)
+            if ev.kind == "token":
+                out.setdefault(key, []).append(ev.token)
+            elif ev.kind in ("done", "rejected"):
+                reasons[key] = ev.reason
+        events += evs
+    assert s.idle(), "the scheduler did not finish"
+    return out, reasons, events, plans
+
+
+def test_budget_goes_to_decodes_first_then_to_prompt_portions_in_order():
+    s = Scheduler(cache(), max_batch_tokens=40, chunk_size=24, ignore_eos=True)
+    s.add(Request(0, list(range(8, 38)), 5))          # 30 tokens
+    s.add(Request(1, list(range(8, 58)), 5))          # 50 tokens
+    p = s.plan()
+    assert [(e.seq.request.id, len(e.tokens), e.sample) for e in p.entries] == [(0, 24, False), (1, 16, False)]
+    s.complete(p, [])
+    p = s.plan()                                       # 0 finishes its prompt, 1 goes on
+    assert [(e.seq.request.id, e.start, len(e.tokens), e.sample) for e in p.entries] == \
+        [(0, 24, 6, True), (1, 16, 24, False)]
+    s.complete(p, [fake_token(0, 30)])
+    p = s.plan()                                       # 0 decodes first, then 1's last portion
+    assert [(e.seq.request.id, len(e.tokens), e.sample) for e in p.entries] == [(0, 1, True), (1, 10, True)]
+    assert p.entries[0].tokens == [fake_token(0, 30)] and p.num_tokens <= 40
+
+
+def test_every_request_emits_exactly_its_budget_and_order_is_fcfs():
+    s = Scheduler(cache(), max_batch_tokens=64, chunk_size=16, ignore_eos=True)
+    lens = [5, 17, 33, 70, 1, 9]
+    for i, n in enumerate(lens):
+        s.add(Request(i, [8 + (j % 50) for j in range(n)], 8 + i))
+    out, reasons, events, plans = run(s)
+    for i, n in enumerate(lens):
+        assert out[(i, 0)] == [fake_token(i, n + k) for k in range(8 + i)]
+        assert reasons[(i, 0)] == "length"
+    first_seen = []
+    for p in plans:
+        for e in p.entries:
+            if e.seq.request.id not in first_seen:
+                first_seen.append(e.seq.request.id)
+    assert first_seen == sorted(first_seen)
+    assert all(p.num_tokens <= 64 for p in plans)
+    assert s.cache.free_seats == 8 and s.cache.groups[0].free_pages() == 64
+
+
+def test_eos_ends_a_request_and_is_not_emitted():
+    s = Scheduler(cache(), eos_token_ids=[fake_token(3, 12)], max_batch_tokens=64)
+    s.add(Request(3, list(range(10, 20)), 20))
+    out, reasons, events, _ = run(s)
+    assert out[(3, 0)] == [fake_token(3, 10), fake_token(3, 11)] and reasons[(3, 0)] == "eos"
+    done = [e for e in events if e.kind == "done"][0]
+    assert done.tokens == 2
+
+
+def test_n_seqs_share_an_id_and_differ_by_seq_index():
+    s = Scheduler(cache(), ignore_eos=True)
+    for i in range(3):
+        s.add(Request(5, [9, 9, 9], 4, seq_index=i))
+    out, reasons, _, _ = run(s)
+    assert sorted(out) == [(5, 0), (5, 1), (5, 2)] and all(len(v) == 4 for v in out.values())
+
+
+def test_pages_run_out_newest_is_preempted_recomputed_and_emits_nothing_twice():
+    def go(pages):
+        s = Scheduler(cache(pages=pages), max_batch_tokens=256, ignore_eos=True)
+        for i in range(3):
+            s.add(Request(i, [8 + i] * 30, 60))       # each ends at 90 tokens = 6 pages
+        return s, run(s)
+    s_big, (out_big, _, ev_big, _) = go(64)
+    s_small, (out_small, reasons, ev_small, plans) = go(12)   # 3 x 6 pages do not fit
+    assert s_big.preemptions == 0 and s_small.preemptions > 0
+    assert out_small == out_big                        # identical tokens, none emitted twice
+    pre = [e for e in ev_small if e.kind == "preempted"]
+    assert pre and pre[0].request_id == 2 and pre[0].reason == "recompute"   # the newest goes first
+    assert all(r == "length" for r in reasons.values())
+    # the preempted request re-enters at the FRONT and is admitted before anything newer
+    assert s_small.cache.groups[0].free_pages() == 12 and not s_small.preemption_pending
+
+
+def test_admission_is_closed_to_new_requests_while_a_preempted_one_is_pending():
+    s = Scheduler(cache(pages=8), max_batch_tokens=256, ignore_eos=True)
+    s.add(Request(0, [9] * 40, 50))                   # ends at 90 tokens = 6 pages
+    s.add(Request(1, [9] * 40, 50))
+    seen_new_while_pending = []
+
+    def watch(plan):
+        if s.preemption_pending:
+            seen_new_while_pending.extend(e.seq.request.id for e in plan.entries if e.seq.request.id == 2)
+    s.plan_calls = 0
+    steps = 0
+    while not s.idle():
+        plan = s.plan()
+        if steps == 3:
+            s.add(Request(2, [9] * 10, 5))             # a fresh request arrives
+        watch(plan)
+        for e in plan.entries:
+            assert s.cache.grow(e.seq.seat, e.start + len(e.tokens))
+        s.complete(plan, [fake_token(e.seq.request.id, e.start + len(e.tokens)) for e in plan.entries if e.sample])
+        s.cache.check()
+        steps += 1
+        assert steps < 2000
+    assert s.preemptions > 0 and not seen_new_while_pending
+
+
+def test_hopeless_requests_fail_loudly_instead_of_waiting_forever():
+    s = Scheduler(cache(pages=4, max_len=512), ignore_eos=True)
+    s.add(Request(0, [9] * 100, 5))                   # 7 pages, the pool has 4
+    s.add(Request(1, [9] * 600, 5))                   # longer than the longest sequence
+    s.add(Request(2, [], 5))
+    s.add(Request(3, [9] * 20, 100))                  # fits at first, outgrows the pool alone
+    out, reasons, _, _ = run(s)
+    assert reasons[(0, 0)] == "kv_cache_exhausted" and reasons[(1, 0)] == "prompt_too_long"
+    assert reasons[(2, 0)] == "empty_request" and reasons[(3, 0)] == "kv_cache_exhausted"
+    assert len(out[(3, 0)]) == 4 * 16 - 20 + 1        # it ran until the pool was full
+    assert s.cache.groups[0].free_pages() == 4
+
+
+def test_a_request_stops_at_the_longest_sequence():
+    s = Scheduler(cache(max_len=40), ignore_eos=True)
+    s.add(Request(0, [9] * 30, 100))
+    out, reasons, _, _ = run(s)
+    assert reasons[(0, 0)] == "sequence_too_long" and len(out[(0, 0)]) == 11
+
+
+def test_reservation_policies_are_the_papers():
+    assert reservation_tokens("max", 40, 25, 2048) == 2048
+    assert reservation_tokens("pow2", 40, 25, 2048) == 72         # 40 + 32, reference engine.cu:314-317
+    assert reservation_tokens("pow2", 0, 25, 2048) == 32          # reference config.h:192-195
+    assert reservation_tokens("oracle", 40, 25, 2048) == 65
+    assert reservation_tokens("oracle", 2000, 100, 2048) == 2048
+    with pytest.raises(ValueError):
+        reservation_tokens("best", 1, 1, 1)
+
+
+def test_contiguous_mode_blocks_at_the_head_never_preempts_and_stops_at_the_reservation():
+    s = Scheduler(cache(pages=16, mode="contiguous", max_len=128), reserve_policy="oracle",
+                  max_batch_tokens=256, ignore_eos=True)
+    s.add(Request(0, [9] * 60, 60))                   # 120 tokens -> 8 pages
+    s.add(Request(1, [9] * 60, 60))                   # 8 pages
+    s.add(Request(2, [9] * 10, 5))                    # waits behind the full pool
+    p = s.plan()
+    assert [e.seq.request.id for e in p.entries] == [0, 1] and len(s.waiting) == 1
+    s.complete(p, [fake_token(0, 60), fake_token(1, 60)])
+    out, reasons, _, _ = run(s)
+    assert s.preemptions == 0 and all(r == "length" for r in reasons.values()) and len(out[(2, 0)]) == 5
+    # under 'max' every request takes the longest sequence: only one fits at a time
+    s = Scheduler(cache(pages=8, mode="contiguous", max_len=128), reserve_policy="max", ignore_eos=True)
+    for i in range(3):
+        s.add(Request(i, [9] * 10, 3))
+    out, reasons, _, plans = run(s)
+    assert max(len(p.entries) for p in plans) == 1 and len(out) == 3
+    # a reservation that is used up ends the request
+    s = Scheduler(cache(pages=16, mode="contiguous", max_len=64), reserve_policy="max", ignore_eos=True)
+    s.add(Request(0, [9] * 60, 100))
+    out, reasons, _, _ = run(s)
+    assert reasons[(0, 0)] == "sequence_too_long" and len(out[(0, 0)]) == 5
