@@ -4,7 +4,8 @@ slots, and the contiguous (buddy) mode as a second way of handing out the same p
 Layout.  Mixer calls with the same needs (:class:`~..parts.base.KVCacheSpec`: heads, head size,
 all keys or a window) form a *group*.  A group owns a pool of ``num_pages`` pages and one block
 table ``[seats, max_blocks]``; a page holds ``page_size`` tokens of every cache slot of the group
-(slot = one mixer call's K and V arrays ``[pages, kv_heads, page_size, head_dim]``), so one
+(slot = one mixer call's K array ``[pages, kv_heads, page_size, head_dim]`` and V array
+``[pages, kv_heads, head_dim, page_size]``), so one
 table row serves all layers of the group.  Groups with other needs have pools and tables of
 their own.
 
@@ -100,9 +101,10 @@ class CacheManager:
     def _allocate_device(self) -> None:
         import torch
         for g in self.groups:
-            shape = (len(g.slot_ids), g.num_pages, g.spec.num_kv_heads, g.page_size, g.spec.head_dim)
-            g.k = torch.zeros(shape, dtype=self.dtype, device=self.device)
-            g.v = torch.zeros(shape, dtype=self.dtype, device=self.device)
+            n, kvh, d = len(g.slot_ids), g.spec.num_kv_heads, g.spec.head_dim
+            g.k = torch.zeros((n, g.num_pages, kvh, g.page_size, d), dtype=self.dtype, device=self.device)
+            # V pages are stored transposed (see csrc/rope_cache.hip)
+            g.v = torch.zeros((n, g.num_pages, kvh, d, g.page_size), dtype=self.dtype, device=self.device)
             pinned = torch.full((self.max_seqs, self.max_blocks), -1, dtype=torch.int32,
                                 pin_memory=True)
             g._table_pinned = pinned

@@ -8,6 +8,9 @@
 // (paged_attention/src/kernels.cu:150-219): fp32 dot product, score scaled, running max m,
 // denominator l and accumulator acc in fp32, out = acc / l.  GQA: kv_head = q_head / (nq / nkv).
 //
+// K pages are [kv_head, page_size, head_dim]; V pages are stored transposed,
+// [kv_head, head_dim, page_size].
+//
 // Keys are taken in blocks of 64 aligned to absolute positions (0..63, 64..127, ...): lane i of
 // the wavefront owns key 64*b + i.  Because the blocks do not depend on where a step starts
 // or on what else is in the batch, the fp32 result for a (request, position) is bit-identical
@@ -92,7 +95,10 @@ attention_rowwise_kernel(T *__restrict__ out, const T *__restrict__ q, int q_row
         m = m_new;
         __syncthreads();  // the previous block's p_s / voff_s have been consumed
         p_s[lane] = p;
-        voff_s[lane] = row_off;
+        // V is stored transposed inside a page: [page, kv_head, head_dim, page_size]
+        voff_s[lane] = valid ? ((long long)bt[key / page_size] * num_kv_heads + kvh) *
+                                       (long long)head_dim * page_size + key % page_size
+                             : 0;
         __syncthreads();
         const int first = (kb * KVA_WAVE >= lo) ? 0 : lo - kb * KVA_WAVE;
         const int last = (pos - kb * KVA_WAVE < KVA_WAVE - 1) ? pos - kb * KVA_WAVE : KVA_WAVE - 1;
@@ -101,7 +107,8 @@ attention_rowwise_kernel(T *__restrict__ out, const T *__restrict__ q, int q_row
             const int j = lane + c * KVA_WAVE;
             if (j < head_dim) {
                 float a = acc[c] * corr;
-                for (int i = first; i <= last; ++i) a += p_s[i] * to_float(v_cache[voff_s[i] + j]);
+                for (int i = first; i <= last; ++i)
+                    a += p_s[i] * to_float(v_cache[voff_s[i] + (long long)j * page_size]);
                 acc[c] = a;
             }
         }

@@ -9,8 +9,11 @@
 // cos and sin come from fp32 tables [max_positions, rot/2] built once on the host.
 // K is rotated BEFORE it is cached, V is cached as it is.
 //
-// Cache layout (both K and V): [num_pages, num_kv_heads, page_size, head_dim]; slot s of the
-// slot mapping is page s / page_size, row s % page_size.  A negative slot skips the write.
+// Cache layout: K is [num_pages, num_kv_heads, page_size, head_dim]; V is stored transposed
+// inside a page, [num_pages, num_kv_heads, head_dim, page_size], so that the attention kernels
+// can load "several keys of one value dimension" as one vector (the matrix-core operand layout
+// of P*V).  Slot s of the slot mapping is page s / page_size, row s % page_size.  A negative
+// slot skips the write.
 #include "common.h"
 
 template <typename T>
@@ -77,7 +80,7 @@ __global__ void rope_kv_write_kernel(T *__restrict__ qkv, T *__restrict__ k_cach
         const T *v = row + (size_t)(num_q_heads + num_kv_heads) * head_dim;
         for (int w = threadIdx.x; w < num_kv_heads * head_dim; w += blockDim.x) {
             const int kvh = w / head_dim, j = w % head_dim;
-            v_cache[(((size_t)page * num_kv_heads + kvh) * page_size + off) * head_dim + j] = v[w];
+            v_cache[(((size_t)page * num_kv_heads + kvh) * head_dim + j) * page_size + off] = v[w];
         }
     }
 }

@@ -1,9 +1,32 @@
-"""Chooses the attention kernel for a step's batch."""
+"""Chooses the attention kernel for a step's batch.
+
+float32 always takes the plain kernel (true fp32 arithmetic, fixed key order).  bfloat16 takes
+the matrix-core kernel when the head size and page size allow it, and splits the keys of long
+contexts over several wavefronts when the batch alone would leave most of the GPU idle.
+"""
 from __future__ import annotations
 
 import torch
 
 from . import kernels as K
+
+# wavefronts wanted in flight: 256 compute units, a few waves each
+_TARGET_WAVES = 2048
+_MIN_KEYS_PER_SPLIT = 128
+
+
+def choose_splits(num_items: int, num_kv_heads: int, max_context: int) -> tuple:
+    """(splits, keys_per_split) for the matrix-core kernel."""
+    waves = max(1, num_items * num_kv_heads)
+    want = max(1, _TARGET_WAVES // waves)
+    most = max(1, (max_context + _MIN_KEYS_PER_SPLIT - 1) // _MIN_KEYS_PER_SPLIT)
+    splits = min(want, most)
+    if splits <= 1:
+        return 1, 0
+    per = (max_context + splits - 1) // splits
+    per = (per + 31) // 32 * 32
+    splits = (max_context + per - 1) // per
+    return (splits, per) if splits > 1 else (1, 0)
 
 
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads: int,
@@ -13,6 +36,15 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
     position-encoded) queries; keys and values are read from ``kv``."""
     if kv is None:
         raise K.KernelError("paged_attention: the mixer has no cache view")
+    if qkv.dtype == torch.bfloat16 and K.attention_mfma_supported(head_dim, kv.page_size) \
+            and qkv.shape[1] % 8 == 0:
+        group = num_q_heads // num_kv_heads
+        item_entry, item_row0 = batch.attention_items(group)
+        splits, per = choose_splits(item_entry.shape[0], num_kv_heads, batch.max_context)
+        return K.attention_mfma(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table,
+                                item_entry, item_row0, batch.entry_seat, batch.entry_q_start,
+                                batch.entry_start_pos, num_q_heads, num_kv_heads, head_dim, scale,
+                                window, splits, per)
     return K.attention_rowwise(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table,
                                batch.tok_seat, batch.positions, num_q_heads, num_kv_heads,
                                head_dim, scale, window)

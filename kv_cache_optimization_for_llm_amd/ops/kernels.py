@@ -43,6 +43,19 @@ def _opt(t: Optional[torch.Tensor], name: str, dtype: Optional[torch.dtype] = No
     return None if t is None else _dev(t, name, dtype)
 
 
+def check_cache_shapes(what: str, k_cache: torch.Tensor, v_cache: torch.Tensor, num_kv_heads: int,
+                       head_dim: int) -> None:
+    """K pages are [kv_heads, page_size, head_dim]; V pages are transposed, [kv_heads, head_dim,
+    page_size]."""
+    if k_cache.dim() != 4 or v_cache.dim() != 4:
+        raise KernelError(f"{what}: cache arrays must be 4-D")
+    pages, nkv, ps, d = k_cache.shape
+    if (nkv, d) != (num_kv_heads, head_dim) or tuple(v_cache.shape) != (pages, nkv, d, ps):
+        raise KernelError(f"{what}: K cache {tuple(k_cache.shape)} / V cache {tuple(v_cache.shape)} are "
+                          f"not [pages, {num_kv_heads}, page, {head_dim}] / [pages, {num_kv_heads}, "
+                          f"{head_dim}, page]")
+
+
 # --------------------------------------------------------------------------------------
 def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """out[t, :] = table[ids[t], :], converted to out's dtype."""
@@ -128,11 +141,11 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int, 
         rot = 2 * cos.shape[1]
     write = k_cache is not None
     if write:
-        if v_cache is None or slot_mapping is None or k_cache.shape != v_cache.shape:
+        if v_cache is None or slot_mapping is None:
             raise KernelError("rope_kv_write: K and V cache and a slot mapping are all needed")
-        if k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (num_kv_heads, page_size, head_dim):
-            raise KernelError(f"rope_kv_write: cache {tuple(k_cache.shape)} is not "
-                              f"[pages, {num_kv_heads}, {page_size}, {head_dim}]")
+        check_cache_shapes("rope_kv_write", k_cache, v_cache, num_kv_heads, head_dim)
+        if k_cache.shape[2] != page_size:
+            raise KernelError(f"rope_kv_write: cache pages hold {k_cache.shape[2]} tokens, not {page_size}")
         if k_cache.dtype != qkv.dtype or slot_mapping.shape != (tokens,):
             raise KernelError("rope_kv_write: cache dtype or slot mapping shape does not fit")
     check(hip_lib().kva_rope_kv_write(
@@ -152,9 +165,7 @@ def attention_rowwise(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_c
     tokens = out.shape[0]
     if out.shape != (tokens, num_q_heads * head_dim):
         raise KernelError("attention: out must be [T, nq * d]")
-    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or k_cache.shape[1] != num_kv_heads \
-            or k_cache.shape[3] != head_dim:
-        raise KernelError(f"attention: cache {tuple(k_cache.shape)} is not [pages, nkv, page, d]")
+    check_cache_shapes("attention", k_cache, v_cache, num_kv_heads, head_dim)
     if block_table.dim() != 2 or tok_seat.shape != (tokens,) or tok_pos.shape != (tokens,):
         raise KernelError("attention: block table [seats, blocks], one seat and position per token")
     if q.dtype != out.dtype or k_cache.dtype != out.dtype:
@@ -219,3 +230,43 @@ def mark_tokens(mask: torch.Tensor, seats: torch.Tensor, tokens: torch.Tensor) -
     check(hip_lib().kva_mark_tokens(_dev(mask, "mask", torch.uint8), _dev(seats, "seats", torch.int32),
                                     _dev(tokens, "tokens", torch.int32), n, mask.shape[1], _stream()),
           "mark_tokens")
+
+
+def attention_mfma_supported(head_dim: int, page_size: int) -> bool:
+    return bool(hip_lib().kva_attention_mfma_supported(int(head_dim), int(page_size)))
+
+
+def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cache: torch.Tensor,
+                   v_cache: torch.Tensor, block_table: torch.Tensor, item_entry: torch.Tensor,
+                   item_row0: torch.Tensor, entry_seat: torch.Tensor, entry_q_start: torch.Tensor,
+                   entry_start_pos: torch.Tensor, num_q_heads: int, num_kv_heads: int, head_dim: int,
+                   scale: float, window: int = 0, splits: int = 1, keys_per_split: int = 0) -> torch.Tensor:
+    """bf16 matrix-core attention over the paged cache.  Items are (entry, first query row) pairs
+    of 16 query rows each, row = token_in_step * (nq / nkv) + head_in_group."""
+    tokens = out.shape[0]
+    if out.dtype != torch.bfloat16 or q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16:
+        raise KernelError("attention_mfma: bfloat16 only")
+    if out.shape != (tokens, num_q_heads * head_dim):
+        raise KernelError("attention_mfma: out must be [T, nq * d]")
+    check_cache_shapes("attention_mfma", k_cache, v_cache, num_kv_heads, head_dim)
+    n_items = item_entry.shape[0]
+    n_entries = entry_seat.shape[0]
+    if item_row0.shape != (n_items,) or entry_q_start.shape != (n_entries + 1,) \
+            or entry_start_pos.shape != (n_entries,) or block_table.dim() != 2:
+        raise KernelError("attention_mfma: index arrays do not fit each other")
+    if q.data_ptr() % 16 or q_row_stride < num_q_heads * head_dim:
+        raise KernelError("attention_mfma: q view is misaligned or its stride is too small")
+    part_o = part_ml = None
+    if splits > 1:
+        part_o = torch.empty((tokens * num_q_heads, splits, head_dim), dtype=torch.float32, device=out.device)
+        part_ml = torch.empty((tokens * num_q_heads, splits, 2), dtype=torch.float32, device=out.device)
+    check(hip_lib().kva_attention_mfma(
+        _dev(out, "out"), _opt(part_o, "part_o"), _opt(part_ml, "part_ml"),
+        _dev(q, "q", contiguous=False), q_row_stride, _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
+        _dev(block_table, "block_table", torch.int32), block_table.shape[1],
+        _dev(item_entry, "item_entry", torch.int32), _dev(item_row0, "item_row0", torch.int32), n_items,
+        _dev(entry_seat, "entry_seat", torch.int32), _dev(entry_q_start, "entry_q_start", torch.int32),
+        _dev(entry_start_pos, "entry_start_pos", torch.int32), tokens * num_q_heads, num_q_heads,
+        num_kv_heads, head_dim, k_cache.shape[2], float(scale), int(window), int(splits),
+        int(keys_per_split), _stream()), "attention_mfma")
+    return out

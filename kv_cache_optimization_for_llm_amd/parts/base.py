@@ -45,8 +45,9 @@ class StateSpec:
 
 @dataclass
 class KVView:
-    """What a mixer call sees of the paged cache: its own K and V arrays
-    ``[pages, kv_heads, page_size, head_dim]``, the block table ``[seats, max_blocks]`` of its
+    """What a mixer call sees of the paged cache: its own K array
+    ``[pages, kv_heads, page_size, head_dim]`` and V array (transposed inside a page)
+    ``[pages, kv_heads, head_dim, page_size]``, the block table ``[seats, max_blocks]`` of its
     group, and for each token of the step the slot (page * page_size + row) to write to."""
 
     k_cache: torch.Tensor
