@@ -115,13 +115,13 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    for (int kstart = k_begin; kstart < k_end; kstart += 32) {
-        // ---- S^T for two 16-key tiles
-        f32x4 s[2];
+    // K operand of one 32-key block: lane (r, g) holds K[key kstart + t*16 + r][ks*KSTEP + g*KSTEP/4 ..]
+    Frag8 kf8[2][NKS];
+    Frag4 kf4[2][NKS];
+    auto load_k = [&](int kstart) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-            const int key = kstart + t * 16 + r;                        // this lane's K row
+            const int key = kstart + t * 16 + r;
             const bool kvalid = key <= item_hi && key >= item_lo;   // pages outside may be unmapped
             const bf16_t *krow = k_cache;
             if (kvalid) {
@@ -130,19 +130,57 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
             }
 #pragma unroll
             for (int ks = 0; ks < NKS; ++ks) {
-                if (KSTEP == 32) {
-                    Frag8 kf;
-                    kf.u4 = kvalid ? *reinterpret_cast<const uint4 *>(krow + ks * 32 + g * 8)
-                                   : make_uint4(0, 0, 0, 0);
-                    s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf8[ks].v, s[t], 0, 0, 0);
-                } else {
-                    Frag4 kf;
-                    kf.u2 = kvalid ? *reinterpret_cast<const uint2 *>(krow + ks * 16 + g * 4)
-                                   : make_uint2(0, 0);
-                    s[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf.v, qf4[ks].v, s[t], 0, 0, 0);
-                }
+                if (KSTEP == 32)
+                    kf8[t][ks].u4 = kvalid ? *reinterpret_cast<const uint4 *>(krow + ks * 32 + g * 8)
+                                           : make_uint4(0, 0, 0, 0);
+                else
+                    kf4[t][ks].u2 = kvalid ? *reinterpret_cast<const uint2 *>(krow + ks * 16 + g * 4)
+                                           : make_uint2(0, 0);
             }
         }
+    };
+    if (k_begin < k_end) load_k(k_begin);
+
+    for (int kstart = k_begin; kstart < k_end; kstart += 32) {
+        // ---- V^T operand of this block, issued early so the loads overlap the first product:
+        // lane (r, g) supplies V^T[dt * 16 + r][keys kstart + 4g .. +3] and [kstart + 16 + 4g .. +3]
+        Frag8 vf[NDT];
+        {
+            size_t vbase[2];
+            bool vvalid[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const int key0 = kstart + t * 16 + 4 * g;
+                vvalid[t] = key0 <= item_hi && key0 + 3 >= item_lo;
+                vbase[t] = 0;
+                if (vvalid[t]) {
+                    const int page = bt[key0 / page_size];
+                    vbase[t] = ((size_t)page * num_kv_heads + kvh) * D * page_size + key0 % page_size;
+                }
+            }
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    vf[dt].u2[t] = vvalid[t] ? *reinterpret_cast<const uint2 *>(
+                                                   v_cache + vbase[t] + (size_t)(dt * 16 + r) * page_size)
+                                             : make_uint2(0, 0);
+        }
+        // ---- S^T for two 16-key tiles
+        f32x4 s[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) {
+                if (KSTEP == 32)
+                    s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf8[t][ks].v, qf8[ks].v, s[t], 0, 0, 0);
+                else
+                    s[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf4[t][ks].v, qf4[ks].v, s[t], 0, 0, 0);
+            }
+        }
+        // the next block's K, in flight during the softmax and the second product
+        if (kstart + 32 < k_end) load_k(kstart + 32);
         // ---- mask, scale, online softmax for query row r (its keys are spread over 4 lane groups)
         float sv[8];
         float mloc = -INFINITY;
@@ -174,30 +212,11 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
         m = m_new;
 
         // ---- O^T += V^T * P^T
-        // lane (r, g) supplies V^T[dt * 16 + r][keys kstart + 4g .. +3] and [kstart + 16 + 4g .. +3]
-        size_t vbase[2];
-        bool vvalid[2];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            const int key0 = kstart + t * 16 + 4 * g;
-            vvalid[t] = key0 <= item_hi && key0 + 3 >= item_lo;
-            vbase[t] = 0;
-            if (vvalid[t]) {
-                const int page = bt[key0 / page_size];
-                vbase[t] = ((size_t)page * num_kv_heads + kvh) * D * page_size + key0 % page_size;
-            }
-        }
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt) {
-            Frag8 vf;
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-                vf.u2[t] = vvalid[t] ? *reinterpret_cast<const uint2 *>(
-                                           v_cache + vbase[t] + (size_t)(dt * 16 + r) * page_size)
-                                     : make_uint2(0, 0);
             f32x4 acc = o[dt];
             acc[0] *= corr; acc[1] *= corr; acc[2] *= corr; acc[3] *= corr;
-            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, acc, 0, 0, 0);
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf.v, acc, 0, 0, 0);
         }
     }
 
@@ -227,22 +246,35 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
     }
 }
 
-// out[row, :] = sum_s o_s * exp(m_s - M) / sum_s l_s * exp(m_s - M),  M = max_s m_s
-__global__ void attention_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o,
-                                       const float *__restrict__ part_ml, int head_dim, int splits) {
+// out[row, :] = sum_s o_s * exp(m_s - M) / sum_s l_s * exp(m_s - M),  M = max_s m_s.
+// One wavefront per row: lanes first own splits (max and denominator by wave reduction, the
+// weights go to LDS), then own value dimensions and add the weighted partials.
+#define MERGE_MAX_SPLITS 256
+__global__ void __launch_bounds__(KVA_WAVE)
+attention_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o,
+                       const float *__restrict__ part_ml, int head_dim, int splits) {
+    __shared__ float w_s[MERGE_MAX_SPLITS];
     const size_t row = blockIdx.x;
-    const float *ml = part_ml + row * splits * 2;
+    const int lane = threadIdx.x;
+    const float2 *ml = reinterpret_cast<const float2 *>(part_ml) + row * splits;
     float M = -INFINITY;
-    for (int s = 0; s < splits; ++s) M = fmaxf(M, ml[2 * s]);
+    for (int s = lane; s < splits; s += KVA_WAVE) M = fmaxf(M, ml[s].x);
+    M = wave_max(M);
     float denom = 0.f;
-    for (int s = 0; s < splits; ++s)
-        if (ml[2 * s] != -INFINITY) denom += ml[2 * s + 1] * __expf(ml[2 * s] - M);
+    for (int s = lane; s < splits; s += KVA_WAVE) {
+        const float2 v = ml[s];
+        const float w = (v.x == -INFINITY) ? 0.f : __expf(v.x - M);
+        w_s[s] = w;
+        denom += v.y * w;
+    }
+    denom = wave_sum(denom);
+    __syncthreads();
     const float inv = 1.f / denom;
-    for (int j = threadIdx.x; j < head_dim; j += blockDim.x) {
+    const float *po = part_o + row * splits * head_dim;
+    for (int j = lane; j < head_dim; j += KVA_WAVE) {
         float acc = 0.f;
-        for (int s = 0; s < splits; ++s)
-            if (ml[2 * s] != -INFINITY)
-                acc += part_o[(row * splits + s) * head_dim + j] * __expf(ml[2 * s] - M);
+#pragma unroll 8
+        for (int s = 0; s < splits; ++s) acc += po[(size_t)s * head_dim + j] * w_s[s];
         out[row * head_dim + j].bits = float_to_bf16_bits(acc * inv);
     }
 }
@@ -273,7 +305,8 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
                 "attention_mfma: head_dim %d / page_size %d not supported (head_dim a multiple of 16 up "
                 "to 128 or 160/192/224/256, page_size a multiple of 4)", head_dim, page_size);
     KVA_REQUIRE(q_row_stride % 8 == 0, "attention_mfma: query row stride %d must be a multiple of 8", q_row_stride);
-    KVA_REQUIRE(splits >= 1 && splits <= 65535 && num_kv_heads <= 65535, "attention_mfma: grid too large");
+    KVA_REQUIRE(splits >= 1 && splits <= MERGE_MAX_SPLITS && num_kv_heads <= 65535,
+                "attention_mfma: at most %d splits and 65535 kv heads", MERGE_MAX_SPLITS);
     KVA_REQUIRE(splits == 1 || (keys_per_split > 0 && keys_per_split % 32 == 0 && part_o && part_ml),
                 "attention_mfma: splits need a key count that is a multiple of 32 and a workspace");
     KVA_REQUIRE(window >= 0, "attention_mfma: negative window");

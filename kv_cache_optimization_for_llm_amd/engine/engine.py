@@ -43,6 +43,7 @@ class EngineOptions:
     cache_tokens: Optional[int] = None  # pool size in tokens (default: max_seqs * max_seq_len)
     max_seqs: int = 8                   # seats (reference: MAX_SEQUENCES)
     max_seq_len: Optional[int] = None   # longest request (default: max_position_embeddings)
+    use_graphs: bool = True             # replay decode-only steps as HIP graphs (bfloat16 engine)
     device: str = "cuda:0"
 
 
@@ -97,6 +98,10 @@ class Engine:
         self.max_seq_len = max_seq_len
         self._seat_of: Dict[object, int] = {}
         self.steps_run = 0
+        self.graphs = None
+        if options.use_graphs and self.dtype == torch.bfloat16 and self.model.graph_safe():
+            from .graphs import DecodeGraphs
+            self.graphs = DecodeGraphs(self.model, self.cache, self.device)
 
     # ------------------------------------------------------------------ requests
     def has_request(self, request_id) -> bool:
@@ -140,8 +145,7 @@ class Engine:
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Runs one batch; returns fp32 logits ``[wanted places, vocab]`` on the device, in the
         order of the entries and of each entry's ``want``."""
-        batch = self.prepare(entries)
-        logits = self.model.forward(batch, self.cache)
+        logits = self._run(entries)
         self.finish(entries)
         return logits
 
@@ -152,17 +156,35 @@ class Engine:
         for e, seat, start in zip(entries, seats, starts):
             if self._seat_of.get(e.request_id) != seat or self.cache.length(seat) != start:
                 raise EngineError(f"plan does not fit the cache: request {e.request_id!r}")
-        batch = self.prepare(entries)
-        logits = self.model.forward(batch, self.cache)
+        logits = self._run(entries)
         self.steps_run += 1
         return logits
 
-    def prepare(self, entries: Sequence[StepEntry]) -> StepBatch:
+    def _run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        seats, starts, toks, wants = self._place(entries)
+        groups = self.cache.groups
+        slot_maps = [[self.cache.slot_mapping(seat, start, len(arr), g.index)
+                      for seat, start, arr in zip(seats, starts, toks)] for g in groups]
+        self.cache.flush_tables()
+        if self.graphs is not None and all(len(t) == 1 for t in toks):
+            logits = self.graphs.run(np.asarray([t[0] for t in toks], dtype=np.int32),
+                                     np.asarray(starts, dtype=np.int32), np.asarray(seats, dtype=np.int32),
+                                     [np.concatenate(m) for m in slot_maps])
+            rows = [e for e, w in enumerate(wants) for _ in w]
+            if rows != list(range(len(entries))):
+                logits = logits[torch.tensor(rows, dtype=torch.long, device=self.device)] if rows \
+                    else logits[:0]
+            return logits
+        batch = build_batch(seats, starts, toks, wants, slot_maps, self.device)
+        return self.model.forward(batch, self.cache)
+
+    def _place(self, entries: Sequence[StepEntry]):
+        """Seats, start positions and pages for every entry of the step."""
         if not entries:
             raise EngineError("a step needs at least one entry")
         seen = set()
         seats, starts, toks, wants = [], [], [], []
-        for e in entries:
+        for e in entries:       # refuse a bad step before anything is admitted or mapped
             if e.request_id in seen:
                 raise EngineError(f"request {e.request_id!r} appears twice in one step")
             seen.add(e.request_id)
@@ -171,17 +193,20 @@ class Engine:
             arr = np.asarray(e.tokens, dtype=np.int64)
             if arr.min() < 0 or arr.max() >= self.vocab_size:
                 raise EngineError(f"request {e.request_id!r}: token id outside [0, {self.vocab_size})")
+            for i in e.want:
+                if not 0 <= i < len(arr):
+                    raise EngineError(f"request {e.request_id!r}: wanted place {i} is outside its "
+                                      f"{len(arr)} tokens")
+            toks.append(arr)
+            wants.append(list(e.want))
+        for e in entries:
             if e.request_id not in self._seat_of:
                 if self.add_request(e.request_id) is None:
                     raise CacheExhausted(f"no seat (or reservation) for request {e.request_id!r}")
             seat = self._seat_of[e.request_id]
-            start = self.cache.length(seat)
             seats.append(seat)
-            starts.append(start)
-            toks.append(arr)
-            wants.append(list(e.want))
-        # map pages for every entry, or for none
-        grown = []
+            starts.append(self.cache.length(seat))
+        # map the pages the step writes to
         for e, seat, start, arr in zip(entries, seats, starts, toks):
             if not self.cache.grow(seat, start + len(arr)):
                 need = self.cache.pages_needed(seat, start + len(arr))
@@ -189,11 +214,7 @@ class Engine:
                     f"request {e.request_id!r} needs {need} more pages for positions "
                     f"{start}..{start + len(arr) - 1} (capacity {self.cache.capacity_tokens(seat)} "
                     f"tokens, free pages {[g.free_pages() for g in self.cache.groups]})")
-            grown.append(seat)
-        slot_maps = [[self.cache.slot_mapping(seat, start, len(arr), g.index)
-                      for seat, start, arr in zip(seats, starts, toks)] for g in self.cache.groups]
-        self.cache.flush_tables()
-        return build_batch(seats, starts, toks, wants, slot_maps, self.device)
+        return seats, starts, toks, wants
 
     def finish(self, entries: Sequence[StepEntry]) -> None:
         for e in entries:

@@ -108,6 +108,17 @@ class Model:
             groups.setdefault(slot_spec[slot], []).append(slot)
         return list(groups.items()), states
 
+    def graph_safe(self) -> bool:
+        """Whether every part may be captured into a HIP graph."""
+        parts = [self.final_norm]
+        for b in self.blocks:
+            parts.append(b)
+            parts.extend(b.parts())
+            pos = getattr(b.mixer, "position", None)
+            if pos is not None:
+                parts.append(pos)
+        return all(getattr(p, "graph_safe", False) for p in parts)
+
     # ---- weights
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         return model_tensor_specs(self.spec, self.blocks, self.final_norm)

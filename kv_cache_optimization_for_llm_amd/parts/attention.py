@@ -23,6 +23,8 @@ from .linear import Linear
 
 @MIXERS.register("gqa_attention")
 class GQAAttention(Mixer):
+    graph_safe = True
+
     def __init__(self, prefix: str, *, hidden_size: int, num_heads: int, num_kv_heads: int,
                  head_dim: int, scale: float, position: PartSpec, window: int = 0):
         super().__init__(prefix)

@@ -68,6 +68,11 @@ class MixerContext:
 class Part:
     """Common behaviour: named tensors relative to a prefix."""
 
+    # True when forward() only launches kernels on the current stream over device tensors it is
+    # given or allocates with torch (no host copies, no synchronisation, no data-dependent
+    # shapes): such a part may be captured into a HIP graph.
+    graph_safe = False
+
     def __init__(self, prefix: str = ""):
         self.prefix = prefix
 

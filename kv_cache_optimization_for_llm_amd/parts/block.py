@@ -17,6 +17,8 @@ from .base import Block, MixerContext
 
 @BLOCKS.register("pre_norm")
 class PreNormBlock(Block):
+    graph_safe = True
+
     def forward(self, hidden: torch.Tensor, delta: Optional[torch.Tensor], ctx: MixerContext):
         x = self.mixer_norm.forward(hidden, delta=delta)
         a = self.mixer.forward(x, ctx)

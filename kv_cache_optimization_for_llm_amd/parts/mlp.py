@@ -18,6 +18,8 @@ from .linear import Linear
 
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(FeedForward):
+    graph_safe = True
+
     def __init__(self, prefix: str, *, hidden_size: int, intermediate_size: int):
         super().__init__(prefix)
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)

@@ -17,6 +17,8 @@ from .base import Norm
 
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, prefix: str, *, width: int, eps: float, weight_name: str = "weight"):
         super().__init__(prefix)
         self.width, self.eps = int(width), float(eps)

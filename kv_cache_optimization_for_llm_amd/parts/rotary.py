@@ -51,6 +51,8 @@ def rotary_inv_freq(rot_dim: int, theta: float, scaling: Optional[dict]) -> np.n
 
 @POSITION_ENCODINGS.register("rotary")
 class RotaryEncoding(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, *, head_dim: int, max_positions: int, theta: float,
                  scaling: Optional[dict] = None, rotary_dim: Optional[int] = None):
         super().__init__("")
@@ -82,6 +84,8 @@ class RotaryEncoding(PositionEncoding):
 @POSITION_ENCODINGS.register("none")
 class NoPositionEncoding(PositionEncoding):
     """No encoding: Q and K pass unchanged; K and V are still written to the cache."""
+
+    graph_safe = True
 
     def __init__(self, **_ignored):
         super().__init__("")
