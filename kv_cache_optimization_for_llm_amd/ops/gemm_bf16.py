@@ -1,8 +1,9 @@
 """bf16 matrix products: picks the kernel for a shape.
 
 ``linear_bf16(x, w, out)`` computes ``out = x @ w^T`` with fp32 accumulation.  ``out`` may be
-bf16 or fp32.  Shapes that no hand-written kernel covers go to the vendor GEMM library through
-``torch.matmul``, which is where the reference's engine uses cuBLAS.
+bf16 or fp32.  Up to 64 rows (decode steps, short portions) take the hand-written matrix-core
+kernel that streams the weight once (``csrc/gemm_skinny.hip``).  Other shapes go to the vendor
+GEMM library through ``torch.matmul``, which is where the reference's engine uses cuBLAS.
 """
 from __future__ import annotations
 
@@ -19,6 +20,8 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Te
                             f"{tuple(out.shape)} do not fit")
     if x.shape[0] == 0:
         return out
+    if K.gemm_skinny_supported(x.shape[0], w.shape[0], w.shape[1]):
+        return K.gemm_skinny(x, w, out)
     if out.dtype == torch.bfloat16:
         torch.matmul(x, w.t(), out=out)
     else:

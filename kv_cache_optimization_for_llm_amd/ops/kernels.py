@@ -270,3 +270,25 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
         num_kv_heads, head_dim, k_cache.shape[2], float(scale), int(window), int(splits),
         int(keys_per_split), _stream()), "attention_mfma")
     return out
+
+
+def gemm_skinny_supported(m: int, n: int, k: int) -> bool:
+    return bool(hip_lib().kva_gemm_skinny_supported(int(m), int(n), int(k)))
+
+
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, swiglu: bool = False) -> torch.Tensor:
+    """out = x @ w^T for at most 64 rows of x (bf16 operands, fp32 accumulation).  ``out`` is
+    bf16 or fp32 ``[M, N]``; with ``swiglu`` the weight is a joined ``[gate; up]`` matrix and
+    ``out`` is bf16 ``[M, N / 2]`` = silu(x gate^T) * (x up^T)."""
+    m, k = x.shape
+    n = w.shape[0]
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape != (n, k):
+        raise KernelError(f"gemm_skinny: bf16 x {tuple(x.shape)} and w {tuple(w.shape)} do not fit")
+    cols = n // 2 if swiglu else n
+    if out.shape != (m, cols) or (swiglu and out.dtype != torch.bfloat16) \
+            or out.dtype not in (torch.bfloat16, torch.float32):
+        raise KernelError(f"gemm_skinny: out {tuple(out.shape)} {out.dtype} does not fit")
+    mode = 2 if swiglu else (1 if out.dtype == torch.float32 else 0)
+    check(hip_lib().kva_gemm_skinny(_dev(out, "out"), _dev(x, "x"), _dev(w, "w"), m, n, k, k, cols, mode,
+                                    _stream()), "gemm_skinny")
+    return out

@@ -41,6 +41,8 @@ _HIP_SIGNATURES = {
     "kva_attention_rowwise": [P, P, I, P, P, P, I, P, P, I, I, I, I, I, F, I, I, P],
     "kva_attention_mfma": [P, P, P, P, I, P, P, P, I, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, P],
     "kva_attention_mfma_supported": [I, I],
+    "kva_gemm_skinny": [P, P, P, I, I, I, I, I, I, P],
+    "kva_gemm_skinny_supported": [I, I, I],
     "kva_gemm_nt_f32": [P, P, P, I, I, I, I, I, I, P],
     "kva_sample": [P, P, I, I, I, P, P, F, P, U, P, P, I, P, P],
     "kva_mark_tokens": [P, P, P, I, I, P],

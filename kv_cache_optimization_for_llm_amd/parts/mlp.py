@@ -43,7 +43,11 @@ class SwiGLU(FeedForward):
         self.down = Linear(tensors[p + "down_proj.weight"])
 
     def forward(self, x: torch.Tensor, ctx: MixerContext) -> torch.Tensor:
-        gu = self.gate_up(x)
         act = torch.empty((x.shape[0], self.intermediate_size), dtype=x.dtype, device=x.device)
-        K.silu_mul(gu, act)
+        w = self.gate_up.weight
+        if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 \
+                and K.gemm_skinny_supported(x.shape[0], w.shape[0], w.shape[1]):
+            K.gemm_skinny(x, w, act, swiglu=True)      # activation fused into the product
+        else:
+            K.silu_mul(self.gate_up(x), act)
         return self.down(act)
