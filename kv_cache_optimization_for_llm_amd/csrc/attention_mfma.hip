@@ -1,10 +1,12 @@
 // Causal grouped-query attention over the paged cache on the matrix cores (bf16, gfx950).
 //
-// One kernel serves prompt portions and decoded tokens.  Work is cut into ITEMS: an item is 16
-// consecutive "query rows" of one request and one kv head, where row = token_in_step * G + g
-// enumerates (token, query head of the kv head's group) pairs, G = num_q_heads / num_kv_heads.
-// A decoded token of a model with G <= 16 is one item; a prompt portion of n tokens is
-// ceil(n * G / 16) items.  One 64-lane wavefront runs one (item, kv head, key split).
+// One kernel serves prompt portions and decoded tokens.  Work is cut into ITEMS: an item is
+// 16 * RT consecutive "query rows" of one request and one kv head, where
+// row = token_in_step * G + g enumerates (token, query head of the kv head's group) pairs,
+// G = num_q_heads / num_kv_heads.  A decoded token of a model with G <= 16 is one item of one
+// row tile (RT = 1); prompt portions may use RT = 2 so that every key and value a wavefront
+// loads serves 32 query rows.  One 64-lane wavefront runs one
+// (item, kv head, key split).
 //
 // Everything is computed transposed so that no operand ever has to change layout:
 //     S^T = K  * Q^T     A = K rows (16 keys x head-dim slice), B = Q^T  -> lane holds, for its
@@ -16,9 +18,13 @@
 // which is free because V pages are stored transposed ([kv_head, head_dim, page_size]) and a
 // lane's 4 keys are 8 contiguous bytes.  K is loaded straight from the page
 // ([kv_head, page_size, head_dim]) in operand layout too, so there is no LDS and no barrier.
+// Operand registers are double-buffered: the loads of block i+1 are issued before block i is
+// computed.  With pages of 16 keys or a multiple, a 16-key tile lies in one page and the
+// block-table lookup is uniform over the wavefront.
 //
 // Softmax is online in fp32 per query row (running max m, denominator l), scores scaled after
-// the product; P is rounded to bf16 for the second product, the accumulator stays fp32.  Keys
+// the product and kept in the base-2 domain (exp(x) = exp2(x log2 e), one instruction); P is
+// rounded to bf16 for the second product, the accumulator stays fp32.  Keys
 // are visited in blocks of 32 aligned to absolute positions.  With `splits` > 1 each split
 // writes an un-normalised partial (o, m, l) and attention_merge combines them (flash-decoding);
 // with one split the normalised result is written directly.
@@ -30,23 +36,29 @@
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 b16x8 __attribute__((ext_vector_type(8)));
-typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 b16x2 __attribute__((ext_vector_type(2)));
 
 union Frag8 {
     b16x8 v;
-    s16x8 s;
     uint4 u4;
     uint2 u2[2];
     uint16_t h[8];
+    b16x2 p2[4];
 };
+
+// two floats -> two bf16, round to nearest even (one v_cvt_pk_bf16_f32)
+__device__ inline b16x2 pack_bf16(float a, float b) {
+    return __builtin_convertvector(f32x2{a, b}, b16x2);
+}
 union Frag4 {
     s16x4 v;
     uint2 u2;
     uint16_t h[4];
 };
 
-template <int D>
+template <int D, int RT, bool FAST>
 __global__ void __launch_bounds__(KVA_WAVE)
 attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
                       const bf16_t *__restrict__ q, int q_row_stride,
@@ -64,24 +76,32 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
     const int lane = threadIdx.x, r = lane & 15, g = lane >> 4;
     const int G = num_q_heads / num_kv_heads;
 
-    const int e = item_entry[item];
-    const int row0 = item_row0[item];
-    const int q_start = entry_q_start[e];
-    const int q_len = entry_q_start[e + 1] - q_start;
-    const int start_pos = entry_start_pos[e];
-    const int *bt = block_table + (size_t)entry_seat[e] * max_blocks;
+    // everything about the item is uniform over the wavefront: keep it in scalar registers
+    const int e = __builtin_amdgcn_readfirstlane(item_entry[item]);
+    const int row0 = __builtin_amdgcn_readfirstlane(item_row0[item]);
+    const int q_start = __builtin_amdgcn_readfirstlane(entry_q_start[e]);
+    const int q_len = __builtin_amdgcn_readfirstlane(entry_q_start[e + 1]) - q_start;
+    const int start_pos = __builtin_amdgcn_readfirstlane(entry_start_pos[e]);
+    const int *bt = block_table + (size_t)__builtin_amdgcn_readfirstlane(entry_seat[e]) * max_blocks;
     const int M = q_len * G;
 
-    const int row = row0 + r;
-    const bool row_valid = row < M;
-    const int tq = row_valid ? row / G : 0;
-    const int hg = row_valid ? row % G : 0;
-    const int head = kvh * G + hg;
-    const int my_pos = start_pos + tq;
-    const int my_lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
+    // per row tile: this lane's query row
+    bool row_valid[RT];
+    int tq[RT], head[RT], my_pos[RT], my_lo[RT], tile_hi[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int row = row0 + rt * 16 + r;
+        row_valid[rt] = row < M;
+        tq[rt] = row_valid[rt] ? row / G : 0;
+        head[rt] = kvh * G + (row_valid[rt] ? row % G : 0);
+        my_pos[rt] = start_pos + tq[rt];
+        my_lo[rt] = (window > 0 && my_pos[rt] - window + 1 > 0) ? my_pos[rt] - window + 1 : 0;
+        const int last = (row0 + rt * 16 + 15 < M - 1) ? row0 + rt * 16 + 15 : M - 1;
+        tile_hi[rt] = (row0 + rt * 16 < M) ? start_pos + last / G : -1;   // last key the tile sees
+    }
 
     // keys any row of this item may see
-    const int last_row = (row0 + 15 < M - 1) ? row0 + 15 : M - 1;
+    const int last_row = (row0 + 16 * RT - 1 < M - 1) ? row0 + 16 * RT - 1 : M - 1;
     const int item_hi = start_pos + last_row / G;                       // inclusive
     const int item_pos_lo = start_pos + row0 / G;
     const int item_lo = (window > 0 && item_pos_lo - window + 1 > 0) ? item_pos_lo - window + 1 : 0;
@@ -94,154 +114,212 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
     }
 
     // Q^T operand: lane (r, g) holds Q[row r][ks * KSTEP + g * KSTEP/4 ...]
-    Frag8 qf8[NKS];
-    Frag4 qf4[NKS];
-    {
-        const bf16_t *qrow = q + (size_t)(q_start + tq) * q_row_stride + (size_t)head * D;
+    Frag8 qf8[RT][NKS];
+    Frag4 qf4[RT][NKS];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const bf16_t *qrow = q + (size_t)(q_start + tq[rt]) * q_row_stride + (size_t)head[rt] * D;
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
             if (KSTEP == 32) {
-                qf8[ks].u4 = row_valid ? *reinterpret_cast<const uint4 *>(qrow + ks * 32 + g * 8)
-                                       : make_uint4(0, 0, 0, 0);
+                qf8[rt][ks].u4 = row_valid[rt] ? *reinterpret_cast<const uint4 *>(qrow + ks * 32 + g * 8)
+                                               : make_uint4(0, 0, 0, 0);
             } else {
-                qf4[ks].u2 = row_valid ? *reinterpret_cast<const uint2 *>(qrow + ks * 16 + g * 4)
-                                       : make_uint2(0, 0);
+                qf4[rt][ks].u2 = row_valid[rt] ? *reinterpret_cast<const uint2 *>(qrow + ks * 16 + g * 4)
+                                               : make_uint2(0, 0);
             }
         }
     }
 
-    float m = -INFINITY, l = 0.f;
-    f32x4 o[NDT];
+    float m[RT], l[RT];
+    f32x4 o[RT][NDT];
 #pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int rt = 0; rt < RT; ++rt) {
+        m[rt] = -INFINITY;
+        l[rt] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) o[rt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
 
-    // K operand of one 32-key block: lane (r, g) holds K[key kstart + t*16 + r][ks*KSTEP + g*KSTEP/4 ..]
-    Frag8 kf8[2][NKS];
-    Frag4 kf4[2][NKS];
-    auto load_k = [&](int kstart) {
+    // Operands of one 32-key block.  K: lane (r, g) holds K[key kstart + t*16 + r][ks*KSTEP +
+    // g*KSTEP/4 ..].  V^T: lane (r, g) holds V^T[dt*16 + r][keys kstart + t*16 + 4g .. +3].
+    // Two sets, so that the loads of block i+1 are in flight while block i is computed.
+    struct BlockFrags {
+        Frag8 k8[2][NKS];
+        Frag4 k4[2][NKS];
+        Frag8 v[NDT];
+    };
+    // FAST: pages of exactly 16 keys (the default).  A 16-key tile is one page, so the block-table lookup and
+    // all address arithmetic up to a per-lane constant are scalar, and every load is
+    // unconditional: a tile outside the keys the item needs is redirected to the nearest needed
+    // tile (whose page is certainly mapped) and its scores are masked away.
+    const int lo_tile = item_lo & ~15, hi_tile = item_hi & ~15;
+    const uint32_t k_lane = (uint32_t)(r * D + g * (KSTEP / 4)) * 2u;          // bytes
+    const uint32_t v_lane = (uint32_t)(r * 16 + 4 * g) * 2u;                   // bytes
+    constexpr uint32_t v_tile_stride = 16u * 16u * 2u;                         // 16 value dims
+    auto load_block = [&](BlockFrags &f, int kstart) {
+        if constexpr (FAST) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                int tile0 = kstart + t * 16;
+                tile0 = tile0 < lo_tile ? lo_tile : (tile0 > hi_tile ? hi_tile : tile0);
+                const int pg = __builtin_amdgcn_readfirstlane(bt[tile0 >> 4]);
+                const size_t page_bytes = ((size_t)pg * num_kv_heads + kvh) * (size_t)(16 * D * 2);
+                const char *kb = reinterpret_cast<const char *>(k_cache) + page_bytes;
+                const char *vb = reinterpret_cast<const char *>(v_cache) + page_bytes;
+#pragma unroll
+                for (int ks = 0; ks < NKS; ++ks) {
+                    if (KSTEP == 32)
+                        f.k8[t][ks].u4 = *reinterpret_cast<const uint4 *>(kb + k_lane + ks * 64);
+                    else
+                        f.k4[t][ks].u2 = *reinterpret_cast<const uint2 *>(kb + k_lane + ks * 32);
+                }
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt)
+                    f.v[dt].u2[t] = *reinterpret_cast<const uint2 *>(vb + v_lane + dt * v_tile_stride);
+            }
+            return;
+        }
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const int key = kstart + t * 16 + r;
-            const bool kvalid = key <= item_hi && key >= item_lo;   // pages outside may be unmapped
+            const int tile0 = kstart + t * 16;
             const bf16_t *krow = k_cache;
-            if (kvalid) {
-                const int page = bt[key / page_size];
-                krow += (((size_t)page * num_kv_heads + kvh) * page_size + key % page_size) * D;
-            }
+            size_t vbase = 0;
+            const int key = tile0 + r, key0 = tile0 + 4 * g;
+            const bool kvalid = key <= item_hi && key >= item_lo;       // pages outside may be unmapped
+            const bool vvalid = key0 <= item_hi && key0 + 3 >= item_lo;
+            if (kvalid)
+                krow += (((size_t)bt[key / page_size] * num_kv_heads + kvh) * page_size +
+                         key % page_size) * D;
+            if (vvalid)
+                vbase = ((size_t)bt[key0 / page_size] * num_kv_heads + kvh) * D * page_size +
+                        key0 % page_size;
 #pragma unroll
             for (int ks = 0; ks < NKS; ++ks) {
                 if (KSTEP == 32)
-                    kf8[t][ks].u4 = kvalid ? *reinterpret_cast<const uint4 *>(krow + ks * 32 + g * 8)
-                                           : make_uint4(0, 0, 0, 0);
+                    f.k8[t][ks].u4 = kvalid ? *reinterpret_cast<const uint4 *>(krow + ks * 32 + g * 8)
+                                            : make_uint4(0, 0, 0, 0);
                 else
-                    kf4[t][ks].u2 = kvalid ? *reinterpret_cast<const uint2 *>(krow + ks * 16 + g * 4)
-                                           : make_uint2(0, 0);
+                    f.k4[t][ks].u2 = kvalid ? *reinterpret_cast<const uint2 *>(krow + ks * 16 + g * 4)
+                                            : make_uint2(0, 0);
             }
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt)
+                f.v[dt].u2[t] = vvalid ? *reinterpret_cast<const uint2 *>(
+                                             v_cache + vbase + (size_t)(dt * 16 + r) * page_size)
+                                       : make_uint2(0, 0);
         }
     };
-    if (k_begin < k_end) load_k(k_begin);
 
-    for (int kstart = k_begin; kstart < k_end; kstart += 32) {
-        // ---- V^T operand of this block, issued early so the loads overlap the first product:
-        // lane (r, g) supplies V^T[dt * 16 + r][keys kstart + 4g .. +3] and [kstart + 16 + 4g .. +3]
-        Frag8 vf[NDT];
-        {
-            size_t vbase[2];
-            bool vvalid[2];
+    // scores are kept in the base-2 domain: exp(x) = exp2(x * log2(e))
+    const float scale2 = scale * 1.44269504088896340736f;
+    const int first_pos = start_pos + row0 / G;          // smallest position among the item's rows
+    const bool all_rows = row0 + 16 * RT <= M;
+
+    auto compute_block = [&](const BlockFrags &f, int kstart) {
+        // blocks wholly visible to every row of the item need no mask
+        const bool masked = window > 0 || kstart + 31 > first_pos || !all_rows;   // incl. redirected tiles
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            if (RT > 1 && kstart > tile_hi[rt]) continue;               // wave-uniform
+            // ---- S^T for two 16-key tiles
+            f32x4 s[2];
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-                const int key0 = kstart + t * 16 + 4 * g;
-                vvalid[t] = key0 <= item_hi && key0 + 3 >= item_lo;
-                vbase[t] = 0;
-                if (vvalid[t]) {
-                    const int page = bt[key0 / page_size];
-                    vbase[t] = ((size_t)page * num_kv_heads + kvh) * D * page_size + key0 % page_size;
+                s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < NKS; ++ks) {
+                    if (KSTEP == 32)
+                        s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k8[t][ks].v, qf8[rt][ks].v, s[t], 0, 0, 0);
+                    else
+                        s[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(f.k4[t][ks].v, qf4[rt][ks].v, s[t], 0, 0, 0);
+                }
+            }
+            // ---- scale, mask, online softmax for query row r (its keys are spread over 4 lane groups)
+            float sv[8];
+            float mloc = -INFINITY;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float x = s[t][i] * scale2;
+                    if (masked) {
+                        const int key = kstart + t * 16 + 4 * g + i;
+                        const bool vis = row_valid[rt] && key <= my_pos[rt] && key >= my_lo[rt];
+                        x = vis ? x : -INFINITY;
+                    }
+                    sv[t * 4 + i] = x;
+                    mloc = fmaxf(mloc, x);
+                }
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 16, KVA_WAVE));
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, KVA_WAVE));
+            const float m_new = fmaxf(m[rt], mloc);
+            // a row that has seen no key yet keeps m = -inf: use 0 as the reference instead
+            const float m_ref = (m_new == -INFINITY) ? 0.f : m_new;
+            const float corr = __builtin_amdgcn_exp2f(m[rt] - m_ref);
+            float lsum = 0.f;
+            Frag8 pf;
+#pragma unroll
+            for (int j = 0; j < 8; j += 2) {
+                const float p0 = __builtin_amdgcn_exp2f(sv[j] - m_ref);   // exp2(-inf) = 0
+                const float p1 = __builtin_amdgcn_exp2f(sv[j + 1] - m_ref);
+                lsum += p0 + p1;
+                pf.p2[j / 2] = pack_bf16(p0, p1);
+            }
+            lsum += __shfl_xor(lsum, 16, KVA_WAVE);
+            lsum += __shfl_xor(lsum, 32, KVA_WAVE);
+            l[rt] = l[rt] * corr + lsum;
+            m[rt] = m_new;
+            // ---- O^T += V^T * P^T
+            if (__builtin_amdgcn_ballot_w64(corr != 1.f) != 0) {           // some row's maximum moved
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt) {
+                    o[rt][dt][0] *= corr; o[rt][dt][1] *= corr; o[rt][dt][2] *= corr; o[rt][dt][3] *= corr;
                 }
             }
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-                for (int t = 0; t < 2; ++t)
-                    vf[dt].u2[t] = vvalid[t] ? *reinterpret_cast<const uint2 *>(
-                                                   v_cache + vbase[t] + (size_t)(dt * 16 + r) * page_size)
-                                             : make_uint2(0, 0);
+                o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.v[dt].v, pf.v, o[rt][dt], 0, 0, 0);
         }
-        // ---- S^T for two 16-key tiles
-        f32x4 s[2];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int ks = 0; ks < NKS; ++ks) {
-                if (KSTEP == 32)
-                    s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf8[t][ks].v, qf8[ks].v, s[t], 0, 0, 0);
-                else
-                    s[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf4[t][ks].v, qf4[ks].v, s[t], 0, 0, 0);
-            }
-        }
-        // the next block's K, in flight during the softmax and the second product
-        if (kstart + 32 < k_end) load_k(kstart + 32);
-        // ---- mask, scale, online softmax for query row r (its keys are spread over 4 lane groups)
-        float sv[8];
-        float mloc = -INFINITY;
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int key = kstart + t * 16 + 4 * g + i;
-                const bool vis = row_valid && key <= my_pos && key >= my_lo;
-                const float x = vis ? s[t][i] * scale : -INFINITY;
-                sv[t * 4 + i] = x;
-                mloc = fmaxf(mloc, x);
-            }
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 16, KVA_WAVE));
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, KVA_WAVE));
-        const float m_new = fmaxf(m, mloc);
-        const float corr = (m_new == -INFINITY) ? 1.f : __expf(m - m_new);
-        float lsum = 0.f;
-        Frag8 pf;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const float p = (sv[j] == -INFINITY) ? 0.f : __expf(sv[j] - m_new);
-            lsum += p;
-            pf.h[j] = float_to_bf16_bits(p);
-        }
-        lsum += __shfl_xor(lsum, 16, KVA_WAVE);
-        lsum += __shfl_xor(lsum, 32, KVA_WAVE);
-        l = l * corr + lsum;
-        m = m_new;
+    };
 
-        // ---- O^T += V^T * P^T
-#pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) {
-            f32x4 acc = o[dt];
-            acc[0] *= corr; acc[1] *= corr; acc[2] *= corr; acc[3] *= corr;
-            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf.v, acc, 0, 0, 0);
+    BlockFrags fa, fb;
+    if (k_begin < k_end) load_block(fa, k_begin);
+    for (int kstart = k_begin; kstart < k_end; kstart += 64) {
+        const bool second = kstart + 32 < k_end;
+        if (second) load_block(fb, kstart + 32);
+        compute_block(fa, kstart);
+        if (second) {
+            if (kstart + 64 < k_end) load_block(fa, kstart + 64);
+            compute_block(fb, kstart + 32);
         }
     }
 
     // lane (r, g) holds O[row r][dt * 16 + 4g + i]
-    if (!row_valid) return;
-    const size_t orow = (size_t)(q_start + tq) * num_q_heads + head;
-    if (splits == 1) {
-        const float inv = 1.f / l;
-        bf16_t *dst = out + orow * D;
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) {
-            Frag4 w;
+    for (int rt = 0; rt < RT; ++rt) {
+        if (!row_valid[rt]) continue;
+        const size_t orow = (size_t)(q_start + tq[rt]) * num_q_heads + head[rt];
+        if (splits == 1) {
+            const float inv = 1.f / l[rt];
+            bf16_t *dst = out + orow * D;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) w.h[i] = float_to_bf16_bits(o[dt][i] * inv);
-            *reinterpret_cast<uint2 *>(dst + dt * 16 + 4 * g) = w.u2;
-        }
-    } else {
-        float *dst = part_o + (orow * splits + split) * D;
+            for (int dt = 0; dt < NDT; ++dt) {
+                union { b16x2 p2[2]; uint2 u2; } w;
+                w.p2[0] = pack_bf16(o[rt][dt][0] * inv, o[rt][dt][1] * inv);
+                w.p2[1] = pack_bf16(o[rt][dt][2] * inv, o[rt][dt][3] * inv);
+                *reinterpret_cast<uint2 *>(dst + dt * 16 + 4 * g) = w.u2;
+            }
+        } else {
+            float *dst = part_o + (orow * splits + split) * D;
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt)
-            *reinterpret_cast<float4 *>(dst + dt * 16 + 4 * g) =
-                make_float4(o[dt][0], o[dt][1], o[dt][2], o[dt][3]);
-        if (g == 0) {
-            part_ml[(orow * splits + split) * 2] = m;
-            part_ml[(orow * splits + split) * 2 + 1] = l;
+            for (int dt = 0; dt < NDT; ++dt)
+                *reinterpret_cast<float4 *>(dst + dt * 16 + 4 * g) =
+                    make_float4(o[rt][dt][0], o[rt][dt][1], o[rt][dt][2], o[rt][dt][3]);
+            if (g == 0) {
+                part_ml[(orow * splits + split) * 2] = m[rt];
+                part_ml[(orow * splits + split) * 2 + 1] = l[rt];
+            }
         }
     }
 }
@@ -263,7 +341,7 @@ attention_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_
     float denom = 0.f;
     for (int s = lane; s < splits; s += KVA_WAVE) {
         const float2 v = ml[s];
-        const float w = (v.x == -INFINITY) ? 0.f : __expf(v.x - M);
+        const float w = (v.x == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(v.x - M);   // m is kept in the base-2 domain
         w_s[s] = w;
         denom += v.y * w;
     }
@@ -289,14 +367,21 @@ extern "C" int kva_attention_mfma_supported(int head_dim, int page_size) {
     }
 }
 
+// Row tiles per item the kernel is built with for a head size when `wide` items are asked for.
+extern "C" int kva_attention_mfma_row_tiles(int head_dim, int wide) {
+    if (!wide) return 1;
+    if (head_dim <= 128) return 2;
+    return 1;
+}
+
 extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, const void *q,
                                   int q_row_stride, const void *k_cache, const void *v_cache,
                                   const int *block_table, int max_blocks, const int *item_entry,
-                                  const int *item_row0, int num_items, const int *entry_seat,
-                                  const int *entry_q_start, const int *entry_start_pos, int total_rows,
-                                  int num_q_heads, int num_kv_heads, int head_dim, int page_size,
-                                  float scale, int window, int splits, int keys_per_split,
-                                  hipStream_t stream) {
+                                  const int *item_row0, int num_items, int row_tiles,
+                                  const int *entry_seat, const int *entry_q_start,
+                                  const int *entry_start_pos, int total_rows, int num_q_heads,
+                                  int num_kv_heads, int head_dim, int page_size, float scale, int window,
+                                  int splits, int keys_per_split, hipStream_t stream) {
     KVA_REQUIRE(num_items >= 0 && num_q_heads > 0 && num_kv_heads > 0 && max_blocks > 0,
                 "attention_mfma: bad sizes");
     KVA_REQUIRE(num_q_heads % num_kv_heads == 0, "attention_mfma: %d query heads is not a multiple of %d kv heads",
@@ -310,29 +395,32 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
     KVA_REQUIRE(splits == 1 || (keys_per_split > 0 && keys_per_split % 32 == 0 && part_o && part_ml),
                 "attention_mfma: splits need a key count that is a multiple of 32 and a workspace");
     KVA_REQUIRE(window >= 0, "attention_mfma: negative window");
+    KVA_REQUIRE(row_tiles == 1 || row_tiles == kva_attention_mfma_row_tiles(head_dim, 1),
+                "attention_mfma: %d row tiles per item is not what head_dim %d is built with", row_tiles, head_dim);
     if (num_items == 0) return KVA_OK;
     dim3 grid(num_items, num_kv_heads, splits), block(KVA_WAVE);
-#define LAUNCH(DD)                                                                              \
-    hipLaunchKernelGGL((attention_mfma_kernel<DD>), grid, block, 0, stream, (bf16_t *)out, part_o, \
-                       part_ml, (const bf16_t *)q, q_row_stride, (const bf16_t *)k_cache,        \
+    const bool fast = page_size == 16;
+#define LAUNCH(DD, RR, FF)                                                                      \
+    hipLaunchKernelGGL((attention_mfma_kernel<DD, RR, FF>), grid, block, 0, stream, (bf16_t *)out, \
+                       part_o, part_ml, (const bf16_t *)q, q_row_stride, (const bf16_t *)k_cache, \
                        (const bf16_t *)v_cache, block_table, max_blocks, item_entry, item_row0,  \
                        entry_seat, entry_q_start, entry_start_pos, num_q_heads, num_kv_heads,    \
                        page_size, scale, window, splits, keys_per_split)
+#define CASE(DD, WIDE)                                                                          \
+    case DD:                                                                                    \
+        if (row_tiles == 1) {                                                                   \
+            if (fast) LAUNCH(DD, 1, true); else LAUNCH(DD, 1, false);                           \
+        } else {                                                                                \
+            if (fast) LAUNCH(DD, WIDE, true); else LAUNCH(DD, WIDE, false);                     \
+        }                                                                                       \
+        break
     switch (head_dim) {
-    case 16: LAUNCH(16); break;
-    case 32: LAUNCH(32); break;
-    case 48: LAUNCH(48); break;
-    case 64: LAUNCH(64); break;
-    case 80: LAUNCH(80); break;
-    case 96: LAUNCH(96); break;
-    case 112: LAUNCH(112); break;
-    case 128: LAUNCH(128); break;
-    case 160: LAUNCH(160); break;
-    case 192: LAUNCH(192); break;
-    case 224: LAUNCH(224); break;
-    case 256: LAUNCH(256); break;
+    CASE(16, 2); CASE(32, 2); CASE(48, 2); CASE(64, 2);
+    CASE(80, 2); CASE(96, 2); CASE(112, 2); CASE(128, 2);
+    CASE(160, 1); CASE(192, 1); CASE(224, 1); CASE(256, 1);
     default: KVA_REQUIRE(false, "attention_mfma: head_dim %d", head_dim);
     }
+#undef CASE
 #undef LAUNCH
     KVA_CHECK_LAUNCH("attention_mfma");
     if (splits > 1) {

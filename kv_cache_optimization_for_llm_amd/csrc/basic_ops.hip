@@ -85,11 +85,110 @@ __global__ void rmsnorm_kernel(T *__restrict__ out, T *__restrict__ hidden,
     }
 }
 
+// The same for bf16 rows whose width is a multiple of 8: 16-byte loads and stores, the row (after
+// the optional add) kept in registers between the two passes when it fits.
+__device__ inline void unpack8(const uint4 &v, float (&f)[8]) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = bf16_bits_to_float((uint16_t)(w[i] & 0xffffu));
+        f[2 * i + 1] = bf16_bits_to_float((uint16_t)(w[i] >> 16));
+    }
+}
+
+__device__ inline uint4 pack8(const float (&f)[8]) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        w[i] = (uint32_t)float_to_bf16_bits(f[2 * i]) | ((uint32_t)float_to_bf16_bits(f[2 * i + 1]) << 16);
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+template <typename TW> __device__ inline void load_weight8(const TW *w, float (&f)[8]);
+template <> __device__ inline void load_weight8<bf16_t>(const bf16_t *w, float (&f)[8]) {
+    unpack8(*reinterpret_cast<const uint4 *>(w), f);
+}
+template <> __device__ inline void load_weight8<float>(const float *w, float (&f)[8]) {
+    const float4 a = *reinterpret_cast<const float4 *>(w), b = *reinterpret_cast<const float4 *>(w + 4);
+    f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+}
+
+#define RMS_VEC_CACHE 4   // vectors of 8 a thread keeps between the passes
+template <typename TW>
+__global__ void rmsnorm_vec_kernel(bf16_t *__restrict__ out, bf16_t *__restrict__ hidden,
+                                   const bf16_t *__restrict__ delta, const TW *__restrict__ weight,
+                                   const int *__restrict__ row_idx, int width, float eps) {
+    __shared__ float scratch[16];
+    const int orow = blockIdx.x;
+    const int irow = row_idx ? row_idx[orow] : orow;
+    bf16_t *x = hidden + (size_t)irow * width;
+    const bf16_t *dl = delta ? delta + (size_t)irow * width : nullptr;
+    const bool write_back = dl && !row_idx;
+    bf16_t *y = out + (size_t)orow * width;
+    float cache[RMS_VEC_CACHE][8];
+    float ss = 0.f;
+    int c = 0;
+    for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8, ++c) {
+        float v[8];
+        unpack8(*reinterpret_cast<const uint4 *>(x + i), v);
+        if (dl) {
+            float d[8];
+            unpack8(*reinterpret_cast<const uint4 *>(dl + i), d);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = bf16_bits_to_float(float_to_bf16_bits(v[j] + d[j]));
+            if (write_back) *reinterpret_cast<uint4 *>(x + i) = pack8(v);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss += v[j] * v[j];
+        if (c < RMS_VEC_CACHE) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) cache[c][j] = v[j];
+        }
+    }
+    const float total = block_sum(ss, scratch, blockDim.x / KVA_WAVE);
+    const float r = (float)sqrt((double)total / (double)width + (double)eps);
+    c = 0;
+    for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8, ++c) {
+        float v[8], w[8];
+        if (c < RMS_VEC_CACHE) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = cache[c][j];
+        } else {
+            unpack8(*reinterpret_cast<const uint4 *>(x + i), v);
+            if (dl && !write_back) {
+                float d[8];
+                unpack8(*reinterpret_cast<const uint4 *>(dl + i), d);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[j] = bf16_bits_to_float(float_to_bf16_bits(v[j] + d[j]));
+            }
+        }
+        load_weight8<TW>(weight + i, w);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = (v[j] / r) * w[j];
+        *reinterpret_cast<uint4 *>(y + i) = pack8(v);
+    }
+}
+
 extern "C" int kva_rmsnorm(void *out, void *hidden, const void *delta, const void *weight,
                            const int *row_idx, int out_rows, int width, float eps, int dtype,
                            int weight_dtype, hipStream_t stream) {
     KVA_REQUIRE(out_rows >= 0 && width > 0, "rmsnorm: bad sizes rows=%d width=%d", out_rows, width);
     if (out_rows == 0) return KVA_OK;
+    if (dtype == KVA_BF16 && width % 8 == 0) {
+        const int threads = width >= 8192 ? 1024 : (width >= 2048 ? 256 : (width >= 1024 ? 128 : 64));
+        dim3 vgrid(out_rows), vblock(threads);
+        if (weight_dtype == KVA_BF16)
+            hipLaunchKernelGGL(rmsnorm_vec_kernel<bf16_t>, vgrid, vblock, 0, stream, (bf16_t *)out,
+                               (bf16_t *)hidden, (const bf16_t *)delta, (const bf16_t *)weight, row_idx,
+                               width, eps);
+        else if (weight_dtype == KVA_F32)
+            hipLaunchKernelGGL(rmsnorm_vec_kernel<float>, vgrid, vblock, 0, stream, (bf16_t *)out,
+                               (bf16_t *)hidden, (const bf16_t *)delta, (const float *)weight, row_idx,
+                               width, eps);
+        else KVA_REQUIRE(false, "rmsnorm: unsupported weight dtype %d", weight_dtype);
+        KVA_CHECK_LAUNCH("rmsnorm");
+        return KVA_OK;
+    }
     dim3 grid(out_rows), block(width >= 2048 ? 512 : 256);
 #define LAUNCH(T, TW)                                                                      \
     hipLaunchKernelGGL((rmsnorm_kernel<T, TW>), grid, block, 0, stream, (T *)out, (T *)hidden, \
@@ -144,11 +243,33 @@ __global__ void silu_mul_kernel(T *__restrict__ out, const T *__restrict__ gate_
     }
 }
 
+__global__ void silu_mul_vec_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ gate_up, int inter) {
+    const int row = blockIdx.y;
+    const bf16_t *g = gate_up + (size_t)row * 2 * inter;
+    const bf16_t *u = g + inter;
+    bf16_t *o = out + (size_t)row * inter;
+    for (int i = (blockIdx.x * blockDim.x + threadIdx.x) * 8; i < inter; i += gridDim.x * blockDim.x * 8) {
+        float gv[8], uv[8];
+        unpack8(*reinterpret_cast<const uint4 *>(g + i), gv);
+        unpack8(*reinterpret_cast<const uint4 *>(u + i), uv);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) gv[j] = gv[j] * (1.f / (1.f + expf(-gv[j]))) * uv[j];
+        *reinterpret_cast<uint4 *>(o + i) = pack8(gv);
+    }
+}
+
 extern "C" int kva_silu_mul(void *out, const void *gate_up, int rows, int inter, int dtype,
                             hipStream_t stream) {
     KVA_REQUIRE(rows >= 0 && inter > 0, "silu_mul: bad sizes");
     KVA_REQUIRE(rows <= 65535, "silu_mul: at most 65535 rows per call, got %d", rows);
     if (rows == 0) return KVA_OK;
+    if (dtype == KVA_BF16 && inter % 8 == 0) {
+        int vbx = (inter / 8 + 255) / 256;
+        hipLaunchKernelGGL(silu_mul_vec_kernel, dim3(vbx, rows), dim3(256), 0, stream, (bf16_t *)out,
+                           (const bf16_t *)gate_up, inter);
+        KVA_CHECK_LAUNCH("silu_mul");
+        return KVA_OK;
+    }
     int bx = (inter + 255) / 256;
     if (bx > 64) bx = 64;
     dim3 grid(bx, rows), block(256);

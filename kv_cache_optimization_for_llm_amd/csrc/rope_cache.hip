@@ -85,6 +85,75 @@ __global__ void rope_kv_write_kernel(T *__restrict__ qkv, T *__restrict__ k_cach
     }
 }
 
+// bf16, full rotary (rot_dim == head_dim), head_dim a multiple of 16: a thread rotates 8 pairs at a
+// time with 16-byte loads and stores.
+__device__ inline void rk_unpack8(const uint4 &v, float (&f)[8]) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = bf16_bits_to_float((uint16_t)(w[i] & 0xffffu));
+        f[2 * i + 1] = bf16_bits_to_float((uint16_t)(w[i] >> 16));
+    }
+}
+
+__device__ inline uint4 rk_pack8(const float (&f)[8]) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        w[i] = (uint32_t)float_to_bf16_bits(f[2 * i]) | ((uint32_t)float_to_bf16_bits(f[2 * i + 1]) << 16);
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+__global__ void rope_kv_write_vec_kernel(bf16_t *__restrict__ qkv, bf16_t *__restrict__ k_cache,
+                                         bf16_t *__restrict__ v_cache, const float *__restrict__ cos_table,
+                                         const float *__restrict__ sin_table,
+                                         const int *__restrict__ positions,
+                                         const int *__restrict__ slot_mapping, int num_q_heads,
+                                         int num_kv_heads, int head_dim, int page_size, int write_cache) {
+    const int t = blockIdx.x;
+    const int row_width = (num_q_heads + 2 * num_kv_heads) * head_dim;
+    bf16_t *row = qkv + (size_t)t * row_width;
+    const int pos = positions[t];
+    const int half = head_dim / 2;
+    const float *cs = cos_table + (size_t)pos * half;
+    const float *sn = sin_table + (size_t)pos * half;
+    int slot = -1;
+    if (write_cache) slot = slot_mapping[t];
+    const int page = slot >= 0 ? slot / page_size : 0;
+    const int off = slot >= 0 ? slot % page_size : 0;
+    const int chunks = half / 8;
+    const int qk_heads = num_q_heads + num_kv_heads;
+    for (int w = threadIdx.x; w < qk_heads * chunks; w += blockDim.x) {
+        const int head = w / chunks, p0 = (w % chunks) * 8;
+        if (head >= num_q_heads && slot < 0) continue;
+        bf16_t *h = row + (size_t)head * head_dim;
+        float x1[8], x2[8], c[8], s[8], o1[8], o2[8];
+        rk_unpack8(*reinterpret_cast<const uint4 *>(h + p0), x1);
+        rk_unpack8(*reinterpret_cast<const uint4 *>(h + half + p0), x2);
+        const float4 c0 = *reinterpret_cast<const float4 *>(cs + p0), c1 = *reinterpret_cast<const float4 *>(cs + p0 + 4);
+        const float4 s0 = *reinterpret_cast<const float4 *>(sn + p0), s1 = *reinterpret_cast<const float4 *>(sn + p0 + 4);
+        c[0] = c0.x; c[1] = c0.y; c[2] = c0.z; c[3] = c0.w; c[4] = c1.x; c[5] = c1.y; c[6] = c1.z; c[7] = c1.w;
+        s[0] = s0.x; s[1] = s0.y; s[2] = s0.z; s[3] = s0.w; s[4] = s1.x; s[5] = s1.y; s[6] = s1.z; s[7] = s1.w;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            o1[j] = x1[j] * c[j] - x2[j] * s[j];
+            o2[j] = x1[j] * s[j] + x2[j] * c[j];
+        }
+        bf16_t *dst = h;
+        if (head >= num_q_heads)
+            dst = k_cache + (((size_t)page * num_kv_heads + (head - num_q_heads)) * page_size + off) * head_dim;
+        *reinterpret_cast<uint4 *>(dst + p0) = rk_pack8(o1);
+        *reinterpret_cast<uint4 *>(dst + half + p0) = rk_pack8(o2);
+    }
+    if (slot >= 0) {
+        const bf16_t *v = row + (size_t)(num_q_heads + num_kv_heads) * head_dim;
+        for (int w = threadIdx.x; w < num_kv_heads * head_dim; w += blockDim.x) {
+            const int kvh = w / head_dim, j = w % head_dim;
+            v_cache[(((size_t)page * num_kv_heads + kvh) * head_dim + j) * page_size + off] = v[w];
+        }
+    }
+}
+
 extern "C" int kva_rope_kv_write(void *qkv, void *k_cache, void *v_cache, const float *cos_table,
                                  const float *sin_table, const int *positions,
                                  const int *slot_mapping, int tokens, int num_q_heads,
@@ -99,6 +168,13 @@ extern "C" int kva_rope_kv_write(void *qkv, void *k_cache, void *v_cache, const 
                 "rope_kv_write: cache write asked for without cache, slots or page size");
     if (tokens == 0) return KVA_OK;
     dim3 grid(tokens), block(256);
+    if (dtype == KVA_BF16 && cos_table && rot_dim == head_dim && head_dim % 16 == 0) {
+        hipLaunchKernelGGL(rope_kv_write_vec_kernel, grid, block, 0, stream, (bf16_t *)qkv,
+                           (bf16_t *)k_cache, (bf16_t *)v_cache, cos_table, sin_table, positions,
+                           slot_mapping, num_q_heads, num_kv_heads, head_dim, page_size, write_cache);
+        KVA_CHECK_LAUNCH("rope_kv_write");
+        return KVA_OK;
+    }
     if (dtype == KVA_F32)
         hipLaunchKernelGGL(rope_kv_write_kernel<float>, grid, block, 0, stream, (float *)qkv,
                            (float *)k_cache, (float *)v_cache, cos_table, sin_table, positions,

@@ -45,23 +45,25 @@ class StepBatch:
     h_entry_start_pos: np.ndarray = field(repr=False, default=None)
     max_q_len: int = 0
     max_context: int = 0
-    _items: Dict[int, tuple] = field(default_factory=dict, repr=False)
+    _items: Dict[tuple, tuple] = field(default_factory=dict, repr=False)
 
-    def attention_items(self, group: int):
+    def attention_items(self, group: int, row_tiles: int = 1):
         """Work items of the matrix-core attention kernel for a query-head group size: (entry,
-        first row) of every 16 query rows, row = token_in_step * group + head_in_group."""
-        if group not in self._items:
+        first row) of every ``16 * row_tiles`` query rows, row = token_in_step * group +
+        head_in_group."""
+        key = (group, row_tiles)
+        if key not in self._items:
             lens = np.diff(self.h_entry_q_start)
             ent, row0 = [], []
             for e, n in enumerate(lens):
-                starts = np.arange(0, int(n) * group, 16, dtype=np.int32)
+                starts = np.arange(0, int(n) * group, 16 * row_tiles, dtype=np.int32)
                 ent.append(np.full(starts.shape[0], e, dtype=np.int32))
                 row0.append(starts)
             both = np.concatenate([np.concatenate(ent), np.concatenate(row0)])
             dev = torch.from_numpy(both).to(self.token_ids.device, non_blocking=True)
             n = both.shape[0] // 2
-            self._items[group] = (dev[:n], dev[n:])
-        return self._items[group]
+            self._items[key] = (dev[:n], dev[n:])
+        return self._items[key]
 
 
 def _align(n: int, a: int = 4) -> int:

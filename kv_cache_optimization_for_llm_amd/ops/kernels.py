@@ -236,13 +236,19 @@ def attention_mfma_supported(head_dim: int, page_size: int) -> bool:
     return bool(hip_lib().kva_attention_mfma_supported(int(head_dim), int(page_size)))
 
 
+def attention_mfma_row_tiles(head_dim: int, wide: bool) -> int:
+    """Row tiles (of 16 query rows) per work item the kernel offers for this head size."""
+    return int(hip_lib().kva_attention_mfma_row_tiles(int(head_dim), 1 if wide else 0))
+
+
 def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cache: torch.Tensor,
                    v_cache: torch.Tensor, block_table: torch.Tensor, item_entry: torch.Tensor,
                    item_row0: torch.Tensor, entry_seat: torch.Tensor, entry_q_start: torch.Tensor,
                    entry_start_pos: torch.Tensor, num_q_heads: int, num_kv_heads: int, head_dim: int,
-                   scale: float, window: int = 0, splits: int = 1, keys_per_split: int = 0) -> torch.Tensor:
+                   scale: float, window: int = 0, splits: int = 1, keys_per_split: int = 0,
+                   row_tiles: int = 1) -> torch.Tensor:
     """bf16 matrix-core attention over the paged cache.  Items are (entry, first query row) pairs
-    of 16 query rows each, row = token_in_step * (nq / nkv) + head_in_group."""
+    of ``16 * row_tiles`` query rows each, row = token_in_step * (nq / nkv) + head_in_group."""
     tokens = out.shape[0]
     if out.dtype != torch.bfloat16 or q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16:
         raise KernelError("attention_mfma: bfloat16 only")
@@ -265,7 +271,7 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
         _dev(q, "q", contiguous=False), q_row_stride, _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
         _dev(block_table, "block_table", torch.int32), block_table.shape[1],
         _dev(item_entry, "item_entry", torch.int32), _dev(item_row0, "item_row0", torch.int32), n_items,
-        _dev(entry_seat, "entry_seat", torch.int32), _dev(entry_q_start, "entry_q_start", torch.int32),
+        int(row_tiles), _dev(entry_seat, "entry_seat", torch.int32), _dev(entry_q_start, "entry_q_start", torch.int32),
         _dev(entry_start_pos, "entry_start_pos", torch.int32), tokens * num_q_heads, num_q_heads,
         num_kv_heads, head_dim, k_cache.shape[2], float(scale), int(window), int(splits),
         int(keys_per_split), _stream()), "attention_mfma")

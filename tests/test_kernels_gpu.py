@@ -206,10 +206,10 @@ def test_attention_rowwise(dtype, nq, nkv, d, page, window, gpu):
     close(out, want, DT[dtype], "attention_rowwise", tol32=3e-6, tol16=8e-3)
 
 
-def items_for(lens, group, gpu):
+def items_for(lens, group, gpu, row_tiles=1):
     ent, row0 = [], []
     for e, n in enumerate(lens):
-        for r in range(0, n * group, 16):
+        for r in range(0, n * group, 16 * row_tiles):
             ent.append(e)
             row0.append(r)
     return (torch.tensor(ent, dtype=torch.int32, device=gpu), torch.tensor(row0, dtype=torch.int32, device=gpu))
@@ -218,11 +218,13 @@ def items_for(lens, group, gpu):
 @pytest.mark.parametrize("nq, nkv, d, page, window", [
     (4, 2, 16, 16, 0), (6, 2, 48, 8, 0), (3, 3, 32, 4, 0), (8, 2, 64, 16, 45), (32, 8, 64, 16, 0),
     (5, 1, 80, 16, 0), (24, 8, 128, 16, 0), (4, 4, 96, 32, 33), (2, 1, 256, 16, 0), (14, 2, 112, 16, 0)])
-@pytest.mark.parametrize("splits", [1, 3])
-def test_attention_mfma(nq, nkv, d, page, window, splits, gpu):
+@pytest.mark.parametrize("splits, wide", [(1, False), (3, False), (1, True), (2, True)])
+def test_attention_mfma(nq, nkv, d, page, window, splits, wide, gpu):
     assert K.attention_mfma_supported(d, page)
     dev, want, T, stride, scale, lens = attention_case("bfloat16", nq, nkv, d, page, window, ENTRIES, 11, gpu)
-    ent, row0 = items_for(lens, nq // nkv, gpu)
+    tiles = K.attention_mfma_row_tiles(d, wide)
+    assert tiles == (1 if not wide or d > 128 else 2)
+    ent, row0 = items_for(lens, nq // nkv, gpu, tiles)
     out = torch.full((T, nq * d), float("nan"), dtype=torch.bfloat16, device=gpu)
     per = 0
     if splits > 1:
@@ -230,8 +232,8 @@ def test_attention_mfma(nq, nkv, d, page, window, splits, gpu):
         per = (per + 31) // 32 * 32
     K.attention_mfma(dev["qkv"], stride, out, dev["kc"], dev["vc"], dev["table"], ent, row0,
                      dev["entry_seat"], dev["q_start"], dev["start_pos"], nq, nkv, d, scale, window,
-                     splits, per)
-    close(out, want, torch.bfloat16, f"attention_mfma splits={splits}", tol16=8e-3)
+                     splits, per, tiles)
+    close(out, want, torch.bfloat16, f"attention_mfma splits={splits} tiles={tiles}", tol16=8e-3)
 
 
 def test_attention_finds_one_far_key_among_hundreds(gpu):
