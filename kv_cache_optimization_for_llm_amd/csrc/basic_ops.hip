@@ -308,3 +308,33 @@ extern "C" int kva_cast(void *out, const void *in, long long n, int in_dtype, in
     KVA_CHECK_LAUNCH("cast");
     return KVA_OK;
 }
+
+// ---------------------------------------------------------------------------------------
+// Finishes an RMSNorm that a matrix product's epilogue prepared: `scaled` holds
+// round(hidden * w_norm), `sumsq` [T, parts] partial sums of hidden^2 per row;
+// out[i, :] = scaled[row, :] * rsqrt(sum(sumsq[row]) / width + eps), row = row_idx[i] or i.
+__global__ void normed_rows_finish_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ scaled,
+                                          const float *__restrict__ sumsq, int parts,
+                                          const int *__restrict__ row_idx, int width, float eps) {
+    __shared__ float scratch[16];
+    const int orow = blockIdx.x;
+    const int irow = row_idx ? row_idx[orow] : orow;
+    float s = 0.f;
+    for (int p = threadIdx.x; p < parts; p += blockDim.x) s += sumsq[(size_t)irow * parts + p];
+    const float total = block_sum(s, scratch, blockDim.x / KVA_WAVE);
+    const float rinv = 1.f / (float)sqrt((double)total / (double)width + (double)eps);
+    const bf16_t *x = scaled + (size_t)irow * width;
+    bf16_t *y = out + (size_t)orow * width;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) y[i] = from_float<bf16_t>(to_float(x[i]) * rinv);
+}
+
+extern "C" int kva_normed_rows_finish(void *out, const void *scaled, const float *sumsq, int parts,
+                                      int out_rows, const int *row_idx, int width, float eps,
+                                      hipStream_t stream) {
+    KVA_REQUIRE(out_rows >= 0 && width > 0 && parts > 0, "normed_rows_finish: bad sizes");
+    if (out_rows == 0) return KVA_OK;
+    hipLaunchKernelGGL(normed_rows_finish_kernel, dim3(out_rows), dim3(256), 0, stream, (bf16_t *)out,
+                       (const bf16_t *)scaled, sumsq, parts, row_idx, width, eps);
+    KVA_CHECK_LAUNCH("normed_rows_finish");
+    return KVA_OK;
+}

@@ -9,14 +9,28 @@
 //   B = X^T, 32 of K x 16 tokens                   lane (r, g) loads X[m0 + r][k + 8g .. 8g+7]
 //   D[n0 + 4g + i][m0 + r]                         -> 4 consecutive outputs of token m0 + r
 // Both operands are read from memory directly in operand layout (16 bytes per lane).  A wave
-// keeps one accumulator per 16-token tile (MT = ceil(M / 16) <= 4), so W is read once whatever M
-// is.  K is split over `k_waves` wavefronts of a workgroup (partials summed through LDS in a
-// fixed order) so that narrow matrices still put >= 2048 waves on the 256 compute units.
+// keeps one accumulator per 16-token tile (MT = ceil(M / 16) <= 4) and per n-tile it owns
+// (NTW = 1, 2 or 4: wide matrices give a wave several n-tiles so that a loaded X fragment is
+// used several times), so W is read once whatever M is.  K is split over `k_waves` wavefronts of
+// a workgroup (partials summed through LDS in a fixed order) so that narrow matrices still put
+// about 2048 waves on the 256 compute units.
 //
 // A column of the result depends only on its own token's row of X: results do not change with
-// the batch.  Epilogues: bf16 or fp32 output; or, for a joined [gate; up] matrix, the SwiGLU
-// activation silu(gate) * up (reference siluKernel, base/src/kernels.cu:45-52) so the 2*I-wide
-// intermediate never goes to memory.
+// the batch.
+//
+// Row scaling.  With `sumsq` the rows of X are un-normalised norm inputs: X = round(h * w_norm)
+// and sumsq[m, 0..parts) are partial sums of h[m,:]^2; the product is multiplied by
+// rsqrt(sum / norm_width + eps) per token at the end (RMSNorm finished inside the product; the
+// reference runs rmsNormKernel, base/src/kernels.cu:10-36, before the GEMM).
+//
+// Epilogues.
+//   EPI_PLAIN   bf16 or fp32 output.
+//   EPI_SWIGLU  W is a joined [gate; up] matrix; output silu(gate) * up (reference siluKernel,
+//               base/src/kernels.cu:45-52): the 2*I-wide intermediate never goes to memory.
+//   EPI_RESID   the residual stream takes the product in place, hidden = round(hidden + y)
+//               (reference residualKernel, base/src/kernels.cu:38-43), and the sum is prepared for
+//               the next norm: scaled = round(hidden * w_next) and one partial sum of squares per
+//               (token, n-tile).
 #include "common.h"
 #include <math.h>
 
@@ -28,131 +42,269 @@ union GFrag8 {
     uint4 u4;
 };
 
-template <int MT, bool SWIGLU>
-__global__ void gemm_skinny_kernel(const bf16_t *__restrict__ X, const bf16_t *__restrict__ W,
-                                   void *__restrict__ Y, int M, int N, int K, int ldx, int ldy,
-                                   int k_waves, int out_f32, int inter) {
+enum { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_RESID = 2 };
+
+struct SkinnyArgs {
+    const bf16_t *X;
+    const bf16_t *W;
+    void *Y;                 // EPI_PLAIN / EPI_SWIGLU output
+    int M, N, K, ldx, ldy;
+    int k_waves, out_f32, inter;
+    // row scaling of the input (optional)
+    const float *sumsq;
+    int sumsq_parts, norm_width;
+    float eps;
+    // EPI_RESID
+    bf16_t *hidden;          // [M, N] in/out
+    const void *next_w;      // [N] weight of the next norm (bf16 or fp32), may be null
+    int next_w_f32;
+    bf16_t *scaled_out;      // [M, N]
+    float *sumsq_out;        // [M, n_tiles]
+};
+
+template <int MT, int NTW, int EPI>
+__global__ void gemm_skinny_kernel(const SkinnyArgs a) {
     extern __shared__ float red[];
-    constexpr int NACC = SWIGLU ? 2 : 1;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int waves = blockDim.x >> 6;
-    const int tiles_per_wg = waves / k_waves;
-    const int tile = blockIdx.x * tiles_per_wg + wave / k_waves;
+    const int k_waves = a.k_waves;
+    const int groups_per_wg = waves / k_waves;                 // tile groups (NTW tiles) per workgroup
+    const int group = blockIdx.x * groups_per_wg + wave / k_waves;
     const int kpart = wave % k_waves;
     const int r = lane & 15, g = lane >> 4;
-    const int rows = SWIGLU ? inter : N;                 // rows of one operand block of W
+    const int rows = EPI == EPI_SWIGLU ? a.inter : a.N;        // output columns
     const int n_tiles = (rows + 15) / 16;
-    const bool tile_ok = tile < n_tiles;
+    // EPI_SWIGLU: a wave's two tiles are the gate tile and the up tile of the same columns
+    const int out_tiles = EPI == EPI_SWIGLU ? 1 : NTW;
+    const int tile0 = group * out_tiles;
+    const bool group_ok = tile0 < n_tiles;
+    const int K = a.K;
     const int kper = K / k_waves;
     const int kbeg = kpart * kper, kend = kbeg + kper;
 
-    int row = tile * 16 + r;
-    if (row > rows - 1) row = rows - 1;
-    if (row < 0) row = 0;
-    const bf16_t *wa = W + (size_t)row * K + 8 * g;
-    const bf16_t *wb = SWIGLU ? W + (size_t)(inter + row) * K + 8 * g : nullptr;
+    const bf16_t *wp[NTW];
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+        int row;
+        if (EPI == EPI_SWIGLU) {
+            row = tile0 * 16 + r;
+            if (row > rows - 1) row = rows - 1;
+            row += t * a.inter;
+        } else {
+            row = (tile0 + t) * 16 + r;
+            if (row > rows - 1) row = rows - 1;
+        }
+        if (row < 0) row = 0;
+        wp[t] = a.W + (size_t)row * K + 8 * g;
+    }
     const bf16_t *xr[MT];
     bool xv[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = mt * 16 + r;
-        xv[mt] = m < M;
-        xr[mt] = X + (size_t)(xv[mt] ? m : 0) * ldx + 8 * g;
+        xv[mt] = m < a.M;
+        xr[mt] = a.X + (size_t)(xv[mt] ? m : 0) * a.ldx + 8 * g;
     }
 
-    gf32x4 acc[NACC][MT];
+    gf32x4 acc[NTW][MT];
 #pragma unroll
-    for (int a = 0; a < NACC; ++a)
+    for (int t = 0; t < NTW; ++t)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) acc[a][mt] = gf32x4{0.f, 0.f, 0.f, 0.f};
+        for (int mt = 0; mt < MT; ++mt) acc[t][mt] = gf32x4{0.f, 0.f, 0.f, 0.f};
 
-    if (tile_ok) {
+    // The first wave of a tile group also needs, per token, the sum of squares that finishes the
+    // input norm.  The loads are issued here, ahead of the main loop, so their latency is hidden
+    // behind the stream of W: lane group g adds a contiguous quarter of the partial sums.
+    float ssum[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) ssum[mt] = 0.f;
+    if (a.sumsq != nullptr && kpart == 0 && group_ok) {
+        const int parts = a.sumsq_parts;
+        const int q = (parts + 3) / 4;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 16 + r;
+            if (m >= a.M) continue;
+            const float *sp = a.sumsq + (size_t)m * parts;
+            const int lo = g * q, hi = (lo + q < parts) ? lo + q : parts;
+            float s = 0.f;
+            if ((parts & 15) == 0) {
+                for (int p = lo; p < hi; p += 4) {
+                    const float4 v = *reinterpret_cast<const float4 *>(sp + p);
+                    s += (v.x + v.y) + (v.z + v.w);
+                }
+            } else {
+                for (int p = lo; p < hi; ++p) s += sp[p];
+            }
+            ssum[mt] = s;
+        }
+    }
+
+    if (group_ok) {
 #pragma unroll 4
         for (int k = kbeg; k < kend; k += 32) {
-            GFrag8 a0, a1;
-            a0.u4 = *reinterpret_cast<const uint4 *>(wa + k);
-            if (SWIGLU) a1.u4 = *reinterpret_cast<const uint4 *>(wb + k);
+            GFrag8 w[NTW];
+#pragma unroll
+            for (int t = 0; t < NTW; ++t) w[t].u4 = *reinterpret_cast<const uint4 *>(wp[t] + k);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 GFrag8 x;
                 x.u4 = xv[mt] ? *reinterpret_cast<const uint4 *>(xr[mt] + k) : make_uint4(0, 0, 0, 0);
-                acc[0][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0.v, x.v, acc[0][mt], 0, 0, 0);
-                if (SWIGLU)
-                    acc[1][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1.v, x.v, acc[1][mt], 0, 0, 0);
+#pragma unroll
+                for (int t = 0; t < NTW; ++t)
+                    acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[t].v, x.v, acc[t][mt], 0, 0, 0);
             }
         }
     }
 
     if (k_waves > 1) {
-        // partial sums of the K slices, added by the first wave of each tile in slice order
-        float *mine = red + (size_t)wave * (NACC * MT * 64 * 4);
-        if (kpart != 0) {
+        // partial sums of the K slices, added by the first wave of each tile group in slice
+        // order; one token tile at a time, so the buffer does not grow with M
+        float *mine = red + (size_t)wave * (NTW * 64 * 4);
 #pragma unroll
-            for (int a = 0; a < NACC; ++a)
+        for (int mt = 0; mt < MT; ++mt) {
+            if (mt > 0) __syncthreads();
+            if (kpart != 0) {
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-                    *reinterpret_cast<float4 *>(mine + ((a * MT + mt) * 64 + lane) * 4) =
-                        make_float4(acc[a][mt][0], acc[a][mt][1], acc[a][mt][2], acc[a][mt][3]);
-        }
-        __syncthreads();
-        if (kpart == 0) {
-            for (int p = 1; p < k_waves; ++p) {
-                const float *other = red + (size_t)(wave + p) * (NACC * MT * 64 * 4);
+                for (int t = 0; t < NTW; ++t)
+                    *reinterpret_cast<float4 *>(mine + (t * 64 + lane) * 4) =
+                        make_float4(acc[t][mt][0], acc[t][mt][1], acc[t][mt][2], acc[t][mt][3]);
+            }
+            __syncthreads();
+            if (kpart == 0) {
+                for (int p = 1; p < k_waves; ++p) {
+                    const float *other = red + (size_t)(wave + p) * (NTW * 64 * 4);
 #pragma unroll
-                for (int a = 0; a < NACC; ++a)
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) {
-                        const float4 v = *reinterpret_cast<const float4 *>(other + ((a * MT + mt) * 64 + lane) * 4);
-                        acc[a][mt][0] += v.x; acc[a][mt][1] += v.y; acc[a][mt][2] += v.z; acc[a][mt][3] += v.w;
+                    for (int t = 0; t < NTW; ++t) {
+                        const float4 v = *reinterpret_cast<const float4 *>(other + (t * 64 + lane) * 4);
+                        acc[t][mt][0] += v.x; acc[t][mt][1] += v.y; acc[t][mt][2] += v.z; acc[t][mt][3] += v.w;
                     }
+                }
             }
         }
     }
-    if (kpart != 0 || !tile_ok) return;
+    if (kpart != 0 || !group_ok) return;
 
-    const int n = tile * 16 + 4 * g;                       // first of this lane's 4 outputs
+    // ---- per-token scale that finishes the input's RMSNorm (the sums were loaded before the loop)
+    float rinv[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-        const int m = mt * 16 + r;
-        if (m >= M) continue;
-        float v[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            if (SWIGLU) {
-                const float gt = acc[0][mt][i];
-                v[i] = gt * (1.f / (1.f + expf(-gt))) * acc[1][mt][i];
-            } else {
-                v[i] = acc[0][mt][i];
-            }
+        rinv[mt] = 1.f;
+        if (a.sumsq != nullptr) {
+            float s = ssum[mt];
+            s += __shfl_xor(s, 16, KVA_WAVE);
+            s += __shfl_xor(s, 32, KVA_WAVE);
+            rinv[mt] = 1.f / sqrtf(s / (float)a.norm_width + a.eps);
         }
-        if (out_f32) {
-            float *dst = reinterpret_cast<float *>(Y) + (size_t)m * ldy + n;
-            if (n + 3 < rows && (ldy % 4 == 0)) {
-                *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
-            } else {
-                for (int i = 0; i < 4; ++i)
-                    if (n + i < rows) dst[i] = v[i];
+    }
+
+#pragma unroll
+    for (int t = 0; t < out_tiles; ++t) {
+        const int tile = tile0 + t;
+        if (tile >= n_tiles) break;
+        const int n = tile * 16 + 4 * g;                   // first of this lane's 4 outputs
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 16 + r;
+            const bool m_ok = m < a.M;
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (EPI == EPI_SWIGLU) {
+                    const float gt = acc[0][mt][i] * rinv[mt];
+                    v[i] = gt * (1.f / (1.f + expf(-gt))) * (acc[1][mt][i] * rinv[mt]);
+                } else {
+                    v[i] = acc[t][mt][i] * rinv[mt];
+                }
             }
-        } else {
-            bf16_t *dst = reinterpret_cast<bf16_t *>(Y) + (size_t)m * ldy + n;
-            if (n + 3 < rows && (ldy % 4 == 0)) {
-                uint2 w;
-                w.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
-                w.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
-                *reinterpret_cast<uint2 *>(dst) = w;
+            if (EPI == EPI_RESID) {
+                float ss = 0.f;
+                if (m_ok) {
+                    bf16_t *hp = a.hidden + (size_t)m * a.N + n;
+                    bf16_t *sp = a.scaled_out + (size_t)m * a.N + n;
+                    if (n + 3 < rows && (a.N % 4 == 0)) {
+                        const uint2 hv = *reinterpret_cast<const uint2 *>(hp);
+                        const float h0[4] = {bf16_bits_to_float((uint16_t)(hv.x & 0xffffu)),
+                                             bf16_bits_to_float((uint16_t)(hv.x >> 16)),
+                                             bf16_bits_to_float((uint16_t)(hv.y & 0xffffu)),
+                                             bf16_bits_to_float((uint16_t)(hv.y >> 16))};
+                        float wn[4] = {1.f, 1.f, 1.f, 1.f};
+                        if (a.next_w != nullptr) {
+                            if (a.next_w_f32) {
+                                const float4 wv = *reinterpret_cast<const float4 *>(
+                                    reinterpret_cast<const float *>(a.next_w) + n);
+                                wn[0] = wv.x; wn[1] = wv.y; wn[2] = wv.z; wn[3] = wv.w;
+                            } else {
+                                const uint2 wv = *reinterpret_cast<const uint2 *>(
+                                    reinterpret_cast<const bf16_t *>(a.next_w) + n);
+                                wn[0] = bf16_bits_to_float((uint16_t)(wv.x & 0xffffu));
+                                wn[1] = bf16_bits_to_float((uint16_t)(wv.x >> 16));
+                                wn[2] = bf16_bits_to_float((uint16_t)(wv.y & 0xffffu));
+                                wn[3] = bf16_bits_to_float((uint16_t)(wv.y >> 16));
+                            }
+                        }
+                        uint16_t sb[4], xb[4];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            sb[i] = float_to_bf16_bits(h0[i] + v[i]);
+                            const float sv = bf16_bits_to_float(sb[i]);
+                            ss += sv * sv;
+                            xb[i] = float_to_bf16_bits(sv * wn[i]);
+                        }
+                        *reinterpret_cast<uint2 *>(hp) =
+                            make_uint2((uint32_t)sb[0] | ((uint32_t)sb[1] << 16), (uint32_t)sb[2] | ((uint32_t)sb[3] << 16));
+                        *reinterpret_cast<uint2 *>(sp) =
+                            make_uint2((uint32_t)xb[0] | ((uint32_t)xb[1] << 16), (uint32_t)xb[2] | ((uint32_t)xb[3] << 16));
+                    } else {
+                        for (int i = 0; i < 4; ++i) {
+                            if (n + i >= rows) break;
+                            const uint16_t sb = float_to_bf16_bits(to_float(hp[i]) + v[i]);
+                            hp[i].bits = sb;
+                            const float sv = bf16_bits_to_float(sb);
+                            ss += sv * sv;
+                            float wn = 1.f;
+                            if (a.next_w != nullptr)
+                                wn = a.next_w_f32 ? reinterpret_cast<const float *>(a.next_w)[n + i]
+                                                  : to_float(reinterpret_cast<const bf16_t *>(a.next_w)[n + i]);
+                            sp[i].bits = float_to_bf16_bits(sv * wn);
+                        }
+                    }
+                }
+                ss += __shfl_xor(ss, 16, KVA_WAVE);
+                ss += __shfl_xor(ss, 32, KVA_WAVE);
+                if (m_ok && g == 0) a.sumsq_out[(size_t)m * n_tiles + tile] = ss;
+                continue;
+            }
+            if (!m_ok) continue;
+            if (a.out_f32) {
+                float *dst = reinterpret_cast<float *>(a.Y) + (size_t)m * a.ldy + n;
+                if (n + 3 < rows && (a.ldy % 4 == 0)) {
+                    *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+                } else {
+                    for (int i = 0; i < 4; ++i)
+                        if (n + i < rows) dst[i] = v[i];
+                }
             } else {
-                for (int i = 0; i < 4; ++i)
-                    if (n + i < rows) dst[i].bits = float_to_bf16_bits(v[i]);
+                bf16_t *dst = reinterpret_cast<bf16_t *>(a.Y) + (size_t)m * a.ldy + n;
+                if (n + 3 < rows && (a.ldy % 4 == 0)) {
+                    uint2 w;
+                    w.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+                    w.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+                    *reinterpret_cast<uint2 *>(dst) = w;
+                } else {
+                    for (int i = 0; i < 4; ++i)
+                        if (n + i < rows) dst[i].bits = float_to_bf16_bits(v[i]);
+                }
             }
         }
     }
 }
 
-// k_waves: how many wavefronts share one n-tile's K range.  Depends on N and K only, never on M,
-// so a token's result does not depend on the batch it is in.
-static int choose_k_waves(int n_tiles, int K) {
+// k_waves: how many wavefronts share one tile group's K range.  Depends on N and K only, never
+// on M, so a token's result does not depend on the batch it is in.
+static int choose_k_waves(int groups, int K) {
     int kw = 1;
-    while (kw < 16 && n_tiles * kw < 2048 && K % (32 * kw * 2) == 0 && K / (kw * 2) >= 128) kw *= 2;
+    while (kw < 16 && groups * kw < 2048 && K % (32 * kw * 2) == 0 && K / (kw * 2) >= 128) kw *= 2;
     return kw;
 }
 
@@ -160,47 +312,67 @@ extern "C" int kva_gemm_skinny_supported(int M, int N, int K) {
     return (M >= 1 && M <= 64 && N >= 1 && K >= 32 && K % 32 == 0) ? 1 : 0;
 }
 
+// Number of partial sums of squares per token that an EPI_RESID product with N columns writes.
+extern "C" int kva_gemm_skinny_sumsq_parts(int N) { return (N + 15) / 16; }
+
+template <int NTW, int EPI>
+static void launch_mt(const SkinnyArgs &a, dim3 grid, dim3 block, size_t lds, hipStream_t stream) {
+    switch ((a.M + 15) / 16) {
+    case 1: hipLaunchKernelGGL((gemm_skinny_kernel<1, NTW, EPI>), grid, block, lds, stream, a); break;
+    case 2: hipLaunchKernelGGL((gemm_skinny_kernel<2, NTW, EPI>), grid, block, lds, stream, a); break;
+    case 3: hipLaunchKernelGGL((gemm_skinny_kernel<3, NTW, EPI>), grid, block, lds, stream, a); break;
+    default: hipLaunchKernelGGL((gemm_skinny_kernel<4, NTW, EPI>), grid, block, lds, stream, a); break;
+    }
+}
+
 // mode 0: Y bf16 [M, N]; mode 1: Y fp32 [M, N]; mode 2: W is [2*inter, K] = [gate; up], Y bf16
-// [M, inter] = silu(X gate^T) * (X up^T)
+// [M, inter] = silu(X gate^T) * (X up^T); mode 3: hidden[M, N] += X W^T in place, plus
+// scaled_out[M, N] = round(hidden * next_w) and sumsq_out[M, ceil(N/16)].
+// sumsq (optional, any mode): partial sums of squares of the un-normalised input rows.
 extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int N, int K, int ldx,
-                               int ldy, int mode, hipStream_t stream) {
+                               int ldy, int mode, const float *sumsq, int sumsq_parts, int norm_width,
+                               float eps, void *hidden, const void *next_w, int next_w_f32,
+                               void *scaled_out, float *sumsq_out, hipStream_t stream) {
     KVA_REQUIRE(kva_gemm_skinny_supported(M, N, K), "gemm_skinny: M=%d N=%d K=%d not supported "
                 "(1 <= M <= 64, K a multiple of 32)", M, N, K);
-    KVA_REQUIRE(mode >= 0 && mode <= 2, "gemm_skinny: unknown mode %d", mode);
+    KVA_REQUIRE(mode >= 0 && mode <= 3, "gemm_skinny: unknown mode %d", mode);
     KVA_REQUIRE(ldx >= K && ldx % 8 == 0, "gemm_skinny: X row stride %d must be a multiple of 8 and >= K", ldx);
     KVA_REQUIRE(mode != 2 || N % 2 == 0, "gemm_skinny: a joined [gate; up] matrix needs an even row count");
-    const int inter = mode == 2 ? N / 2 : 0;
-    const int rows = mode == 2 ? inter : N;
-    KVA_REQUIRE(ldy >= rows, "gemm_skinny: Y row stride %d is smaller than its %d columns", ldy, rows);
+    KVA_REQUIRE(sumsq == nullptr || (sumsq_parts >= 1 && norm_width >= 1),
+                "gemm_skinny: row scaling needs a part count and the norm's width");
+    KVA_REQUIRE(mode != 3 || (hidden && scaled_out && sumsq_out),
+                "gemm_skinny: the residual epilogue needs hidden, scaled_out and sumsq_out");
+    SkinnyArgs a;
+    a.X = (const bf16_t *)X; a.W = (const bf16_t *)W; a.Y = Y;
+    a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldy = ldy;
+    a.inter = mode == 2 ? N / 2 : 0;
+    a.out_f32 = mode == 1 ? 1 : 0;
+    a.sumsq = sumsq; a.sumsq_parts = sumsq_parts; a.norm_width = norm_width; a.eps = eps;
+    a.hidden = (bf16_t *)hidden; a.next_w = next_w; a.next_w_f32 = next_w_f32;
+    a.scaled_out = (bf16_t *)scaled_out; a.sumsq_out = sumsq_out;
+    const int rows = mode == 2 ? a.inter : N;
+    KVA_REQUIRE(mode == 3 || ldy >= rows, "gemm_skinny: Y row stride %d is smaller than its %d columns", ldy, rows);
     const int n_tiles = (rows + 15) / 16;
-    const int kw = choose_k_waves(n_tiles, K);
-    const int tiles_per_wg = kw >= 4 ? 1 : 4 / kw;
-    const int waves = kw * tiles_per_wg;
-    const int mt = (M + 15) / 16;
-    const int nacc = mode == 2 ? 2 : 1;
-    const size_t lds = kw > 1 ? (size_t)waves * nacc * mt * 64 * 4 * sizeof(float) : 0;
+    // tiles per wave: wide matrices reuse each loaded X fragment for several n-tiles
+    int ntw = 1;
+    if (mode == 2) ntw = 2;
+    else if (mode == 3) ntw = 1;
+    else if (n_tiles >= 4096) ntw = 4;
+    else if (n_tiles >= 2048) ntw = 2;
+    const int out_tiles = mode == 2 ? 1 : ntw;
+    const int groups = (n_tiles + out_tiles - 1) / out_tiles;
+    const int kw = choose_k_waves(groups, K);
+    a.k_waves = kw;
+    const int groups_per_wg = kw >= 4 ? 1 : 4 / kw;
+    const int waves = kw * groups_per_wg;
+    const size_t lds = kw > 1 ? (size_t)waves * ntw * 64 * 4 * sizeof(float) : 0;
     KVA_REQUIRE(lds <= 64 * 1024, "gemm_skinny: reduction buffer of %zu bytes does not fit", lds);
-    dim3 grid((n_tiles + tiles_per_wg - 1) / tiles_per_wg), block(64 * waves);
-    const int f32 = mode == 1 ? 1 : 0;
-#define LAUNCH(MTV, SW)                                                                         \
-    hipLaunchKernelGGL((gemm_skinny_kernel<MTV, SW>), grid, block, lds, stream, (const bf16_t *)X, \
-                       (const bf16_t *)W, Y, M, N, K, ldx, ldy, kw, f32, inter)
-    if (mode == 2) {
-        switch (mt) {
-        case 1: LAUNCH(1, true); break;
-        case 2: LAUNCH(2, true); break;
-        case 3: LAUNCH(3, true); break;
-        default: LAUNCH(4, true); break;
-        }
-    } else {
-        switch (mt) {
-        case 1: LAUNCH(1, false); break;
-        case 2: LAUNCH(2, false); break;
-        case 3: LAUNCH(3, false); break;
-        default: LAUNCH(4, false); break;
-        }
-    }
-#undef LAUNCH
+    dim3 grid((groups + groups_per_wg - 1) / groups_per_wg), block(64 * waves);
+    if (mode == 2) launch_mt<2, EPI_SWIGLU>(a, grid, block, lds, stream);
+    else if (mode == 3) launch_mt<1, EPI_RESID>(a, grid, block, lds, stream);
+    else if (ntw == 4) launch_mt<4, EPI_PLAIN>(a, grid, block, lds, stream);
+    else if (ntw == 2) launch_mt<2, EPI_PLAIN>(a, grid, block, lds, stream);
+    else launch_mt<1, EPI_PLAIN>(a, grid, block, lds, stream);
     KVA_CHECK_LAUNCH("gemm_skinny");
     return KVA_OK;
 }

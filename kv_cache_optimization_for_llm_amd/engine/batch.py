@@ -45,6 +45,7 @@ class StepBatch:
     h_entry_start_pos: np.ndarray = field(repr=False, default=None)
     max_q_len: int = 0
     max_context: int = 0
+    logits_for_all_rows: bool = False    # logit_rows is exactly 0, 1, ..., T-1
     _items: Dict[tuple, tuple] = field(default_factory=dict, repr=False)
 
     def attention_items(self, group: int, row_tiles: int = 1):
@@ -121,6 +122,7 @@ def build_batch(seats: Sequence[int], starts: Sequence[int], token_lists: Sequen
         entry_start_pos=view("entry_start_pos"),
         h_positions=positions, h_tok_seat=tok_seat, h_entry_seat=segs["entry_seat"],
         h_entry_q_start=q_start, h_entry_start_pos=segs["entry_start_pos"],
+        logits_for_all_rows=rows == list(range(T)),
         max_q_len=max(lens) if lens else 0,
         max_context=max((s + n for s, n in zip(starts, lens)), default=0),
     )

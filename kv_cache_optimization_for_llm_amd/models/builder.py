@@ -11,7 +11,7 @@ from . import llama as _llama   # noqa: F401  (registers LlamaForCausalLM)
 from ..config.registry import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, architecture_for)
 from ..models.spec import LayerCall, ModelSpec, TensorSpec
 from ..ops import kernels as K
-from ..parts.base import Block, KVCacheSpec, KVView, MixerContext, StateSpec
+from ..parts.base import Block, KVCacheSpec, KVView, MixerContext, NormedRows, StateSpec
 from ..parts.linear import Linear
 
 
@@ -140,8 +140,11 @@ class Model:
         hidden = torch.empty((T, self.spec.hidden_size), dtype=self.dtype, device=self.device)
         K.embed_gather(self.embedding, batch.token_ids, hidden)
         delta = None
-        for call, slot in self.calls:
+        for i, (call, slot) in enumerate(self.calls):
             block = self.blocks[call.layer]
+            # the norm that reads the residual stream after this block
+            next_norm = (self.blocks[self.calls[i + 1][0].layer].first_norm()
+                         if i + 1 < len(self.calls) else self.final_norm)
             ctx = MixerContext(batch=batch)
             group = cache.group_of(slot)
             if group is not None:
@@ -150,11 +153,17 @@ class Model:
                                 group.page_size, writes=call.writes_cache)
             if slot in cache.state:
                 ctx.state = cache.state[slot]
-            hidden, delta = block.forward(hidden, delta, ctx)
+            hidden, delta = block.forward(hidden, delta, ctx, next_norm)
         R = batch.num_logit_rows
         logits = torch.empty((R, self.spec.vocab_size), dtype=torch.float32, device=self.device)
         if R == 0:
             return logits
-        x = self.final_norm.forward(hidden, delta=delta, row_idx=batch.logit_rows)
+        if isinstance(delta, NormedRows):
+            if R == T and batch.logits_for_all_rows:
+                x = delta                    # the head's product finishes the final norm
+            else:
+                x = delta.materialize(batch.logit_rows)
+        else:
+            x = self.final_norm.forward(hidden, delta=delta, row_idx=batch.logit_rows)
         self.head(x, out=logits)
         return logits

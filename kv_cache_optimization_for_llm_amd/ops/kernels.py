@@ -282,19 +282,69 @@ def gemm_skinny_supported(m: int, n: int, k: int) -> bool:
     return bool(hip_lib().kva_gemm_skinny_supported(int(m), int(n), int(k)))
 
 
-def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, swiglu: bool = False) -> torch.Tensor:
-    """out = x @ w^T for at most 64 rows of x (bf16 operands, fp32 accumulation).  ``out`` is
-    bf16 or fp32 ``[M, N]``; with ``swiglu`` the weight is a joined ``[gate; up]`` matrix and
-    ``out`` is bf16 ``[M, N / 2]`` = silu(x gate^T) * (x up^T)."""
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor], swiglu: bool = False, *,
+                sumsq: Optional[torch.Tensor] = None, norm_width: int = 0, eps: float = 0.0,
+                hidden: Optional[torch.Tensor] = None, next_weight: Optional[torch.Tensor] = None,
+                scaled_out: Optional[torch.Tensor] = None, sumsq_out: Optional[torch.Tensor] = None):
+    """out = x @ w^T for at most 64 rows of x (bf16 operands, fp32 accumulation).
+
+    * ``out`` bf16 or fp32 ``[M, N]``; with ``swiglu`` the weight is a joined ``[gate; up]``
+      matrix and ``out`` is bf16 ``[M, N / 2]`` = silu(x gate^T) * (x up^T).
+    * ``sumsq`` ``[M, parts]`` fp32: the rows of ``x`` are un-normalised norm inputs
+      (``round(h * w_norm)``) and the product is scaled per token by
+      ``rsqrt(sum(sumsq[m]) / norm_width + eps)``.
+    * ``hidden`` (instead of ``out``): ``hidden += x @ w^T`` in place (fp32 add, rounded), plus
+      ``scaled_out = round(hidden * next_weight)`` and ``sumsq_out[M, ceil(N / 16)]``."""
     m, k = x.shape
     n = w.shape[0]
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape != (n, k):
         raise KernelError(f"gemm_skinny: bf16 x {tuple(x.shape)} and w {tuple(w.shape)} do not fit")
+    lib = hip_lib()
+    if sumsq is not None and (sumsq.dim() != 2 or sumsq.shape[0] != m or norm_width <= 0):
+        raise KernelError("gemm_skinny: sumsq must be [M, parts] and norm_width positive")
+    parts = sumsq.shape[1] if sumsq is not None else 0
+    if hidden is not None:
+        if swiglu or out is not None:
+            raise KernelError("gemm_skinny: the residual epilogue has no other output")
+        p_out = lib.kva_gemm_skinny_sumsq_parts(n)
+        if hidden.shape != (m, n) or hidden.dtype != torch.bfloat16 or scaled_out is None \
+                or scaled_out.shape != (m, n) or scaled_out.dtype != torch.bfloat16 \
+                or sumsq_out is None or sumsq_out.shape != (m, p_out):
+            raise KernelError("gemm_skinny: hidden / scaled_out [M, N] bf16 and sumsq_out [M, ceil(N/16)] needed")
+        if next_weight is not None and next_weight.shape != (n,):
+            raise KernelError("gemm_skinny: the next norm's weight must be [N]")
+        check(lib.kva_gemm_skinny(
+            None, _dev(x, "x"), _dev(w, "w"), m, n, k, k, n, 3, _opt(sumsq, "sumsq", torch.float32), parts,
+            int(norm_width), float(eps), _dev(hidden, "hidden"), _opt(next_weight, "next_weight"),
+            1 if next_weight is not None and next_weight.dtype == torch.float32 else 0,
+            _dev(scaled_out, "scaled_out"), _dev(sumsq_out, "sumsq_out", torch.float32), _stream()),
+            "gemm_skinny")
+        return hidden
     cols = n // 2 if swiglu else n
     if out.shape != (m, cols) or (swiglu and out.dtype != torch.bfloat16) \
             or out.dtype not in (torch.bfloat16, torch.float32):
         raise KernelError(f"gemm_skinny: out {tuple(out.shape)} {out.dtype} does not fit")
     mode = 2 if swiglu else (1 if out.dtype == torch.float32 else 0)
-    check(hip_lib().kva_gemm_skinny(_dev(out, "out"), _dev(x, "x"), _dev(w, "w"), m, n, k, k, cols, mode,
-                                    _stream()), "gemm_skinny")
+    check(lib.kva_gemm_skinny(_dev(out, "out"), _dev(x, "x"), _dev(w, "w"), m, n, k, k, cols, mode,
+                              _opt(sumsq, "sumsq", torch.float32), parts, int(norm_width), float(eps),
+                              None, None, 0, None, None, _stream()), "gemm_skinny")
+    return out
+
+
+def gemm_skinny_sumsq_parts(n: int) -> int:
+    return int(hip_lib().kva_gemm_skinny_sumsq_parts(int(n)))
+
+
+def normed_rows_finish(scaled: torch.Tensor, sumsq: torch.Tensor, norm_width: int, eps: float,
+                       out: torch.Tensor, row_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[i] = scaled[row] * rsqrt(sum(sumsq[row]) / norm_width + eps), row = row_idx[i] or i."""
+    rows, width = out.shape
+    if scaled.dim() != 2 or scaled.shape[1] != width or sumsq.shape[0] != scaled.shape[0] \
+            or scaled.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
+        raise KernelError("normed_rows_finish: bf16 scaled [T, H], sumsq [T, parts], out [rows, H]")
+    if row_idx is None and rows != scaled.shape[0]:
+        raise KernelError("normed_rows_finish: out needs as many rows as scaled")
+    check(hip_lib().kva_normed_rows_finish(
+        _dev(out, "out"), _dev(scaled, "scaled"), _dev(sumsq, "sumsq", torch.float32), sumsq.shape[1],
+        rows, _opt(row_idx, "row_idx", torch.int32), width, float(eps), _stream()), "normed_rows_finish")
     return out

@@ -42,7 +42,9 @@ _HIP_SIGNATURES = {
     "kva_attention_mfma": [P, P, P, P, I, P, P, P, I, P, P, I, I, P, P, P, I, I, I, I, I, F, I, I, I, P],
     "kva_attention_mfma_row_tiles": [I, I],
     "kva_attention_mfma_supported": [I, I],
-    "kva_gemm_skinny": [P, P, P, I, I, I, I, I, I, P],
+    "kva_gemm_skinny": [P, P, P, I, I, I, I, I, I, P, I, I, F, P, P, I, P, P, P],
+    "kva_gemm_skinny_sumsq_parts": [I],
+    "kva_normed_rows_finish": [P, P, P, I, I, P, I, F, P],
     "kva_gemm_skinny_supported": [I, I, I],
     "kva_gemm_nt_f32": [P, P, P, I, I, I, I, I, I, P],
     "kva_sample": [P, P, I, I, I, P, P, F, P, U, P, P, I, P, P],

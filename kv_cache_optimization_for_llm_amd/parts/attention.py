@@ -17,7 +17,7 @@ import torch
 from ..config.registry import MIXERS, POSITION_ENCODINGS
 from ..models.spec import PartSpec, TensorSpec
 from ..ops import attention as attn_ops
-from .base import KVCacheSpec, Mixer, MixerContext
+from .base import BranchTail, KVCacheSpec, Mixer, MixerContext
 from .linear import Linear
 
 
@@ -57,7 +57,12 @@ class GQAAttention(Mixer):
         return KVCacheSpec(self.num_kv_heads, self.head_dim,
                            kind="window" if self.window > 0 else "full", window=self.window)
 
-    def forward(self, x: torch.Tensor, ctx: MixerContext) -> torch.Tensor:
+    fuses_tail = True
+
+    def forward(self, x, ctx: MixerContext, tail: Optional[BranchTail] = None):
+        """``x`` may be NormedRows (the input norm is then finished inside the QKV product); with
+        a ``tail`` the output projection adds into the residual stream and prepares the next
+        norm when the shapes allow, and NormedRows are returned instead of the plain output."""
         batch, kv = ctx.batch, ctx.kv
         qkv = self.qkv(x)
         self.position.apply_and_cache(qkv, batch.positions, self.num_heads, self.num_kv_heads,
@@ -65,4 +70,8 @@ class GQAAttention(Mixer):
         out = torch.empty((x.shape[0], self.num_heads * self.head_dim), dtype=x.dtype, device=x.device)
         attn_ops.paged_attention(qkv, out, kv, batch, self.num_heads, self.num_kv_heads,
                                  self.head_dim, self.scale, self.window)
+        if tail is not None:
+            fused = self.o.into_residual(out, tail)
+            if fused is not None:
+                return fused
         return self.o(out)

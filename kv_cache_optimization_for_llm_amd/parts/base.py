@@ -9,9 +9,16 @@ checkpoint and how to run on a batch.  It never knows which model it is in.
   needs (:class:`KVCacheSpec`: all keys or a window of them) and/or a fixed-size per-request
   state (:class:`StateSpec`)
 * :class:`FeedForward`      ``forward(x, ctx)``
-* :class:`Block`            ``forward(hidden, delta, ctx)`` -> ``(hidden, delta)``: the arrangement
-  of norms, mixer, feed-forward and residual sums; ``delta`` is a branch output that has not
-  been added to the residual stream yet, so the next norm can fuse the add
+* :class:`Block`            ``forward(hidden, delta, ctx, next_norm=None)`` -> ``(hidden, delta)``:
+  the arrangement of norms, mixer, feed-forward and residual sums; ``delta`` is a branch output
+  that has not been added to the residual stream yet (the next norm fuses the add), or
+  :class:`NormedRows` when the add is done and the next norm is already prepared
+
+Fusing across parts.  A part that sets ``fuses_tail = True`` takes two optional extras in
+``forward``: its input may be :class:`NormedRows` (an unfinished norm) and ``tail``
+(:class:`BranchTail`) asks it to add its output to the residual stream and prepare the next
+norm inside its last product.  Parts without the flag get plain tensors and return plain tensors;
+the block does the rest with separate kernels.
 """
 from __future__ import annotations
 
@@ -65,6 +72,55 @@ class MixerContext:
     state: Optional[torch.Tensor] = None  # [seats, *StateSpec.shape] of this mixer call
 
 
+@dataclass
+class NormedRows:
+    """Rows of the residual stream handed to a norm that has not been finished yet.
+
+    A matrix product whose output goes into the residual stream can prepare the next norm in its
+    epilogue: ``scaled = round(hidden * norm_weight)`` and, per row, partial sums of
+    ``hidden^2`` (``sumsq [T, parts]``).  The normalised rows are
+    ``scaled * rsqrt(sum(sumsq) / width + eps)``; a product that takes them as input applies the
+    per-row factor to its result instead, so the norm costs no pass over memory.  ``norm`` is
+    the norm object these rows were prepared for."""
+
+    scaled: torch.Tensor
+    sumsq: torch.Tensor
+    width: int
+    eps: float
+    norm: object = None
+
+    @property
+    def shape(self):
+        return self.scaled.shape
+
+    @property
+    def dtype(self):
+        return self.scaled.dtype
+
+    @property
+    def device(self):
+        return self.scaled.device
+
+    def materialize(self, row_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """The normalised rows as a plain tensor (all rows, or those named by ``row_idx``)."""
+        from ..ops import kernels as K
+        rows = self.scaled.shape[0] if row_idx is None else row_idx.shape[0]
+        out = torch.empty((rows, self.scaled.shape[1]), dtype=self.scaled.dtype, device=self.scaled.device)
+        return K.normed_rows_finish(self.scaled, self.sumsq, self.width, self.eps, out, row_idx)
+
+
+@dataclass
+class BranchTail:
+    """What is to happen to a branch's output: it is added to ``hidden`` (the residual stream, in
+    place) and the sum is handed to ``norm``, the norm that reads the stream next.  A mixer or
+    feed-forward that is given a tail MAY do both inside its last product and return the
+    :class:`NormedRows` prepared for ``norm``; returning its plain output instead is always
+    allowed (the block then adds and normalises itself)."""
+
+    hidden: torch.Tensor
+    norm: object
+
+
 class Part:
     """Common behaviour: named tensors relative to a prefix."""
 
@@ -90,6 +146,11 @@ class Norm(Part):
                 row_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
         raise NotImplementedError
 
+    def prepared_by_product(self):
+        """``(weight, width, eps)`` if a product's epilogue may prepare this norm as
+        :class:`NormedRows` (it must be ``x * rsqrt(mean(x^2) + eps) * weight``), else ``None``."""
+        return None
+
 
 class PositionEncoding(Part):
     def apply_and_cache(self, qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int,
@@ -100,6 +161,8 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    fuses_tail = False      # True: forward(x, ctx, tail=None) accepts NormedRows and a BranchTail
+
     def kv_cache_spec(self) -> Optional[KVCacheSpec]:
         return None
 
@@ -111,6 +174,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    fuses_tail = False
+
     def forward(self, x: torch.Tensor, ctx: MixerContext) -> torch.Tensor:
         raise NotImplementedError
 
@@ -124,5 +189,12 @@ class Block(Part):
     def parts(self):
         return (self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward)
 
-    def forward(self, hidden: torch.Tensor, delta: Optional[torch.Tensor], ctx: MixerContext):
+    def forward(self, hidden: torch.Tensor, delta, ctx: MixerContext, next_norm: Optional[Norm] = None):
+        """``delta`` is None, a plain branch output still to be added, or NormedRows prepared for
+        this block's first norm.  ``next_norm`` is the norm that will read the stream after this
+        block (the next block's first norm or the final norm)."""
         raise NotImplementedError
+
+    def first_norm(self) -> Norm:
+        """The norm that reads the residual stream first in this block."""
+        return self.mixer_norm

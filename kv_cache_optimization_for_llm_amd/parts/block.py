@@ -12,16 +12,29 @@ from typing import Optional
 import torch
 
 from ..config.registry import BLOCKS
-from .base import Block, MixerContext
+from .base import Block, BranchTail, MixerContext, Norm, NormedRows
 
 
 @BLOCKS.register("pre_norm")
 class PreNormBlock(Block):
     graph_safe = True
 
-    def forward(self, hidden: torch.Tensor, delta: Optional[torch.Tensor], ctx: MixerContext):
-        x = self.mixer_norm.forward(hidden, delta=delta)
-        a = self.mixer.forward(x, ctx)
-        x = self.ffn_norm.forward(hidden, out=x, delta=a)
-        f = self.feed_forward.forward(x, ctx)
+    def forward(self, hidden: torch.Tensor, delta, ctx: MixerContext, next_norm: Optional[Norm] = None):
+        # first norm: already prepared by the previous product, or add-and-normalise here
+        if isinstance(delta, NormedRows):
+            x = delta if getattr(self.mixer, "fuses_tail", False) else delta.materialize()
+        else:
+            x = self.mixer_norm.forward(hidden, delta=delta)
+        if getattr(self.mixer, "fuses_tail", False):
+            a = self.mixer.forward(x, ctx, tail=BranchTail(hidden, self.ffn_norm))
+        else:
+            a = self.mixer.forward(x, ctx)
+        if isinstance(a, NormedRows):               # hidden has taken the mixer's output already
+            x = a if getattr(self.feed_forward, "fuses_tail", False) else a.materialize()
+        else:
+            x = self.ffn_norm.forward(hidden, delta=a)
+        if getattr(self.feed_forward, "fuses_tail", False):
+            f = self.feed_forward.forward(x, ctx, tail=BranchTail(hidden, next_norm))
+        else:
+            f = self.feed_forward.forward(x, ctx)
         return hidden, f

@@ -15,6 +15,7 @@ from typing import Optional
 import torch
 
 from ..ops import kernels as K
+from .base import BranchTail, NormedRows
 
 
 class Linear:
@@ -24,8 +25,42 @@ class Linear:
         self.weight = weight.contiguous()
         self.out_features, self.in_features = weight.shape
 
-    def __call__(self, x: torch.Tensor, out: Optional[torch.Tensor] = None,
+    def fusable(self, x) -> bool:
+        """Whether this product can finish a norm on its input and/or feed the residual stream
+        in its epilogue for these rows (bf16 everywhere, few rows)."""
+        return (self.weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
+                and K.gemm_skinny_supported(x.shape[0], self.out_features, self.in_features))
+
+    def into_residual(self, x, tail: BranchTail) -> Optional[NormedRows]:
+        """hidden += x @ W^T in place and the sum prepared for ``tail.norm``; ``None`` when this
+        cannot be fused (the caller then takes the plain product)."""
+        prep = tail.norm.prepared_by_product() if tail is not None and tail.norm is not None else None
+        if prep is None or not self.fusable(x) or tail.hidden.dtype != torch.bfloat16:
+            return None
+        next_w, width, eps = prep
+        if width != self.out_features:
+            return None
+        rows = x.shape[0]
+        scaled = torch.empty((rows, self.out_features), dtype=torch.bfloat16, device=x.device)
+        sumsq = torch.empty((rows, K.gemm_skinny_sumsq_parts(self.out_features)), dtype=torch.float32,
+                            device=x.device)
+        if isinstance(x, NormedRows):
+            K.gemm_skinny(x.scaled, self.weight, None, sumsq=x.sumsq, norm_width=x.width, eps=x.eps,
+                          hidden=tail.hidden, next_weight=next_w, scaled_out=scaled, sumsq_out=sumsq)
+        else:
+            K.gemm_skinny(x, self.weight, None, hidden=tail.hidden, next_weight=next_w,
+                          scaled_out=scaled, sumsq_out=sumsq)
+        return NormedRows(scaled, sumsq, width, eps, tail.norm)
+
+    def __call__(self, x, out: Optional[torch.Tensor] = None,
                  out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        if isinstance(x, NormedRows):
+            if self.fusable(x):
+                if out is None:
+                    out = torch.empty((x.shape[0], self.out_features), dtype=out_dtype or x.dtype,
+                                      device=x.device)
+                return K.gemm_skinny(x.scaled, self.weight, out, sumsq=x.sumsq, norm_width=x.width, eps=x.eps)
+            x = x.materialize()
         w = self.weight
         rows = x.shape[0]
         want = out_dtype or (out.dtype if out is not None else x.dtype)

@@ -12,7 +12,7 @@ import torch
 from ..config.registry import FEED_FORWARDS
 from ..models.spec import TensorSpec
 from ..ops import kernels as K
-from .base import FeedForward, MixerContext
+from .base import BranchTail, FeedForward, MixerContext, NormedRows
 from .linear import Linear
 
 
@@ -42,12 +42,24 @@ class SwiGLU(FeedForward):
         self.gate_up = Linear(torch.cat([g, u], dim=0))
         self.down = Linear(tensors[p + "down_proj.weight"])
 
-    def forward(self, x: torch.Tensor, ctx: MixerContext) -> torch.Tensor:
-        act = torch.empty((x.shape[0], self.intermediate_size), dtype=x.dtype, device=x.device)
+    fuses_tail = True
+
+    def forward(self, x, ctx: MixerContext, tail: Optional[BranchTail] = None):
+        """``x`` may be NormedRows; with a ``tail`` the down projection adds into the residual
+        stream and prepares the next norm when the shapes allow (NormedRows are returned)."""
+        rows = x.shape[0]
+        act = torch.empty((rows, self.intermediate_size), dtype=x.dtype, device=x.device)
         w = self.gate_up.weight
-        if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 \
-                and K.gemm_skinny_supported(x.shape[0], w.shape[0], w.shape[1]):
-            K.gemm_skinny(x, w, act, swiglu=True)      # activation fused into the product
+        if self.gate_up.fusable(x):
+            # activation fused into the product; an unfinished input norm is finished there too
+            if isinstance(x, NormedRows):
+                K.gemm_skinny(x.scaled, w, act, swiglu=True, sumsq=x.sumsq, norm_width=x.width, eps=x.eps)
+            else:
+                K.gemm_skinny(x, w, act, swiglu=True)
         else:
             K.silu_mul(self.gate_up(x), act)
+        if tail is not None:
+            fused = self.down.into_residual(act, tail)
+            if fused is not None:
+                return fused
         return self.down(act)

@@ -31,6 +31,9 @@ class RMSNorm(Norm):
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.weight = tensors[self.weight_name].contiguous()
 
+    def prepared_by_product(self):
+        return (self.weight, self.width, self.eps)
+
     def forward(self, x, out=None, delta=None, row_idx=None):
         if out is None:
             rows = x.shape[0] if row_idx is None else row_idx.shape[0]

@@ -49,3 +49,63 @@ def test_skinny_product_refuses_what_it_cannot_do(gpu):
     x, w = rnd(4, 40).to(gpu), rnd(16, 40).to(gpu)
     with pytest.raises(K.KernelError):
         K.gemm_skinny(x, w, torch.empty((4, 16), dtype=torch.bfloat16, device=gpu))
+
+
+def rms(h, w, eps):
+    return h * torch.rsqrt((h * h).mean(-1, keepdim=True) + eps) * w
+
+
+@pytest.mark.parametrize("m", [1, 8, 33, 64])
+@pytest.mark.parametrize("n, k", [(2048, 2048), (96, 160), (389, 64)])
+def test_product_adds_into_the_stream_and_prepares_the_next_norm(m, n, k, gpu):
+    """EPI_RESID: hidden += x W^T (rounded), scaled = round(hidden * w_next), partial sums of
+    hidden^2; a following product that takes (scaled, sumsq) equals norm-then-product."""
+    x, w = rnd(m, k), rnd(n, k, scale=0.05, seed=1)
+    h0 = rnd(m, n, seed=2)
+    w_next = (1 + 0.1 * torch.randn(n, generator=torch.Generator().manual_seed(3)))
+    eps = 2e-6
+    for wn in (w_next.to(torch.bfloat16), w_next.float()):            # norm weight stored in bf16 or fp32
+        hidden = h0.clone().to(gpu)
+        scaled = torch.empty((m, n), dtype=torch.bfloat16, device=gpu)
+        parts = K.gemm_skinny_sumsq_parts(n)
+        assert parts == (n + 15) // 16
+        sumsq = torch.full((m, parts), float("nan"), device=gpu)
+        K.gemm_skinny(x.to(gpu), w.to(gpu), None, hidden=hidden, next_weight=wn.to(gpu), scaled_out=scaled,
+                      sumsq_out=sumsq)
+        want_h = (h0.float() + (x.double() @ w.double().t()).float()).to(torch.bfloat16)
+        diff = (hidden.cpu().float() - want_h.float()).abs().max() / want_h.float().abs().max()
+        assert diff <= 8e-3                                            # one bf16 ulp where a sum sits on a tie
+        hf = hidden.cpu().float()
+        assert torch.allclose(sumsq.cpu().sum(-1), (hf * hf).sum(-1), rtol=1e-5)
+        assert torch.equal(scaled.cpu(), (hf * wn.float()).to(torch.bfloat16))
+        # finishing the norm alone
+        fin = torch.empty((m, n), dtype=torch.bfloat16, device=gpu)
+        K.normed_rows_finish(scaled, sumsq, n, eps, fin)
+        want_norm = rms(hf, wn.float(), eps)
+        assert (fin.cpu().float() - want_norm).abs().max() <= 1.2e-2 * want_norm.abs().max()
+        rows = torch.tensor([m - 1, 0, m - 1], dtype=torch.int32, device=gpu)
+        fin3 = torch.empty((3, n), dtype=torch.bfloat16, device=gpu)
+        K.normed_rows_finish(scaled, sumsq, n, eps, fin3, rows)
+        assert torch.equal(fin3.cpu(), fin.cpu()[rows.cpu().long()])
+        # a following product finishes the norm in its epilogue (needs its K = n to be a multiple of 32)
+        if n % 32 == 0:
+            w2 = rnd(80, n, scale=0.05, seed=4)
+            out = torch.empty((m, 80), dtype=torch.float32, device=gpu)
+            K.gemm_skinny(scaled, w2.to(gpu), out, sumsq=sumsq, norm_width=n, eps=eps)
+            want = want_norm.double() @ w2.double().t()
+            assert (out.cpu().double() - want).abs().max() <= 6e-3 * want.abs().max()
+            act = torch.empty((m, 40), dtype=torch.bfloat16, device=gpu)
+            K.gemm_skinny(scaled, w2.to(gpu), act, swiglu=True, sumsq=sumsq, norm_width=n, eps=eps)
+            g, u = want[:, :40], want[:, 40:]
+            want_act = g * (1 / (1 + torch.exp(-g))) * u
+            assert (act.cpu().double() - want_act).abs().max() <= 1e-2 * want_act.abs().max()
+
+
+def test_wide_matrices_give_a_wave_several_tiles(gpu):
+    """N >= 32768 and >= 65536 switch to 2 and 4 n-tiles per wave (the vocabulary-sized product)."""
+    for n in (32768 + 48, 65536 + 16, 128256):
+        x, w = rnd(5, 64), rnd(n, 64, scale=0.1, seed=n)
+        out = torch.full((5, n), float("nan"), dtype=torch.float32, device=gpu)
+        K.gemm_skinny(x.to(gpu), w.to(gpu), out)
+        want = x.double() @ w.double().t()
+        assert (out.cpu().double() - want).abs().max() <= 1e-5 * want.abs().max()
