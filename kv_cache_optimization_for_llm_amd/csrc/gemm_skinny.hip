@@ -8,7 +8,8 @@
 //   A = 16 rows of W (an "n-tile") x 32 of K      lane (r, g) loads W[n0 + r][k + 8g .. 8g+7]
 //   B = X^T, 32 of K x 16 tokens                   lane (r, g) loads X[m0 + r][k + 8g .. 8g+7]
 //   D[n0 + 4g + i][m0 + r]                         -> 4 consecutive outputs of token m0 + r
-// Both operands are read from memory directly in operand layout (16 bytes per lane).  A wave
+// W comes pre-tiled ([n-tile][K/32][16][32], made once at load time): a wave's 1 KiB per step is
+// contiguous.  Both operands are read from memory directly in operand layout (16 bytes per lane).  A wave
 // keeps one accumulator per 16-token tile (MT = ceil(M / 16) <= 4) and per n-tile it owns
 // (NTW = 1, 2 or 4: wide matrices give a wave several n-tiles so that a loaded X fragment is
 // used several times), so W is read once whatever M is.  K is split over `k_waves` wavefronts of
@@ -82,20 +83,16 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
     const int kper = K / k_waves;
     const int kbeg = kpart * kper, kend = kbeg + kper;
 
+    // W is stored tiled: [n-tile][K / 32][16 rows][32 of K], so the 1 KiB a wave needs per step is
+    // contiguous and a wave walks its n-tile as one sequential stream.  Lane (r, g) takes bytes
+    // (4r + g) * 16 of the chunk.  For EPI_SWIGLU the up tiles follow the gate tiles.
     const bf16_t *wp[NTW];
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
-        int row;
-        if (EPI == EPI_SWIGLU) {
-            row = tile0 * 16 + r;
-            if (row > rows - 1) row = rows - 1;
-            row += t * a.inter;
-        } else {
-            row = (tile0 + t) * 16 + r;
-            if (row > rows - 1) row = rows - 1;
-        }
-        if (row < 0) row = 0;
-        wp[t] = a.W + (size_t)row * K + 8 * g;
+        int tile = EPI == EPI_SWIGLU ? tile0 + t * n_tiles : tile0 + t;
+        const int last = (EPI == EPI_SWIGLU ? 2 * n_tiles : n_tiles) - 1;
+        if (tile > last) tile = last;
+        wp[t] = a.W + (size_t)tile * (size_t)(K / 32) * 512 + (4 * r + g) * 8;
     }
     const bf16_t *xr[MT];
     bool xv[MT];
@@ -141,11 +138,11 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
     }
 
     if (group_ok) {
-#pragma unroll 4
+#pragma unroll 8
         for (int k = kbeg; k < kend; k += 32) {
             GFrag8 w[NTW];
 #pragma unroll
-            for (int t = 0; t < NTW; ++t) w[t].u4 = *reinterpret_cast<const uint4 *>(wp[t] + k);
+            for (int t = 0; t < NTW; ++t) w[t].u4 = *reinterpret_cast<const uint4 *>(wp[t] + (size_t)k * 16);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 GFrag8 x;
@@ -304,7 +301,8 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
 // on M, so a token's result does not depend on the batch it is in.
 static int choose_k_waves(int groups, int K) {
     int kw = 1;
-    while (kw < 16 && groups * kw < 2048 && K % (32 * kw * 2) == 0 && K / (kw * 2) >= 128) kw *= 2;
+    // up to about 2048 waves, each with at least 8 steps of 32 along K
+    while (kw < 16 && groups * kw * 2 <= 2048 && K % (32 * kw * 2) == 0 && K / (kw * 2) >= 256) kw *= 2;
     return kw;
 }
 
@@ -325,6 +323,8 @@ static void launch_mt(const SkinnyArgs &a, dim3 grid, dim3 block, size_t lds, hi
     }
 }
 
+// W: the tiled copy of the [N, K] weight (rows padded to a multiple of 16 with zeros; for mode 2
+// the gate half and the up half are tiled separately, gate tiles first).
 // mode 0: Y bf16 [M, N]; mode 1: Y fp32 [M, N]; mode 2: W is [2*inter, K] = [gate; up], Y bf16
 // [M, inter] = silu(X gate^T) * (X up^T); mode 3: hidden[M, N] += X W^T in place, plus
 // scaled_out[M, N] = round(hidden * next_w) and sumsq_out[M, ceil(N/16)].
@@ -361,7 +361,7 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
     else if (n_tiles >= 2048) ntw = 2;
     const int out_tiles = mode == 2 ? 1 : ntw;
     const int groups = (n_tiles + out_tiles - 1) / out_tiles;
-    const int kw = choose_k_waves(groups, K);
+    int kw = choose_k_waves(groups, K);
     a.k_waves = kw;
     const int groups_per_wg = kw >= 4 ? 1 : 4 / kw;
     const int waves = kw * groups_per_wg;

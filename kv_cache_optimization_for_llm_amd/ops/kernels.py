@@ -282,23 +282,48 @@ def gemm_skinny_supported(m: int, n: int, k: int) -> bool:
     return bool(hip_lib().kva_gemm_skinny_supported(int(m), int(n), int(k)))
 
 
-def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor], swiglu: bool = False, *,
+class TiledWeight:
+    """A bf16 ``[N, K]`` weight re-laid for the few-rows product: ``[n-tile][K/32][16][32]``, rows
+    padded with zeros to a multiple of 16, so that the 1 KiB a wavefront needs per step is
+    contiguous.  With ``halves=2`` (a joined ``[gate; up]`` matrix) each half is tiled on its own
+    and the gate tiles come first."""
+
+    def __init__(self, weight: torch.Tensor, halves: int = 1):
+        n, k = weight.shape
+        if weight.dtype != torch.bfloat16 or k % 32 or n % halves:
+            raise KernelError(f"TiledWeight: bf16 [N, K] with K % 32 == 0 needed, got {tuple(weight.shape)} {weight.dtype}")
+        self.n, self.k, self.halves = n, k, halves
+        parts = []
+        for h in weight.view(halves, n // halves, k):
+            rows = h.shape[0]
+            pad = (-rows) % 16
+            if pad:
+                h = torch.cat([h, torch.zeros((pad, k), dtype=h.dtype, device=h.device)])
+            parts.append(h.view((rows + pad) // 16, 16, k // 32, 32).permute(0, 2, 1, 3).contiguous())
+        self.data = torch.cat(parts).contiguous()
+
+
+def gemm_skinny(x: torch.Tensor, w: TiledWeight, out: Optional[torch.Tensor], swiglu: bool = False, *,
                 sumsq: Optional[torch.Tensor] = None, norm_width: int = 0, eps: float = 0.0,
                 hidden: Optional[torch.Tensor] = None, next_weight: Optional[torch.Tensor] = None,
                 scaled_out: Optional[torch.Tensor] = None, sumsq_out: Optional[torch.Tensor] = None):
-    """out = x @ w^T for at most 64 rows of x (bf16 operands, fp32 accumulation).
+    """out = x @ W^T for at most 64 rows of x (bf16 operands, fp32 accumulation); ``w`` is the
+    :class:`TiledWeight` of W.
 
     * ``out`` bf16 or fp32 ``[M, N]``; with ``swiglu`` the weight is a joined ``[gate; up]``
-      matrix and ``out`` is bf16 ``[M, N / 2]`` = silu(x gate^T) * (x up^T).
+      matrix (tiled with ``halves=2``) and ``out`` is bf16 ``[M, N / 2]`` = silu(x gate^T) * (x up^T).
     * ``sumsq`` ``[M, parts]`` fp32: the rows of ``x`` are un-normalised norm inputs
       (``round(h * w_norm)``) and the product is scaled per token by
       ``rsqrt(sum(sumsq[m]) / norm_width + eps)``.
-    * ``hidden`` (instead of ``out``): ``hidden += x @ w^T`` in place (fp32 add, rounded), plus
+    * ``hidden`` (instead of ``out``): ``hidden += x @ W^T`` in place (fp32 add, rounded), plus
       ``scaled_out = round(hidden * next_weight)`` and ``sumsq_out[M, ceil(N / 16)]``."""
+    if not isinstance(w, TiledWeight):
+        raise KernelError("gemm_skinny: the weight must be a TiledWeight")
     m, k = x.shape
-    n = w.shape[0]
-    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape != (n, k):
-        raise KernelError(f"gemm_skinny: bf16 x {tuple(x.shape)} and w {tuple(w.shape)} do not fit")
+    n = w.n
+    if x.dtype != torch.bfloat16 or k != w.k or (swiglu != (w.halves == 2)):
+        raise KernelError(f"gemm_skinny: bf16 x {tuple(x.shape)} does not fit weight [{w.n}, {w.k}] "
+                          f"(halves {w.halves})")
     lib = hip_lib()
     if sumsq is not None and (sumsq.dim() != 2 or sumsq.shape[0] != m or norm_width <= 0):
         raise KernelError("gemm_skinny: sumsq must be [M, parts] and norm_width positive")
@@ -314,7 +339,7 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor], s
         if next_weight is not None and next_weight.shape != (n,):
             raise KernelError("gemm_skinny: the next norm's weight must be [N]")
         check(lib.kva_gemm_skinny(
-            None, _dev(x, "x"), _dev(w, "w"), m, n, k, k, n, 3, _opt(sumsq, "sumsq", torch.float32), parts,
+            None, _dev(x, "x"), _dev(w.data, "w"), m, n, k, k, n, 3, _opt(sumsq, "sumsq", torch.float32), parts,
             int(norm_width), float(eps), _dev(hidden, "hidden"), _opt(next_weight, "next_weight"),
             1 if next_weight is not None and next_weight.dtype == torch.float32 else 0,
             _dev(scaled_out, "scaled_out"), _dev(sumsq_out, "sumsq_out", torch.float32), _stream()),
@@ -325,7 +350,7 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor], s
             or out.dtype not in (torch.bfloat16, torch.float32):
         raise KernelError(f"gemm_skinny: out {tuple(out.shape)} {out.dtype} does not fit")
     mode = 2 if swiglu else (1 if out.dtype == torch.float32 else 0)
-    check(lib.kva_gemm_skinny(_dev(out, "out"), _dev(x, "x"), _dev(w, "w"), m, n, k, k, cols, mode,
+    check(lib.kva_gemm_skinny(_dev(out, "out"), _dev(x, "x"), _dev(w.data, "w"), m, n, k, k, cols, mode,
                               _opt(sumsq, "sumsq", torch.float32), parts, int(norm_width), float(eps),
                               None, None, 0, None, None, _stream()), "gemm_skinny")
     return out

@@ -19,17 +19,23 @@ from .base import BranchTail, NormedRows
 
 
 class Linear:
-    def __init__(self, weight: torch.Tensor):
+    def __init__(self, weight: torch.Tensor, halves: int = 1):
+        """``halves=2``: the weight is two matrices joined along the rows (gate and up)."""
         if weight.dim() != 2:
             raise ValueError(f"Linear weight must be 2-D, got {tuple(weight.shape)}")
         self.weight = weight.contiguous()
         self.out_features, self.in_features = weight.shape
+        # a second, tiled copy for the few-rows kernel (decode); the plain layout serves prompts
+        self.tiled = None
+        if weight.is_cuda and weight.dtype == torch.bfloat16 and self.in_features % 32 == 0:
+            self.tiled = K.TiledWeight(self.weight, halves)
 
     def fusable(self, x) -> bool:
         """Whether this product can finish a norm on its input and/or feed the residual stream
         in its epilogue for these rows (bf16 everywhere, few rows)."""
-        return (self.weight.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
-                and K.gemm_skinny_supported(x.shape[0], self.out_features, self.in_features))
+        from ..ops.gemm_bf16 import use_skinny
+        return (self.tiled is not None and x.dtype == torch.bfloat16
+                and use_skinny(x.shape[0], self.out_features, self.in_features))
 
     def into_residual(self, x, tail: BranchTail) -> Optional[NormedRows]:
         """hidden += x @ W^T in place and the sum prepared for ``tail.norm``; ``None`` when this
@@ -45,10 +51,10 @@ class Linear:
         sumsq = torch.empty((rows, K.gemm_skinny_sumsq_parts(self.out_features)), dtype=torch.float32,
                             device=x.device)
         if isinstance(x, NormedRows):
-            K.gemm_skinny(x.scaled, self.weight, None, sumsq=x.sumsq, norm_width=x.width, eps=x.eps,
+            K.gemm_skinny(x.scaled, self.tiled, None, sumsq=x.sumsq, norm_width=x.width, eps=x.eps,
                           hidden=tail.hidden, next_weight=next_w, scaled_out=scaled, sumsq_out=sumsq)
         else:
-            K.gemm_skinny(x, self.weight, None, hidden=tail.hidden, next_weight=next_w,
+            K.gemm_skinny(x, self.tiled, None, hidden=tail.hidden, next_weight=next_w,
                           scaled_out=scaled, sumsq_out=sumsq)
         return NormedRows(scaled, sumsq, width, eps, tail.norm)
 
@@ -59,7 +65,7 @@ class Linear:
                 if out is None:
                     out = torch.empty((x.shape[0], self.out_features), dtype=out_dtype or x.dtype,
                                       device=x.device)
-                return K.gemm_skinny(x.scaled, self.weight, out, sumsq=x.sumsq, norm_width=x.width, eps=x.eps)
+                return K.gemm_skinny(x.scaled, self.tiled, out, sumsq=x.sumsq, norm_width=x.width, eps=x.eps)
             x = x.materialize()
         w = self.weight
         rows = x.shape[0]
@@ -79,4 +85,4 @@ class Linear:
         if x.dtype != torch.bfloat16:
             raise K.KernelError("Linear: a bfloat16 weight needs bfloat16 activations")
         from ..ops import gemm_bf16
-        return gemm_bf16.linear_bf16(x, w, out)
+        return gemm_bf16.linear_bf16(x, w, out, self.tiled)

@@ -39,7 +39,7 @@ class SwiGLU(FeedForward):
         g, u = tensors[p + "gate_proj.weight"], tensors[p + "up_proj.weight"]
         if g.dtype != u.dtype:
             raise ValueError(f"{p}: gate and up projection weights are stored in different dtypes")
-        self.gate_up = Linear(torch.cat([g, u], dim=0))
+        self.gate_up = Linear(torch.cat([g, u], dim=0), halves=2)
         self.down = Linear(tensors[p + "down_proj.weight"])
 
     fuses_tail = True
@@ -49,7 +49,7 @@ class SwiGLU(FeedForward):
         stream and prepares the next norm when the shapes allow (NormedRows are returned)."""
         rows = x.shape[0]
         act = torch.empty((rows, self.intermediate_size), dtype=x.dtype, device=x.device)
-        w = self.gate_up.weight
+        w = self.gate_up.tiled
         if self.gate_up.fusable(x):
             # activation fused into the product; an unfinished input norm is finished there too
             if isinstance(x, NormedRows):

@@ -20,14 +20,14 @@ def test_skinny_product_bf16_and_fp32_outputs(m, n, k, gpu):
     want = x.double() @ w.double().t()
     for dt, tol in ((torch.float32, 1e-5), (torch.bfloat16, 6e-3)):
         out = torch.full((m, n), float("nan"), dtype=dt, device=gpu)
-        K.gemm_skinny(x.to(gpu), w.to(gpu), out)
+        K.gemm_skinny(x.to(gpu), K.TiledWeight(w.to(gpu)), out)
         err = (out.double().cpu() - want).abs().max() / want.abs().max()
         assert err <= tol, f"{dt}: {err:.3g}"
     # a token's result does not depend on the batch it is in (bitwise)
     one = torch.empty((1, n), dtype=torch.float32, device=gpu)
     full = torch.empty((m, n), dtype=torch.float32, device=gpu)
-    K.gemm_skinny(x.to(gpu), w.to(gpu), full)
-    K.gemm_skinny(x[m - 1:].contiguous().to(gpu), w.to(gpu), one)
+    K.gemm_skinny(x.to(gpu), K.TiledWeight(w.to(gpu)), full)
+    K.gemm_skinny(x[m - 1:].contiguous().to(gpu), K.TiledWeight(w.to(gpu)), one)
     assert torch.equal(one[0], full[m - 1])
 
 
@@ -39,7 +39,7 @@ def test_skinny_product_with_swiglu_epilogue(m, inter, k, gpu):
     u = x.double() @ w[inter:].double().t()
     want = g * (1 / (1 + torch.exp(-g))) * u
     out = torch.full((m, inter), float("nan"), dtype=torch.bfloat16, device=gpu)
-    K.gemm_skinny(x.to(gpu), w.to(gpu), out, swiglu=True)
+    K.gemm_skinny(x.to(gpu), K.TiledWeight(w.to(gpu), halves=2), out, swiglu=True)
     err = (out.double().cpu() - want).abs().max() / want.abs().max()
     assert err <= 6e-3, f"{err:.3g}"
 
@@ -48,7 +48,11 @@ def test_skinny_product_refuses_what_it_cannot_do(gpu):
     assert not K.gemm_skinny_supported(65, 16, 32) and not K.gemm_skinny_supported(4, 16, 40)
     x, w = rnd(4, 40).to(gpu), rnd(16, 40).to(gpu)
     with pytest.raises(K.KernelError):
+        K.TiledWeight(w)                                   # K is not a multiple of 32
+    with pytest.raises(K.KernelError):
         K.gemm_skinny(x, w, torch.empty((4, 16), dtype=torch.bfloat16, device=gpu))
+    tw = K.TiledWeight(rnd(50, 64).to(gpu))                # 50 rows are padded to 64
+    assert tw.data.shape == (4, 2, 16, 32) and tw.data[3, :, 2:].abs().max() == 0
 
 
 def rms(h, w, eps):
@@ -70,7 +74,7 @@ def test_product_adds_into_the_stream_and_prepares_the_next_norm(m, n, k, gpu):
         parts = K.gemm_skinny_sumsq_parts(n)
         assert parts == (n + 15) // 16
         sumsq = torch.full((m, parts), float("nan"), device=gpu)
-        K.gemm_skinny(x.to(gpu), w.to(gpu), None, hidden=hidden, next_weight=wn.to(gpu), scaled_out=scaled,
+        K.gemm_skinny(x.to(gpu), K.TiledWeight(w.to(gpu)), None, hidden=hidden, next_weight=wn.to(gpu), scaled_out=scaled,
                       sumsq_out=sumsq)
         want_h = (h0.float() + (x.double() @ w.double().t()).float()).to(torch.bfloat16)
         diff = (hidden.cpu().float() - want_h.float()).abs().max() / want_h.float().abs().max()
@@ -91,11 +95,11 @@ def test_product_adds_into_the_stream_and_prepares_the_next_norm(m, n, k, gpu):
         if n % 32 == 0:
             w2 = rnd(80, n, scale=0.05, seed=4)
             out = torch.empty((m, 80), dtype=torch.float32, device=gpu)
-            K.gemm_skinny(scaled, w2.to(gpu), out, sumsq=sumsq, norm_width=n, eps=eps)
+            K.gemm_skinny(scaled, K.TiledWeight(w2.to(gpu)), out, sumsq=sumsq, norm_width=n, eps=eps)
             want = want_norm.double() @ w2.double().t()
             assert (out.cpu().double() - want).abs().max() <= 6e-3 * want.abs().max()
             act = torch.empty((m, 40), dtype=torch.bfloat16, device=gpu)
-            K.gemm_skinny(scaled, w2.to(gpu), act, swiglu=True, sumsq=sumsq, norm_width=n, eps=eps)
+            K.gemm_skinny(scaled, K.TiledWeight(w2.to(gpu), halves=2), act, swiglu=True, sumsq=sumsq, norm_width=n, eps=eps)
             g, u = want[:, :40], want[:, 40:]
             want_act = g * (1 / (1 + torch.exp(-g))) * u
             assert (act.cpu().double() - want_act).abs().max() <= 1e-2 * want_act.abs().max()
@@ -106,6 +110,6 @@ def test_wide_matrices_give_a_wave_several_tiles(gpu):
     for n in (32768 + 48, 65536 + 16, 128256):
         x, w = rnd(5, 64), rnd(n, 64, scale=0.1, seed=n)
         out = torch.full((5, n), float("nan"), dtype=torch.float32, device=gpu)
-        K.gemm_skinny(x.to(gpu), w.to(gpu), out)
+        K.gemm_skinny(x.to(gpu), K.TiledWeight(w.to(gpu)), out)
         want = x.double() @ w.double().t()
         assert (out.cpu().double() - want).abs().max() <= 1e-5 * want.abs().max()
