@@ -32,6 +32,13 @@
 //               (reference residualKernel, base/src/kernels.cu:38-43), and the sum is prepared for
 //               the next norm: scaled = round(hidden * w_next) and one partial sum of squares per
 //               (token, n-tile).
+//   EPI_ROPE    W is the joined [q; k; v] projection.  A wave owns two tiles of one head: for a
+//               Q or K head the tiles with features f and f + d/2 (the rotate-half pair,
+//               reference ropePackedKernel, base/src/kernels.cu:289-319), for a V head two
+//               neighbouring tiles.  The product is rounded to bf16 as a separate GEMM would
+//               leave it, rotated by the token's position with the fp32 cos/sin tables, and goes
+//               to its place: Q to a [M, nq*d] buffer, K and V to the token's slot of the paged
+//               cache (reference scatterKVPackedKernel, paged_attention/src/kernels.cu:335-363).
 #include "common.h"
 #include <math.h>
 
@@ -43,7 +50,7 @@ union GFrag8 {
     uint4 u4;
 };
 
-enum { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_RESID = 2 };
+enum { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_RESID = 2, EPI_ROPE = 3 };
 
 struct SkinnyArgs {
     const bf16_t *X;
@@ -61,6 +68,12 @@ struct SkinnyArgs {
     int next_w_f32;
     bf16_t *scaled_out;      // [M, N]
     float *sumsq_out;        // [M, n_tiles]
+    // EPI_ROPE (Y is the Q output [M, nq * head_dim] with row stride ldy)
+    const float *cos_t, *sin_t;   // [positions, head_dim / 2], both null: no rotation
+    const int *positions;         // [M]
+    const int *slots;             // [M] cache slot per token (negative: no write), null: no cache write
+    bf16_t *k_cache, *v_cache;    // [pages, nkv, page, d] and [pages, nkv, d, page]
+    int nq, nkv, head_dim, page_size;
 };
 
 template <int MT, int NTW, int EPI>
@@ -76,9 +89,18 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
     const int rows = EPI == EPI_SWIGLU ? a.inter : a.N;        // output columns
     const int n_tiles = (rows + 15) / 16;
     // EPI_SWIGLU: a wave's two tiles are the gate tile and the up tile of the same columns
-    const int out_tiles = EPI == EPI_SWIGLU ? 1 : NTW;
+    const int out_tiles = (EPI == EPI_SWIGLU || EPI == EPI_ROPE) ? 1 : NTW;
     const int tile0 = group * out_tiles;
-    const bool group_ok = tile0 < n_tiles;
+    // EPI_ROPE: group = (head, j) with j in [0, d/32); N is a multiple of 32
+    const bool group_ok = EPI == EPI_ROPE ? group < n_tiles / 2 : tile0 < n_tiles;
+    int rope_head = 0, rope_j = 0;
+    bool rope_rotated = false;
+    if (EPI == EPI_ROPE) {
+        const int hp = a.head_dim / 32;
+        rope_head = group / hp;
+        rope_j = group - rope_head * hp;
+        rope_rotated = rope_head < a.nq + a.nkv;
+    }
     const int K = a.K;
     const int kper = K / k_waves;
     const int kbeg = kpart * kper, kend = kbeg + kper;
@@ -90,6 +112,10 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
         int tile = EPI == EPI_SWIGLU ? tile0 + t * n_tiles : tile0 + t;
+        if (EPI == EPI_ROPE) {
+            const int first = rope_head * (a.head_dim / 16);
+            tile = rope_rotated ? first + rope_j + t * (a.head_dim / 32) : first + 2 * rope_j + t;
+        }
         const int last = (EPI == EPI_SWIGLU ? 2 * n_tiles : n_tiles) - 1;
         if (tile > last) tile = last;
         wp[t] = a.W + (size_t)tile * (size_t)(K / 32) * 512 + (4 * r + g) * 8;
@@ -137,8 +163,59 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
         }
     }
 
+    // Operands of the epilogue that do not depend on the product are loaded here as well (the
+    // token's position, its cache slot and its cos/sin entries; the residual stream and the next
+    // norm's weight), so that no memory latency is left after the main loop.
+    int pre_slot[MT];
+    float4 pre_cos[MT], pre_sin[MT];
+    uint2 pre_hidden[MT];
+    float pre_wn[4] = {1.f, 1.f, 1.f, 1.f};
+    constexpr bool kPreRope = EPI == EPI_ROPE && MT <= 2;
+    constexpr bool kPreResid = EPI == EPI_RESID && NTW == 1 && MT <= 2;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        pre_slot[mt] = -1;
+        pre_cos[mt] = make_float4(1.f, 1.f, 1.f, 1.f);
+        pre_sin[mt] = make_float4(0.f, 0.f, 0.f, 0.f);
+        pre_hidden[mt] = make_uint2(0u, 0u);
+    }
+    if (kPreRope && kpart == 0 && group_ok) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 16 + r;
+            if (m >= a.M) continue;
+            if (a.slots != nullptr && rope_head >= a.nq) pre_slot[mt] = a.slots[m];
+            if (rope_rotated && a.cos_t != nullptr) {
+                const size_t at = (size_t)a.positions[m] * (a.head_dim / 2) + rope_j * 16 + 4 * g;
+                pre_cos[mt] = *reinterpret_cast<const float4 *>(a.cos_t + at);
+                pre_sin[mt] = *reinterpret_cast<const float4 *>(a.sin_t + at);
+            }
+        }
+    }
+    const bool resid_vec = kPreResid && (a.N % 4 == 0) && tile0 * 16 + 4 * g + 3 < rows;
+    if (kPreResid && kpart == 0 && group_ok && resid_vec) {
+        const int n = tile0 * 16 + 4 * g;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 16 + r;
+            if (m < a.M) pre_hidden[mt] = *reinterpret_cast<const uint2 *>(a.hidden + (size_t)m * a.N + n);
+        }
+        if (a.next_w != nullptr) {
+            if (a.next_w_f32) {
+                const float4 wv = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(a.next_w) + n);
+                pre_wn[0] = wv.x; pre_wn[1] = wv.y; pre_wn[2] = wv.z; pre_wn[3] = wv.w;
+            } else {
+                const uint2 wv = *reinterpret_cast<const uint2 *>(reinterpret_cast<const bf16_t *>(a.next_w) + n);
+                pre_wn[0] = bf16_bits_to_float((uint16_t)(wv.x & 0xffffu));
+                pre_wn[1] = bf16_bits_to_float((uint16_t)(wv.x >> 16));
+                pre_wn[2] = bf16_bits_to_float((uint16_t)(wv.y & 0xffffu));
+                pre_wn[3] = bf16_bits_to_float((uint16_t)(wv.y >> 16));
+            }
+        }
+    }
+
     if (group_ok) {
-#pragma unroll 8
+#pragma unroll (NTW == 1 ? 16 : 8)
         for (int k = kbeg; k < kend; k += 32) {
             GFrag8 w[NTW];
 #pragma unroll
@@ -195,6 +272,70 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
         }
     }
 
+    if (EPI == EPI_ROPE) {
+        const int D = a.head_dim;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 16 + r;
+            if (m >= a.M) continue;
+            float va[4], vb[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                va[i] = bf16_bits_to_float(float_to_bf16_bits(acc[0][mt][i] * rinv[mt]));
+                vb[i] = bf16_bits_to_float(float_to_bf16_bits(acc[NTW - 1][mt][i] * rinv[mt]));
+            }
+            int slot = -1;
+            if (kPreRope) slot = pre_slot[mt];
+            else if (a.slots != nullptr && rope_head >= a.nq) slot = a.slots[m];
+            const int page = slot >= 0 ? slot / a.page_size : 0;
+            const int off = slot >= 0 ? slot - page * a.page_size : 0;
+            if (rope_rotated) {
+                const int f = rope_j * 16 + 4 * g;             // feature in [0, d/2); partner f + d/2
+                float o1[4], o2[4];
+                if (a.cos_t != nullptr) {
+                    float4 c4 = pre_cos[mt], s4 = pre_sin[mt];
+                    if (!kPreRope) {
+                        const int pos = a.positions[m];
+                        c4 = *reinterpret_cast<const float4 *>(a.cos_t + (size_t)pos * (D / 2) + f);
+                        s4 = *reinterpret_cast<const float4 *>(a.sin_t + (size_t)pos * (D / 2) + f);
+                    }
+                    const float c[4] = {c4.x, c4.y, c4.z, c4.w}, s[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        o1[i] = va[i] * c[i] - vb[i] * s[i];
+                        o2[i] = va[i] * s[i] + vb[i] * c[i];
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { o1[i] = va[i]; o2[i] = vb[i]; }
+                }
+                bf16_t *dst;
+                if (rope_head < a.nq) {
+                    dst = reinterpret_cast<bf16_t *>(a.Y) + (size_t)m * a.ldy + (size_t)rope_head * D + f;
+                } else {
+                    if (slot < 0) continue;
+                    dst = a.k_cache + (((size_t)page * a.nkv + (rope_head - a.nq)) * a.page_size + off) * D + f;
+                }
+                *reinterpret_cast<uint2 *>(dst) =
+                    make_uint2((uint32_t)float_to_bf16_bits(o1[0]) | ((uint32_t)float_to_bf16_bits(o1[1]) << 16),
+                               (uint32_t)float_to_bf16_bits(o1[2]) | ((uint32_t)float_to_bf16_bits(o1[3]) << 16));
+                *reinterpret_cast<uint2 *>(dst + D / 2) =
+                    make_uint2((uint32_t)float_to_bf16_bits(o2[0]) | ((uint32_t)float_to_bf16_bits(o2[1]) << 16),
+                               (uint32_t)float_to_bf16_bits(o2[2]) | ((uint32_t)float_to_bf16_bits(o2[3]) << 16));
+            } else {
+                if (slot < 0) continue;
+                const int f = rope_j * 32 + 4 * g;             // value features f..f+3 and f+16..f+19
+                bf16_t *dst = a.v_cache + (((size_t)page * a.nkv + (rope_head - a.nq - a.nkv)) * D + f) * a.page_size + off;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    dst[(size_t)i * a.page_size].bits = float_to_bf16_bits(va[i]);
+                    dst[(size_t)(16 + i) * a.page_size].bits = float_to_bf16_bits(vb[i]);
+                }
+            }
+        }
+        return;
+    }
+
 #pragma unroll
     for (int t = 0; t < out_tiles; ++t) {
         const int tile = tile0 + t;
@@ -220,13 +361,13 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
                     bf16_t *hp = a.hidden + (size_t)m * a.N + n;
                     bf16_t *sp = a.scaled_out + (size_t)m * a.N + n;
                     if (n + 3 < rows && (a.N % 4 == 0)) {
-                        const uint2 hv = *reinterpret_cast<const uint2 *>(hp);
+                        const uint2 hv = kPreResid ? pre_hidden[mt] : *reinterpret_cast<const uint2 *>(hp);
                         const float h0[4] = {bf16_bits_to_float((uint16_t)(hv.x & 0xffffu)),
                                              bf16_bits_to_float((uint16_t)(hv.x >> 16)),
                                              bf16_bits_to_float((uint16_t)(hv.y & 0xffffu)),
                                              bf16_bits_to_float((uint16_t)(hv.y >> 16))};
-                        float wn[4] = {1.f, 1.f, 1.f, 1.f};
-                        if (a.next_w != nullptr) {
+                        float wn[4] = {pre_wn[0], pre_wn[1], pre_wn[2], pre_wn[3]};
+                        if (!kPreResid && a.next_w != nullptr) {
                             if (a.next_w_f32) {
                                 const float4 wv = *reinterpret_cast<const float4 *>(
                                     reinterpret_cast<const float *>(a.next_w) + n);
@@ -298,11 +439,20 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
 }
 
 // k_waves: how many wavefronts share one tile group's K range.  Depends on N and K only, never
-// on M, so a token's result does not depend on the batch it is in.
-static int choose_k_waves(int groups, int K) {
+// on M, so a token's result does not depend on the batch it is in.  These products are bound by
+// memory latency until the waves together keep tens of megabytes in flight, so K is cut as deep
+// as a workgroup allows (16 waves) while a wave keeps at least 4 steps of 32, the chip is not
+// oversubscribed (4096 waves) and the waves do not already cover the bandwidth-delay product.
+static int choose_k_waves(int groups, int K, int ntw) {
     int kw = 1;
-    // up to about 2048 waves, each with at least 8 steps of 32 along K
-    while (kw < 16 && groups * kw * 2 <= 2048 && K % (32 * kw * 2) == 0 && K / (kw * 2) >= 256) kw *= 2;
+    while (kw < 16) {
+        const int next = kw * 2;
+        if (K % (32 * next) != 0 || K / next < 128) break;
+        if ((long)groups * next > 4096) break;
+        const long in_flight = (long)groups * kw * ntw * 8192;     // 8 steps of 1 KiB per tile and wave
+        if (in_flight >= (48L << 20)) break;
+        kw = next;
+    }
     return kw;
 }
 
@@ -342,7 +492,7 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
                 "gemm_skinny: row scaling needs a part count and the norm's width");
     KVA_REQUIRE(mode != 3 || (hidden && scaled_out && sumsq_out),
                 "gemm_skinny: the residual epilogue needs hidden, scaled_out and sumsq_out");
-    SkinnyArgs a;
+    SkinnyArgs a = {};
     a.X = (const bf16_t *)X; a.W = (const bf16_t *)W; a.Y = Y;
     a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldy = ldy;
     a.inter = mode == 2 ? N / 2 : 0;
@@ -361,7 +511,7 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
     else if (n_tiles >= 2048) ntw = 2;
     const int out_tiles = mode == 2 ? 1 : ntw;
     const int groups = (n_tiles + out_tiles - 1) / out_tiles;
-    int kw = choose_k_waves(groups, K);
+    int kw = choose_k_waves(groups, K, ntw);
     a.k_waves = kw;
     const int groups_per_wg = kw >= 4 ? 1 : 4 / kw;
     const int waves = kw * groups_per_wg;
@@ -374,5 +524,50 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
     else if (ntw == 2) launch_mt<2, EPI_PLAIN>(a, grid, block, lds, stream);
     else launch_mt<1, EPI_PLAIN>(a, grid, block, lds, stream);
     KVA_CHECK_LAUNCH("gemm_skinny");
+    return KVA_OK;
+}
+
+// The joined Q/K/V projection with rotary encoding and the cache write in its epilogue.
+// W: tiled copy of the [(nq + 2 nkv) * d, K] weight; q_out bf16 [M, nq * d] (row stride ldq).
+// cos/sin [positions, d / 2] fp32 or both null (no rotation); slots null: nothing is cached.
+// head_dim must be a multiple of 32 (a wave takes the tile pair f, f + d/2).
+extern "C" int kva_gemm_skinny_qkv_rope_supported(int M, int K, int head_dim) {
+    return (M >= 1 && M <= 64 && K >= 32 && K % 32 == 0 && head_dim >= 32 && head_dim % 32 == 0) ? 1 : 0;
+}
+
+extern "C" int kva_gemm_skinny_qkv_rope(void *q_out, int ldq, const void *X, const void *W, int M, int K,
+                                        int ldx, int nq, int nkv, int head_dim, const float *sumsq,
+                                        int sumsq_parts, int norm_width, float eps, const float *cos_t,
+                                        const float *sin_t, const int *positions, const int *slots,
+                                        void *k_cache, void *v_cache, int page_size, hipStream_t stream) {
+    KVA_REQUIRE(nq >= 1 && nkv >= 1, "gemm_skinny_qkv_rope: bad head counts %d, %d", nq, nkv);
+    KVA_REQUIRE(kva_gemm_skinny_qkv_rope_supported(M, K, head_dim),
+                "gemm_skinny_qkv_rope: M=%d K=%d head_dim=%d not supported (1 <= M <= 64, K and "
+                "head_dim multiples of 32)", M, K, head_dim);
+    KVA_REQUIRE(ldx >= K && ldx % 8 == 0, "gemm_skinny_qkv_rope: X row stride %d must be a multiple of 8 and >= K", ldx);
+    KVA_REQUIRE(ldq >= nq * head_dim && ldq % 4 == 0, "gemm_skinny_qkv_rope: Q row stride %d does not fit", ldq);
+    KVA_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "gemm_skinny_qkv_rope: one table missing");
+    KVA_REQUIRE(cos_t == nullptr || positions != nullptr, "gemm_skinny_qkv_rope: rotation needs positions");
+    KVA_REQUIRE(slots == nullptr || (k_cache && v_cache && page_size > 0),
+                "gemm_skinny_qkv_rope: cache write asked for without cache or page size");
+    KVA_REQUIRE(sumsq == nullptr || (sumsq_parts >= 1 && norm_width >= 1),
+                "gemm_skinny_qkv_rope: row scaling needs a part count and the norm's width");
+    SkinnyArgs a = {};
+    a.X = (const bf16_t *)X; a.W = (const bf16_t *)W; a.Y = q_out;
+    a.M = M; a.N = (nq + 2 * nkv) * head_dim; a.K = K; a.ldx = ldx; a.ldy = ldq;
+    a.sumsq = sumsq; a.sumsq_parts = sumsq_parts; a.norm_width = norm_width; a.eps = eps;
+    a.cos_t = cos_t; a.sin_t = sin_t; a.positions = positions; a.slots = slots;
+    a.k_cache = (bf16_t *)k_cache; a.v_cache = (bf16_t *)v_cache;
+    a.nq = nq; a.nkv = nkv; a.head_dim = head_dim; a.page_size = page_size;
+    const int groups = a.N / 32;
+    const int kw = choose_k_waves(groups, K, 2);
+    a.k_waves = kw;
+    const int groups_per_wg = kw >= 4 ? 1 : 4 / kw;
+    const int waves = kw * groups_per_wg;
+    const size_t lds = kw > 1 ? (size_t)waves * 2 * 64 * 4 * sizeof(float) : 0;
+    KVA_REQUIRE(lds <= 64 * 1024, "gemm_skinny_qkv_rope: reduction buffer of %zu bytes does not fit", lds);
+    dim3 grid((groups + groups_per_wg - 1) / groups_per_wg), block(64 * waves);
+    launch_mt<2, EPI_ROPE>(a, grid, block, lds, stream);
+    KVA_CHECK_LAUNCH("gemm_skinny_qkv_rope");
     return KVA_OK;
 }

@@ -356,6 +356,53 @@ def gemm_skinny(x: torch.Tensor, w: TiledWeight, out: Optional[torch.Tensor], sw
     return out
 
 
+def gemm_skinny_qkv_rope_supported(m: int, k: int, head_dim: int) -> bool:
+    return bool(hip_lib().kva_gemm_skinny_qkv_rope_supported(int(m), int(k), int(head_dim)))
+
+
+def gemm_skinny_qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, num_q_heads: int,
+                         num_kv_heads: int, head_dim: int, positions: torch.Tensor,
+                         cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+                         k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                         slot_mapping: Optional[torch.Tensor], page_size: int, *,
+                         sumsq: Optional[torch.Tensor] = None, norm_width: int = 0, eps: float = 0.0):
+    """The joined Q/K/V projection of at most 64 rows with rotation and cache write in its
+    epilogue: ``q_out`` [M, nq*d] takes the rotated Q heads, the cache takes rotated K and plain V
+    at ``slot_mapping`` (``k_cache`` None: nothing is cached).  ``cos``/``sin`` are the full
+    tables [positions, d/2], or both None for no rotation.  ``sumsq`` as in :func:`gemm_skinny`."""
+    if not isinstance(w, TiledWeight) or w.halves != 1:
+        raise KernelError("gemm_skinny_qkv_rope: the weight must be a plain TiledWeight")
+    m, k = x.shape
+    if x.dtype != torch.bfloat16 or k != w.k or w.n != (num_q_heads + 2 * num_kv_heads) * head_dim:
+        raise KernelError(f"gemm_skinny_qkv_rope: bf16 x {tuple(x.shape)} does not fit weight [{w.n}, {w.k}] "
+                          f"for {num_q_heads}+2*{num_kv_heads} heads of {head_dim}")
+    if q_out.shape != (m, num_q_heads * head_dim) or q_out.dtype != torch.bfloat16:
+        raise KernelError("gemm_skinny_qkv_rope: q_out must be bf16 [M, nq * d]")
+    if positions.shape != (m,):
+        raise KernelError("gemm_skinny_qkv_rope: one position per row")
+    if (cos is None) != (sin is None) or (cos is not None and (
+            cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] * 2 != head_dim)):
+        raise KernelError("gemm_skinny_qkv_rope: cos and sin tables must both be [positions, d/2]")
+    if sumsq is not None and (sumsq.dim() != 2 or sumsq.shape[0] != m or norm_width <= 0):
+        raise KernelError("gemm_skinny_qkv_rope: sumsq must be [M, parts] and norm_width positive")
+    write = k_cache is not None
+    if write:
+        if v_cache is None or slot_mapping is None or slot_mapping.shape != (m,):
+            raise KernelError("gemm_skinny_qkv_rope: K and V cache and one slot per row are all needed")
+        check_cache_shapes("gemm_skinny_qkv_rope", k_cache, v_cache, num_kv_heads, head_dim)
+        if k_cache.shape[2] != page_size or k_cache.dtype != torch.bfloat16:
+            raise KernelError("gemm_skinny_qkv_rope: cache page size or dtype does not fit")
+    check(hip_lib().kva_gemm_skinny_qkv_rope(
+        _dev(q_out, "q_out"), q_out.shape[1], _dev(x, "x"), _dev(w.data, "w"), m, k, k, num_q_heads,
+        num_kv_heads, head_dim, _opt(sumsq, "sumsq", torch.float32), sumsq.shape[1] if sumsq is not None else 0,
+        int(norm_width), float(eps), _opt(cos, "cos", torch.float32), _opt(sin, "sin", torch.float32),
+        _dev(positions, "positions", torch.int32),
+        _dev(slot_mapping, "slot_mapping", torch.int32) if write else None,
+        _opt(k_cache, "k_cache") if write else None, _opt(v_cache, "v_cache") if write else None,
+        int(page_size), _stream()), "gemm_skinny_qkv_rope")
+    return q_out
+
+
 def gemm_skinny_sumsq_parts(n: int) -> int:
     return int(hip_lib().kva_gemm_skinny_sumsq_parts(int(n)))
 

@@ -17,7 +17,8 @@ import torch
 from ..config.registry import MIXERS, POSITION_ENCODINGS
 from ..models.spec import PartSpec, TensorSpec
 from ..ops import attention as attn_ops
-from .base import BranchTail, KVCacheSpec, Mixer, MixerContext
+from ..ops import kernels as K
+from .base import BranchTail, KVCacheSpec, Mixer, MixerContext, NormedRows
 from .linear import Linear
 
 
@@ -59,14 +60,37 @@ class GQAAttention(Mixer):
 
     fuses_tail = True
 
+    def _project_encode_cache(self, x, batch, kv):
+        """Q (position-encoded) for the attention kernel, with K and V of the step's tokens put
+        into the cache.  Few rows: one product does all of it in its epilogue; otherwise the
+        product is followed by the position encoding's own kernel.  Returns a tensor whose first
+        ``nq * d`` columns are the queries."""
+        tables = None
+        if self.qkv.fusable(x) and K.gemm_skinny_qkv_rope_supported(x.shape[0], self.hidden_size, self.head_dim):
+            tables = self.position.rotate_half_tables(x.device, self.head_dim)
+        if tables is None:
+            qkv = self.qkv(x)
+            self.position.apply_and_cache(qkv, batch.positions, self.num_heads, self.num_kv_heads,
+                                          self.head_dim, kv)
+            return qkv
+        write = kv is not None and kv.writes
+        q = torch.empty((x.shape[0], self.num_heads * self.head_dim), dtype=torch.bfloat16, device=x.device)
+        norm = {}
+        if isinstance(x, NormedRows):
+            norm = dict(sumsq=x.sumsq, norm_width=x.width, eps=x.eps)
+            x = x.scaled
+        K.gemm_skinny_qkv_rope(x, self.qkv.tiled, q, self.num_heads, self.num_kv_heads, self.head_dim,
+                               batch.positions, tables[0], tables[1],
+                               kv.k_cache if write else None, kv.v_cache if write else None,
+                               kv.slot_mapping if write else None, kv.page_size if kv is not None else 0, **norm)
+        return q
+
     def forward(self, x, ctx: MixerContext, tail: Optional[BranchTail] = None):
         """``x`` may be NormedRows (the input norm is then finished inside the QKV product); with
         a ``tail`` the output projection adds into the residual stream and prepares the next
         norm when the shapes allow, and NormedRows are returned instead of the plain output."""
         batch, kv = ctx.batch, ctx.kv
-        qkv = self.qkv(x)
-        self.position.apply_and_cache(qkv, batch.positions, self.num_heads, self.num_kv_heads,
-                                      self.head_dim, kv)
+        qkv = self._project_encode_cache(x, batch, kv)
         out = torch.empty((x.shape[0], self.num_heads * self.head_dim), dtype=x.dtype, device=x.device)
         attn_ops.paged_attention(qkv, out, kv, batch, self.num_heads, self.num_kv_heads,
                                  self.head_dim, self.scale, self.window)

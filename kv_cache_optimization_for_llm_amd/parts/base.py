@@ -159,6 +159,14 @@ class PositionEncoding(Part):
         writing, stores the encoded K and the plain V at the tokens' cache slots."""
         raise NotImplementedError
 
+    def rotate_half_tables(self, device, head_dim: int):
+        """For encodings that a projection's epilogue can apply: ``(cos, sin)`` fp32 tables
+        ``[positions, head_dim / 2]`` of a rotate-half rotation over the whole head
+        (``out[j] = x[j] cos - x[j + d/2] sin``, ``out[j + d/2] = x[j] sin + x[j + d/2] cos``), or
+        ``(None, None)`` if Q and K pass unchanged.  ``None`` (the default): the encoding is
+        something else and only ``apply_and_cache`` applies it."""
+        return None
+
 
 class Mixer(Part):
     fuses_tail = False      # True: forward(x, ctx, tail=None) accepts NormedRows and a BranchTail

@@ -73,6 +73,11 @@ class RotaryEncoding(PositionEncoding):
             self._sin = torch.from_numpy(np.sin(angle).astype(np.float32)).to(device)
         return self._cos, self._sin
 
+    def rotate_half_tables(self, device, head_dim: int):
+        if self.rotary_dim != head_dim:
+            return None
+        return self.tables(device)
+
     def apply_and_cache(self, qkv, positions, num_q_heads, num_kv_heads, head_dim, kv: Optional[KVView]):
         cos, sin = self.tables(qkv.device)
         write = kv is not None and kv.writes
@@ -89,6 +94,9 @@ class NoPositionEncoding(PositionEncoding):
 
     def __init__(self, **_ignored):
         super().__init__("")
+
+    def rotate_half_tables(self, device, head_dim: int):
+        return (None, None)
 
     def apply_and_cache(self, qkv, positions, num_q_heads, num_kv_heads, head_dim, kv: Optional[KVView]):
         write = kv is not None and kv.writes

@@ -113,3 +113,79 @@ def test_wide_matrices_give_a_wave_several_tiles(gpu):
         K.gemm_skinny(x.to(gpu), K.TiledWeight(w.to(gpu)), out)
         want = x.double() @ w.double().t()
         assert (out.cpu().double() - want).abs().max() <= 1e-5 * want.abs().max()
+
+
+@pytest.mark.parametrize("m", [1, 7, 16, 35])
+@pytest.mark.parametrize("nq, nkv, d, page, k", [(4, 2, 32, 16, 64), (6, 1, 96, 8, 160), (3, 3, 64, 4, 2048),
+                                                 (32, 8, 64, 16, 2048)])
+@pytest.mark.parametrize("rotate, normed", [(True, False), (True, True), (False, False)])
+def test_qkv_product_rotates_and_writes_the_cache(m, nq, nkv, d, page, k, rotate, normed, gpu):
+    """The fused projection equals product -> round -> rotate-half rotation -> cache write done
+    one after the other in fp32 (the cache is checked slot by slot, untouched slots stay zero)."""
+    import plain_llama as plain
+    n = (nq + 2 * nkv) * d
+    x, w = rnd(m, k), rnd(n, k, scale=0.05, seed=1)
+    pos = [(37 * i + 3) % 300 for i in range(m)]
+    pages = (m + page - 1) // page + 3
+    perm = torch.randperm(pages * page, generator=torch.Generator().manual_seed(m))[:m].to(torch.int32)
+    slots = perm.clone()
+    if m > 2:
+        slots[2] = -1
+    inv = plain.rope_inv_freq(d, 20000.0, dict(rope_type="llama3", factor=4.0, low_freq_factor=1.0,
+                                               high_freq_factor=2.0, original_max_position_embeddings=64))
+    cos, sin = plain.rope_cos_sin(range(300), inv)
+    y = x.double() @ w.double().t()
+    extra = {}
+    xin = x
+    if normed:
+        # x is an unfinished norm input: (scaled, partial sums of squares of the stream)
+        parts = 5
+        sumsq = torch.rand(m, parts, generator=torch.Generator().manual_seed(9)) * 40 + 1
+        eps, width = 3e-6, 100
+        y = y * torch.rsqrt(sumsq.double().sum(-1, keepdim=True) / width + eps)
+        extra = dict(sumsq=sumsq.to(gpu), norm_width=width, eps=eps)
+    y = y.float().to(torch.bfloat16).float()                            # what a separate product leaves
+    q_want = y[:, :nq * d].view(m, nq, d).clone()
+    k_want = y[:, nq * d:(nq + nkv) * d].view(m, nkv, d).clone()
+    v_want = y[:, (nq + nkv) * d:].view(m, nkv, d)
+    if rotate:
+        c, s = plain.rope_cos_sin(pos, inv)
+        q_want = plain.apply_rope(q_want, c, s)
+        k_want = plain.apply_rope(k_want, c, s)
+    k_cache = torch.zeros(pages, nkv, page, d, dtype=torch.bfloat16, device=gpu)
+    v_cache = torch.zeros(pages, nkv, d, page, dtype=torch.bfloat16, device=gpu)
+    q = torch.full((m, nq * d), float("nan"), dtype=torch.bfloat16, device=gpu)
+    assert K.gemm_skinny_qkv_rope_supported(m, k, d)
+    K.gemm_skinny_qkv_rope(xin.to(gpu), K.TiledWeight(w.to(gpu)), q, nq, nkv, d,
+                           torch.tensor(pos, dtype=torch.int32, device=gpu),
+                           torch.from_numpy(cos).to(gpu) if rotate else None,
+                           torch.from_numpy(sin).to(gpu) if rotate else None,
+                           k_cache, v_cache, slots.to(gpu), page, **extra)
+    scale = y.abs().max()
+    assert (q.float().cpu().view(m, nq, d) - q_want).abs().max() <= 1e-2 * scale
+    kc, vc = k_cache.float().cpu(), v_cache.float().cpu()
+    for t in range(m):
+        sl = int(slots[t])
+        if sl < 0:
+            continue
+        assert (kc[sl // page, :, sl % page, :] - k_want[t]).abs().max() <= 1e-2 * scale, f"k of row {t}"
+        assert (vc[sl // page, :, :, sl % page] - v_want[t]).abs().max() <= 1e-2 * scale, f"v of row {t}"
+    written = {int(sl) for sl in slots if sl >= 0}
+    for sl in range(pages * page):
+        if sl not in written:
+            assert kc[sl // page, :, sl % page, :].abs().max() == 0 and vc[sl // page, :, :, sl % page].abs().max() == 0
+    # without a cache only Q is produced
+    q2 = torch.empty_like(q)
+    K.gemm_skinny_qkv_rope(xin.to(gpu), K.TiledWeight(w.to(gpu)), q2, nq, nkv, d,
+                           torch.tensor(pos, dtype=torch.int32, device=gpu),
+                           torch.from_numpy(cos).to(gpu) if rotate else None,
+                           torch.from_numpy(sin).to(gpu) if rotate else None, None, None, None, 0, **extra)
+    assert torch.equal(q2, q)
+
+
+def test_qkv_product_refuses_head_sizes_it_cannot_pair(gpu):
+    assert not K.gemm_skinny_qkv_rope_supported(4, 64, 48) and not K.gemm_skinny_qkv_rope_supported(4, 64, 16)
+    w = K.TiledWeight(rnd(4 * 48, 64).to(gpu))
+    with pytest.raises(K.KernelError):
+        K.gemm_skinny_qkv_rope(rnd(4, 64).to(gpu), w, torch.empty((4, 96), dtype=torch.bfloat16, device=gpu), 2, 1, 48,
+                               torch.zeros(4, dtype=torch.int32, device=gpu), None, None, None, None, None, 0)
