@@ -4,8 +4,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 Prints ONE JSON line.  ``value`` is decoded tokens per second of the default run: a batch of 8
-requests, each holding a context of 8,192 tokens, one decode step (model forward over the paged
-cache + greedy sampling + token ids back on the host) per "step".  The same line carries the
+requests whose contexts end at 8,192 tokens, driven by the serving loop; a "step" is one decode
+step (scheduling, model forward over the paged cache, greedy sampling, token ids back on the host).  The same line carries the
 2,048-token prefill, the decode roofline (bytes the step has to read / time / HBM peak) and the
 batch-1 and batch-64 points.
 """
@@ -74,7 +74,7 @@ def main():
     import torch
     from kv_cache_optimization_for_llm_amd.engine.batch import StepEntry
     from kv_cache_optimization_for_llm_amd.engine.engine import Engine, EngineOptions
-    from kv_cache_optimization_for_llm_amd.sampling.sampler import SampleRow, Sampler
+    from kv_cache_optimization_for_llm_amd.engine.runner import Runner, ServeOptions
 
     cfg = dict(CONFIG_1B)
     full_layers = cfg["num_hidden_layers"]
@@ -88,41 +88,48 @@ def main():
                                         max_seqs=max_batch, max_seq_len=cfg["max_position_embeddings"]),
                     config_dict=cfg, random_seed=0)
     dev = engine.device
-    for g in engine.cache.groups:       # random keys and values stand for the context
-        g.k.normal_(0.0, 1.0)
-        g.v.normal_(0.0, 1.0)
-    sampler = Sampler(engine.vocab_size, max_batch, dev)
     gen = torch.Generator().manual_seed(0)
 
     def decode_run(batch, steps, warmup, context):
-        """Times ``steps`` decode steps of ``batch`` requests whose contexts END at ``context``."""
-        ids = [f"d{batch}_{i}" for i in range(batch)]
-        first = context - (steps + warmup)
-        for rid in ids:
-            engine.preload_context(rid, first)
-        toks = [int(t) for t in torch.randint(0, engine.vocab_size, (batch,), generator=gen)]
-        rows = [SampleRow(engine.seat_of(r)) for r in ids]
-
-        def one():
-            nonlocal toks
-            logits = engine.step([StepEntry(r, [t], [0]) for r, t in zip(ids, toks)])
-            toks = [int(t) for t in sampler.sample(logits, rows)]
+        """Times ``steps`` decode steps of ``batch`` requests through the serving loop (scheduler,
+        step function, sampler; a step is launched while the host still waits for the previous
+        step's tokens).  The prompts are prefilled first, in portions; their lengths are set so
+        that the longest context ENDS at ``context``.  Returns (seconds, mean context length
+        over the timed steps)."""
+        budget = 32768
+        runner = Runner(engine, ServeOptions(ignore_eos=True, run_ahead=True, max_batch_tokens=budget))
+        lead = warmup + steps + 2
+        first = context - lead
+        first -= (batch * first + budget - 1) // budget + 1      # steps that other requests' prompts take
+        if first < 1:
+            raise SystemExit(f"context {context} is too short for {steps} + {warmup} steps")
+        for _ in range(batch):
+            prompt = [int(t) for t in torch.randint(0, engine.vocab_size, (first,), generator=gen)]
+            runner.submit(prompt, context - first - 1)
+        sched = runner.scheduler
+        while sched.waiting or any(s.prefilling for s in sched.running):
+            runner.step()
         for _ in range(warmup):
-            one()
+            runner.step()
         torch.cuda.synchronize()
+        assert len(sched.running) == batch and not any(s.prefilling for s in sched.running)
+        ctx0 = sum(s.computed for s in sched.running) / batch
         t0 = time.perf_counter()
         for _ in range(steps):
-            one()
+            runner.step()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        for rid in ids:
-            engine.release(rid)
-        return dt
+        assert len(sched.running) == batch and max(s.computed for s in sched.running) <= context
+        mean_ctx = ctx0 + steps / 2
+        # drop the requests (their remaining budget is not part of the measurement)
+        runner._resolve_in_flight()
+        for s_ in list(sched.running) + list(sched.closing):
+            sched._finish(s_, "length", [])
+        return dt, mean_ctx
 
-    dt = decode_run(args.batch, args.steps, args.warmup, ctx)
+    dt, mean_ctx = decode_run(args.batch, args.steps, args.warmup, ctx)
     ms_per_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
-    mean_ctx = ctx - args.steps / 2
     step_bytes = weight_bytes(cfg) + args.batch * mean_ctx * kv_bytes_per_token(cfg)
     achieved = step_bytes / (ms_per_step * 1e-3) / 1e9
 
@@ -145,18 +152,18 @@ def main():
     if not args.skip_points:
         for b in (1, 64):
             k = max(16, args.steps // 2)
-            d = decode_run(b, k, 8, ctx)
+            d, _ = decode_run(b, k, 8, ctx)
             points[f"decode_b{b}"] = round(b * k / d, 1)
         # the workload BASELINE.json words: 512-token prompts, 256 generated tokens
         for b in (1, 8, 64):
-            d = decode_run(b, 256, 8, 512 + 256 + 8)
-            points[f"decode_b{b}_p512_g256"] = round(b * 256 / d, 1)
+            d, _ = decode_run(b, 240, 8, 512 + 256)
+            points[f"decode_b{b}_p512_g256"] = round(b * 240 / d, 1)
 
     out = {
         "metric": "decode tok/s at batch 8 (context 8192), Llama-3.2-1B shape", "value": round(value, 1),
         "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16", "data": "synthetic: random weights N(0,0.02), seeded uniform token ids, random cache contents for the context",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic: random weights N(0,0.02), seeded uniform token ids (prompts are prefilled, then decoded)",
         "config": {"model": "llama-3.2-1b-shape", "global_batch": args.batch, "seq_len": ctx,
                    "parallelism": "single-gpu", "layers": cfg["num_hidden_layers"], "layers_full": full_layers,
                    "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],

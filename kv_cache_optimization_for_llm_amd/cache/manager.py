@@ -94,6 +94,7 @@ class CacheManager:
         self._seats: List[Optional[_Seat]] = [None] * max_seqs
         self._free_seats = list(range(max_seqs - 1, -1, -1))   # popped from the back: lowest first
         self.peak_held_pages = 0
+        self._flush_event = None     # set while an upload of table spans may still be reading the host table
         if device is not None:
             self._allocate_device()
 
@@ -117,11 +118,24 @@ class CacheManager:
 
     def flush_tables(self) -> None:
         """Brings the device block tables up to date (only the spans that changed)."""
+        queued = False
         for g in self.groups:
             if g.table_dev is not None:
                 for seat, (lo, hi) in g.dirty.items():
                     g.table_dev[seat, lo:hi].copy_(g._table_pinned[seat, lo:hi], non_blocking=True)
+                    queued = True
             g.dirty.clear()
+        if queued:
+            import torch
+            self._flush_event = torch.cuda.Event()
+            self._flush_event.record()
+
+    def _before_table_write(self) -> None:
+        """The uploads read the pinned host table when they execute, not when they are queued: a
+        caller that runs ahead of the device must not change the table under them."""
+        if self._flush_event is not None:
+            self._flush_event.synchronize()
+            self._flush_event = None
 
     def kv_arrays(self, cache_slot: int):
         for g in self.groups:
@@ -167,6 +181,7 @@ class CacheManager:
         reservation of ``reserve_tokens`` tokens cannot be placed."""
         if not self._free_seats:
             return None
+        self._before_table_write()
         ng = len(self.groups)
         st = _Seat(request_id, 0, [0] * ng, [0] * ng, [None] * ng)
         seat = self._free_seats[-1]
@@ -198,6 +213,7 @@ class CacheManager:
     def free(self, seat: int) -> None:
         """Gives back everything the seat holds."""
         s = self.seat(seat)
+        self._before_table_write()
         for g in self.groups:
             gi = g.index
             if self.mode == "paged":
@@ -244,6 +260,8 @@ class CacheManager:
         need = self.pages_needed(seat, new_len)
         if any(n > g.free_pages() for n, g in zip(need, self.groups)):
             return False
+        if any(need):
+            self._before_table_write()
         for n, g in zip(need, self.groups):
             if n == 0:
                 continue
@@ -285,6 +303,7 @@ class CacheManager:
             lo = s.first_block[g.index]
             hi = min(keep_from, s.next_block[g.index])
             if hi > lo:
+                self._before_table_write()
                 pages = [int(p) for p in g.table_host[seat, lo:hi] if p >= 0]
                 g.pool.drop(pages)
                 g.table_host[seat, lo:hi] = -1

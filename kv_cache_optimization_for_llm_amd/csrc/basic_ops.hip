@@ -21,23 +21,30 @@ void kva_set_error(const char *fmt, ...) {
 }
 
 // ---------------------------------------------------------------------------------------
+// A negative id names a token that is still on the device: id = -1 - r stands for feedback[r]
+// (the token a sampling kernel left in row r of its output), so a decode step can be launched
+// before the host has seen the token it continues from.
 template <typename TW, typename TO>
 __global__ void embed_gather_kernel(TO *__restrict__ out, const TW *__restrict__ table,
-                                    const int *__restrict__ ids, int width) {
+                                    const int *__restrict__ ids, const int *__restrict__ feedback,
+                                    int width) {
     const int row = blockIdx.x;
-    const TW *src = table + (size_t)ids[row] * width;
+    int id = ids[row];
+    if (id < 0) id = feedback[-1 - id];
+    const TW *src = table + (size_t)id * width;
     TO *dst = out + (size_t)row * width;
     for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = from_float<TO>(to_float(src[i]));
 }
 
-extern "C" int kva_embed_gather(void *out, const void *table, const int *ids, int rows, int width,
-                                int table_dtype, int out_dtype, hipStream_t stream) {
+// feedback may be null when no id is negative (the caller checks the ids it uploads).
+extern "C" int kva_embed_gather(void *out, const void *table, const int *ids, const int *feedback,
+                                int rows, int width, int table_dtype, int out_dtype, hipStream_t stream) {
     KVA_REQUIRE(rows >= 0 && width > 0, "embed_gather: bad sizes rows=%d width=%d", rows, width);
     if (rows == 0) return KVA_OK;
     dim3 grid(rows), block(256);
 #define LAUNCH(TW, TO)                                                                    \
     hipLaunchKernelGGL((embed_gather_kernel<TW, TO>), grid, block, 0, stream, (TO *)out, \
-                       (const TW *)table, ids, width)
+                       (const TW *)table, ids, feedback, width)
     if (table_dtype == KVA_F32 && out_dtype == KVA_F32) LAUNCH(float, float);
     else if (table_dtype == KVA_BF16 && out_dtype == KVA_BF16) LAUNCH(bf16_t, bf16_t);
     else if (table_dtype == KVA_F32 && out_dtype == KVA_BF16) LAUNCH(float, bf16_t);

@@ -19,8 +19,14 @@ import torch
 @dataclass
 class StepEntry:
     request_id: object
-    tokens: Sequence[int]
+    tokens: Sequence[int]           # a single token may be ``feedback_token(r)``: row r of the
+                                    # engine's feedback buffer, a token still on the device
     want: Sequence[int] = ()        # indices into ``tokens`` whose logits are returned
+
+
+def feedback_token(row: int) -> int:
+    """The id that stands for 'the token in row ``row`` of the engine's feedback buffer'."""
+    return -1 - int(row)
 
 
 @dataclass
@@ -46,6 +52,7 @@ class StepBatch:
     max_q_len: int = 0
     max_context: int = 0
     logits_for_all_rows: bool = False    # logit_rows is exactly 0, 1, ..., T-1
+    feedback: torch.Tensor = None        # device int32: tokens that negative token_ids stand for
     _items: Dict[tuple, tuple] = field(default_factory=dict, repr=False)
 
     def attention_items(self, group: int, row_tiles: int = 1):

@@ -98,10 +98,13 @@ class Engine:
         self.max_seq_len = max_seq_len
         self._seat_of: Dict[object, int] = {}
         self.steps_run = 0
+        # tokens that stay on the device between steps: a sampler leaves its output here and the
+        # next step's single-token entries may name a row of it instead of a token id
+        self.feedback = torch.zeros(max(1, options.max_seqs), dtype=torch.int32, device=self.device)
         self.graphs = None
         if options.use_graphs and self.dtype == torch.bfloat16 and self.model.graph_safe():
             from .graphs import DecodeGraphs
-            self.graphs = DecodeGraphs(self.model, self.cache, self.device)
+            self.graphs = DecodeGraphs(self.model, self.cache, self.device, self.feedback)
 
     # ------------------------------------------------------------------ requests
     def has_request(self, request_id) -> bool:
@@ -176,6 +179,7 @@ class Engine:
                     else logits[:0]
             return logits
         batch = build_batch(seats, starts, toks, wants, slot_maps, self.device)
+        batch.feedback = self.feedback
         return self.model.forward(batch, self.cache)
 
     def _place(self, entries: Sequence[StepEntry]):
@@ -191,7 +195,8 @@ class Engine:
             if len(e.tokens) == 0:
                 raise EngineError(f"request {e.request_id!r}: an entry needs at least one token")
             arr = np.asarray(e.tokens, dtype=np.int64)
-            if arr.min() < 0 or arr.max() >= self.vocab_size:
+            lowest = -self.feedback.shape[0] if len(arr) == 1 else 0     # a lone token may be a feedback row
+            if arr.min() < lowest or arr.max() >= self.vocab_size:
                 raise EngineError(f"request {e.request_id!r}: token id outside [0, {self.vocab_size})")
             for i in e.want:
                 if not 0 <= i < len(arr):

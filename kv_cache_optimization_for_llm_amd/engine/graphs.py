@@ -33,7 +33,7 @@ def context_bucket(max_context: int) -> int:
 class _DecodeSlot:
     """Static buffers, batch view and (once captured) the graph for one (entries, bucket) shape."""
 
-    def __init__(self, n: int, bucket: int, num_groups: int, device):
+    def __init__(self, n: int, bucket: int, num_groups: int, device, feedback=None):
         self.n, self.bucket = n, bucket
         # layout of the int32 staging buffer: token_ids, positions, tok_seat, entry_start_pos,
         # then one slot mapping per cache group; each n long
@@ -48,7 +48,7 @@ class _DecodeSlot:
             token_ids=v(0), positions=v(1), tok_seat=v(2), logit_rows=self.const[n + 1:],
             slot_mapping=[v(4 + g) for g in range(num_groups)],
             entry_seat=v(2), entry_q_start=self.const[:n + 1], entry_start_pos=v(3),
-            max_q_len=1, max_context=bucket, logits_for_all_rows=True)
+            max_q_len=1, max_context=bucket, logits_for_all_rows=True, feedback=feedback)
         # attention work items depend on this array only, so they are the same every step; the
         # eager warm-up run uploads them, the captured run finds them cached
         self.batch.h_entry_q_start = np.arange(n + 1, dtype=np.int32)
@@ -70,8 +70,8 @@ class _DecodeSlot:
 
 
 class DecodeGraphs:
-    def __init__(self, model, cache, device):
-        self.model, self.cache, self.device = model, cache, device
+    def __init__(self, model, cache, device, feedback=None):
+        self.model, self.cache, self.device, self.feedback = model, cache, device, feedback
         self.slots: Dict[Tuple[int, int], _DecodeSlot] = {}
         self.replays = 0
         self.captures = 0
@@ -84,7 +84,7 @@ class DecodeGraphs:
         key = (n, bucket)
         slot = self.slots.get(key)
         if slot is None:
-            slot = self.slots[key] = _DecodeSlot(n, bucket, len(self.cache.groups), self.device)
+            slot = self.slots[key] = _DecodeSlot(n, bucket, len(self.cache.groups), self.device, self.feedback)
         slot.fill(tokens, positions, seats, slot_maps)
         if not slot.warm:
             # first step of this shape runs eagerly: it warms up lazy initialisation (GEMM

@@ -7,7 +7,7 @@ from typing import Dict, Iterable, List, Optional, Sequence
 from ..sampling.sampler import SampleRow, Sampler
 from .batch import StepEntry
 from .engine import Engine, EngineOptions
-from .scheduler import Event, Request, Scheduler, StepPlan
+from .scheduler import Event, Request, Scheduler, StepPlan, UnresolvedTokens
 
 
 @dataclass
@@ -22,6 +22,7 @@ class ServeOptions:
     max_batch_tokens: int = 3072        # MAX_BATCH_TOKENS: a step's token budget
     chunk_size: Optional[int] = None    # most prompt tokens of one request per step
     reserve_policy: str = "max"         # ORCA_POLICY: max | pow2 | oracle (contiguous mode)
+    run_ahead: bool = True              # launch a step before the host has seen the previous step's tokens
 
 
 class Runner:
@@ -39,6 +40,7 @@ class Runner:
         self.scheduler.on_admit = self._on_admit
         self.scheduler.on_release = self._on_release
         self._next_id = 0
+        self._in_flight = None        # (ticket, pending tokens) of the step launched last
 
     # the scheduler owns seats; the engine only needs to know which request sits where
     def _on_admit(self, seq) -> None:
@@ -63,13 +65,10 @@ class Runner:
         return request_id
 
     def idle(self) -> bool:
-        return self.scheduler.idle()
+        return self.scheduler.idle() and self._in_flight is None
 
-    def step(self) -> List[Event]:
-        plan = self.scheduler.plan()
-        events = list(plan.events)
-        if not plan.entries:
-            return events
+    def _launch(self, plan: StepPlan):
+        """Queues the forward pass and the sampling of a planned step; nothing is waited for."""
         entries, rows = [], []
         for e in plan.entries:
             rid = ("sched", e.seq.request.id, e.seq.request.seq_index, e.seq.request.arrival)
@@ -81,8 +80,37 @@ class Runner:
                                       e.start + len(e.tokens), apply_penalty=emitted_before > 0))
         logits = self.engine.step_planned(entries, [e.seq.seat for e in plan.entries],
                                           [e.start for e in plan.entries])
-        sampled = self.sampler.sample(logits, rows)
-        events.extend(self.scheduler.complete(plan, sampled))
+        # the tokens also stay on the device, where the next step's entries can name them
+        return self.sampler.sample_async(logits, rows, out=self.engine.feedback)
+
+    def _resolve_in_flight(self) -> List[Event]:
+        if self._in_flight is None:
+            return []
+        ticket, pending = self._in_flight
+        self._in_flight = None
+        return self.scheduler.resolve(ticket, pending.wait())
+
+    def step(self) -> List[Event]:
+        """Plans and launches one step.  With ``run_ahead`` the events of a step are returned by
+        the call after the one that launched it (the device works on a step while the host
+        prepares the next); without it every call waits for its own tokens."""
+        events: List[Event] = []
+        try:
+            plan = self.scheduler.plan()
+        except UnresolvedTokens:
+            events.extend(self._resolve_in_flight())
+            plan = self.scheduler.plan()
+        launched = None
+        if plan.entries:
+            if len([e for e in plan.entries if e.sample]) > self.engine.feedback.shape[0]:
+                raise RuntimeError("more sampled rows than the engine's feedback buffer holds")
+            pending = self._launch(plan)
+            launched = (self.scheduler.book(plan), pending)
+        events.extend(self._resolve_in_flight())      # the step before the one just launched
+        events.extend(plan.events)
+        self._in_flight = launched
+        if launched is not None and not self.options.run_ahead:
+            events.extend(self._resolve_in_flight())
         return events
 
     def run_until_idle(self) -> Iterable[Event]:

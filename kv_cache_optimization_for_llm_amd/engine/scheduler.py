@@ -23,6 +23,16 @@ admission by policy - ``max`` (the longest sequence), ``pow2`` (prompt + output 
 up to a power of two), ``oracle`` (prompt + output budget) - the queue head blocks until its
 reservation can be placed, nothing is ever preempted, and a request that fills its reservation
 finishes with ``sequence_too_long``.
+
+Running ahead of the device.  Booking a step does not need the values of the tokens it sampled,
+only their number: :meth:`Scheduler.book` advances every request as if no end-of-sequence token
+had come and returns a :class:`Ticket`; the next step can be planned and launched at once, its
+decode entries naming the tokens by their row in the previous sampling (they are still on the
+device).  :meth:`Scheduler.resolve` later takes the values: it emits the token events, and a
+request whose token was end-of-sequence is finished then - the one token computed for it in the
+step already in flight is dropped.  Anything that must know the values first (preempting or
+failing a request) makes :meth:`plan` raise :class:`UnresolvedTokens` before it changes anything.
+:meth:`complete` is ``resolve(book(plan), sampled)``.
 """
 from __future__ import annotations
 
@@ -44,6 +54,7 @@ class Request:
     temperature: float = 0.0
     resumed_tokens: int = 0           # how many of ``tokens`` (at the end) were generated before a preemption
     arrival: int = -1
+    preempted: bool = False           # re-entered after a preemption (possibly with nothing generated yet)
 
 
 @dataclass
@@ -55,7 +66,11 @@ class Sequence_:
     generated: List[int] = field(default_factory=list)
     remaining: int = 0
     was_preempted: bool = False
-    next_token: Optional[int] = None  # sampled, not yet run through the model
+    next_token: Optional[int] = None  # sampled, not yet run through the model; negative: row
+                                      # ``-1 - next_token`` of the last sampling, value not seen yet
+    next_from: object = None          # the Ticket whose sampling ``next_token`` names
+    unresolved: int = 0               # placeholders in ``generated``
+    dead: bool = False                # finished; entries of it still in flight are dropped
 
     @property
     def prefilling(self) -> bool:
@@ -92,6 +107,19 @@ class StepPlan:
         return sum(len(e.tokens) for e in self.entries)
 
 
+@dataclass
+class Ticket:
+    """A booked step whose sampled tokens the host has not seen yet."""
+    plan: StepPlan
+    rows: List[Tuple[Sequence_, int, bool]]   # per sampled entry: sequence, index of its
+                                              # placeholder in ``generated``, ends by length
+
+
+class UnresolvedTokens(RuntimeError):
+    """Planning has to finish or preempt a request whose last tokens are not known to the host
+    yet: resolve the step in flight, then plan again."""
+
+
 def reservation_tokens(policy: str, prompt_len: int, max_new_tokens: int, max_seq_len: int) -> int:
     """Tokens a contiguous-mode request reserves (reference: ``base/src/engine.cu:301-330``)."""
     if policy == "max":
@@ -122,6 +150,7 @@ class Scheduler:
         self.reserve_policy = reserve_policy
         self.waiting: Deque[Request] = deque()
         self.running: List[Sequence_] = []
+        self.closing: List[Sequence_] = []     # out of tokens, waiting for their last value
         self._arrivals = 0
         self.preemption_pending = False
         self._preempted_in_flight = 0
@@ -137,24 +166,29 @@ class Scheduler:
         self.waiting.append(request)
 
     def idle(self) -> bool:
-        return not self.waiting and not self.running
+        return not self.waiting and not self.running and not self.closing
 
     # ------------------------------------------------------------------ helpers
     def _release(self, seq: Sequence_) -> None:
         if self.on_release:
             self.on_release(seq)
         self.cache.free(seq.seat)
-        self.running.remove(seq)
+        seq.dead = True
+        (self.running if seq in self.running else self.closing).remove(seq)
 
     def _finish(self, seq: Sequence_, reason: str, events: List[Event]) -> None:
         events.append(Event("done", seq.request.id, seq.request.seq_index, seq.seat,
                             tokens=seq.request.resumed_tokens + len(seq.generated), reason=reason))
         if seq.was_preempted:
-            self._preempted_in_flight -= 1
-            if self._preempted_in_flight <= 0:
-                self._preempted_in_flight = 0
-                self.preemption_pending = False
+            self._preempted_gone()
         self._release(seq)
+
+    def _preempted_gone(self) -> None:
+        """A request that had been preempted has left for good; admission opens again with the last."""
+        self._preempted_in_flight -= 1
+        if self._preempted_in_flight <= 0:
+            self._preempted_in_flight = 0
+            self.preemption_pending = False
 
     def _preempt(self, seq: Sequence_, events: List[Event]) -> None:
         """Recompute-style preemption: everything so far becomes the prompt of a request that
@@ -165,7 +199,7 @@ class Scheduler:
                             generated=done_before, reason="recompute"))
         resumed = Request(seq.request.id, tokens, seq.remaining, seq.request.seq_index,
                           seq.request.temperature, resumed_tokens=done_before,
-                          arrival=seq.request.arrival)
+                          arrival=seq.request.arrival, preempted=True)
         if not seq.was_preempted:
             self._preempted_in_flight += 1
         self.preemption_pending = True
@@ -181,6 +215,20 @@ class Scheduler:
         events: List[Event] = []
         cache = self.cache
         paged = cache.mode == "paged"
+
+        # finishing or preempting a request needs all its tokens' values: refuse before any change
+        pending = [s for s in self.running if s.unresolved]
+        if pending:
+            if any(not s.prefilling and s.computed + 1 > cache.capacity_tokens(s.seat) for s in pending):
+                raise UnresolvedTokens("a request with unseen tokens has filled its room in the cache")
+            if paged:
+                need = [0] * len(cache.groups)
+                for s in self.running:
+                    if not s.prefilling:
+                        for i, n in enumerate(cache.pages_needed(s.seat, s.computed + 1)):
+                            need[i] += n
+                if any(n > f for n, f in zip(need, self._free_pages())):
+                    raise UnresolvedTokens("pages run out while tokens of running requests are unseen")
 
         # a request that has filled what the cache can hold for it ends before the forward
         for seq in list(self.running):
@@ -252,7 +300,7 @@ class Scheduler:
         # 3. admissions, first come first served
         while self.waiting and budget > 0 and cache.free_seats > 0:
             head = self.waiting[0]
-            if self.preemption_pending and head.resumed_tokens == 0:
+            if self.preemption_pending and not head.preempted:
                 break
             plen = len(head.tokens)
             if plen == 0 or head.max_new_tokens < 1:
@@ -272,6 +320,8 @@ class Scheduler:
                         self.waiting.popleft()
                         events.append(Event("done", head.id, head.seq_index, tokens=head.resumed_tokens,
                                             reason="kv_cache_exhausted"))
+                        if head.preempted:
+                            self._preempted_gone()
                         continue
                     break
             else:
@@ -283,11 +333,13 @@ class Scheduler:
                     self.waiting.popleft()
                     events.append(Event("done", head.id, head.seq_index, tokens=head.resumed_tokens,
                                         reason="kv_cache_exhausted"))
+                    if head.preempted:
+                        self._preempted_gone()
                     continue
                 break       # the queue head waits for room (head-of-line, as in the reference)
             self.waiting.popleft()
             seq = Sequence_(head, seat, list(head.tokens), remaining=head.max_new_tokens,
-                            was_preempted=head.resumed_tokens > 0)
+                            was_preempted=head.preempted)
             self.running.append(seq)
             if self.on_admit:
                 self.on_admit(seq)
@@ -297,22 +349,51 @@ class Scheduler:
     # ------------------------------------------------------------------ after the forward
     def complete(self, plan: StepPlan, sampled: Sequence[int]) -> List[Event]:
         """Books the step: ``sampled`` holds one token per entry with ``sample`` set, in order."""
-        events: List[Event] = []
-        it = iter(sampled)
+        return self.resolve(self.book(plan), sampled)
+
+    def book(self, plan: StepPlan) -> Ticket:
+        """The part of booking that does not need the sampled values: lengths, counts, and a
+        placeholder per sampled token.  A request that has used up its budget of new tokens
+        leaves the running set (it is not scheduled again) and keeps its seat until
+        :meth:`resolve`."""
+        ticket = Ticket(plan, [])
         for e in plan.entries:
             seq = e.seq
             seq.computed += len(e.tokens)
             self.cache.commit(seq.seat, seq.computed)
             if not e.sample:
                 continue
-            tok = int(next(it))
+            seq.generated.append(None)
+            seq.unresolved += 1
+            seq.next_token = -1 - len(ticket.rows)
+            seq.next_from = ticket
+            seq.remaining -= 1
+            ending = seq.remaining <= 0
+            if ending:
+                self.running.remove(seq)
+                self.closing.append(seq)
+            ticket.rows.append((seq, len(seq.generated) - 1, ending))
+        return ticket
+
+    def resolve(self, ticket: Ticket, sampled: Sequence[int]) -> List[Event]:
+        """Takes the values of a booked step's sampled tokens, one per row of the ticket."""
+        events: List[Event] = []
+        if len(sampled) != len(ticket.rows):
+            raise ValueError(f"{len(sampled)} tokens for {len(ticket.rows)} sampled entries")
+        for (seq, idx, ending), tok in zip(ticket.rows, sampled):
+            if seq.dead:
+                continue            # ended by an earlier token while this step was in flight
+            tok = int(tok)
+            seq.unresolved -= 1
             if tok in self.eos and not self.ignore_eos:
+                del seq.generated[idx:]
+                seq.unresolved = 0
                 self._finish(seq, "eos", events)
                 continue
-            seq.generated.append(tok)
-            seq.next_token = tok
-            seq.remaining -= 1
+            seq.generated[idx] = tok
+            if seq.next_from is ticket:
+                seq.next_token, seq.next_from = tok, None
             events.append(Event("token", seq.request.id, seq.request.seq_index, seq.seat, token=tok))
-            if seq.remaining <= 0:
+            if ending:
                 self._finish(seq, "length", events)
         return events

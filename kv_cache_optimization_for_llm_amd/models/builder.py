@@ -138,7 +138,7 @@ class Model:
         ``[len(batch.logit_rows), vocab]``."""
         T = batch.num_tokens
         hidden = torch.empty((T, self.spec.hidden_size), dtype=self.dtype, device=self.device)
-        K.embed_gather(self.embedding, batch.token_ids, hidden)
+        K.embed_gather(self.embedding, batch.token_ids, hidden, getattr(batch, "feedback", None))
         delta = None
         for i, (call, slot) in enumerate(self.calls):
             block = self.blocks[call.layer]

@@ -57,14 +57,18 @@ def check_cache_shapes(what: str, k_cache: torch.Tensor, v_cache: torch.Tensor, 
 
 
 # --------------------------------------------------------------------------------------
-def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[t, :] = table[ids[t], :], converted to out's dtype."""
+def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor,
+                 feedback: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t, :] = table[ids[t], :], converted to out's dtype.  A negative id ``-1 - r`` stands
+    for ``feedback[r]`` (a token still on the device); the caller guarantees ``r`` is inside
+    ``feedback`` and that no id is negative when there is none."""
     rows, width = out.shape
     if table.dim() != 2 or table.shape[1] != width or ids.shape != (rows,):
         raise KernelError(f"embed_gather: shapes table {tuple(table.shape)} ids {tuple(ids.shape)} "
                           f"out {tuple(out.shape)} do not fit")
     check(hip_lib().kva_embed_gather(_dev(out, "out"), _dev(table, "table"),
-                                     _dev(ids, "ids", torch.int32), rows, width,
+                                     _dev(ids, "ids", torch.int32),
+                                     _opt(feedback, "feedback", torch.int32), rows, width,
                                      dtype_code(table.dtype), dtype_code(out.dtype), _stream()),
           "embed_gather")
     return out

@@ -32,7 +32,7 @@ LL = c_longlong
 U = c_uint
 
 _HIP_SIGNATURES = {
-    "kva_embed_gather": [P, P, P, I, I, I, I, P],
+    "kva_embed_gather": [P, P, P, P, I, I, I, I, P],
     "kva_rmsnorm": [P, P, P, P, P, I, I, F, I, I, P],
     "kva_residual_add": [P, P, LL, I, P],
     "kva_silu_mul": [P, P, I, I, I, P],

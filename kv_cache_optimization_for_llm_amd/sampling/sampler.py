@@ -50,6 +50,21 @@ def _as_i32(values: Sequence[int]) -> np.ndarray:
     return (np.asarray(values, dtype=np.int64) & 0xFFFFFFFF).astype(np.uint32).view(np.int32)
 
 
+class PendingTokens:
+    """Sampled tokens on their way to the host: the copy into pinned memory has been queued and
+    :meth:`wait` blocks until it has arrived."""
+
+    def __init__(self, host: torch.Tensor, event: "torch.cuda.Event", n: int):
+        self._host, self._event, self._n = host, event, n
+        self._value: Optional[np.ndarray] = None
+
+    def wait(self) -> np.ndarray:
+        if self._value is None:
+            self._event.synchronize()
+            self._value = self._host.numpy()[:self._n].copy()
+        return self._value
+
+
 class Sampler:
     def __init__(self, vocab_size: int, max_seqs: int, device, *, seed: int = 0,
                  repetition_penalty: float = 1.0, chunks: int = 128):
@@ -61,6 +76,9 @@ class Sampler:
         self.mask: Optional[torch.Tensor] = None
         if self.penalty != 1.0:
             self.mask = torch.zeros((max_seqs, vocab_size), dtype=torch.uint8, device=device)
+        # pinned landing buffers for sample_async, used in turn (two samplings may be in flight)
+        self._landing: List[torch.Tensor] = []
+        self._landing_next = 0
 
     def reset_seat(self, seat: int, emitted: Sequence[int] = ()) -> None:
         """A request takes the seat: clear its mask and mark what it has emitted before (a
@@ -80,12 +98,30 @@ class Sampler:
 
     def sample(self, logits: torch.Tensor, rows: Sequence[SampleRow]) -> np.ndarray:
         """One token per logits row; returns host int32."""
+        return self.sample_async(logits, rows).wait()
+
+    def sample_async(self, logits: torch.Tensor, rows: Sequence[SampleRow],
+                     out: Optional[torch.Tensor] = None) -> PendingTokens:
+        """Queues the sampling of one token per logits row and their copy to the host, without
+        waiting for either.  ``out`` (device int32, at least ``len(rows)`` long) takes the tokens,
+        row by row, and may be read by later work on the same stream."""
         n = len(rows)
         if logits.shape != (n, self.vocab_size):
             raise ValueError(f"logits {tuple(logits.shape)} do not fit {n} rows of {self.vocab_size}")
-        out = torch.empty(n, dtype=torch.int32, device=self.device)
+        if out is None:
+            out = torch.empty(max(n, 1), dtype=torch.int32, device=self.device)
+        if out.dtype != torch.int32 or out.dim() != 1 or out.shape[0] < n:
+            raise ValueError("sample: out must be a device int32 vector with a place per row")
+        out = out[:n]
+        if len(self._landing) < 3 or self._landing[0].shape[0] < n:
+            size = max(64, n)
+            self._landing = [torch.zeros(size, dtype=torch.int32, pin_memory=True) for _ in range(3)]
+        host = self._landing[self._landing_next]
+        self._landing_next = (self._landing_next + 1) % len(self._landing)
+        event = torch.cuda.Event()
         if n == 0:
-            return np.zeros(0, dtype=np.int32)
+            event.record()
+            return PendingTokens(host, event, 0)
         any_sampled = any(r.temperature > 0 for r in rows)
         inv_t = key = step = seat_t = None
         if any_sampled:
@@ -100,7 +136,9 @@ class Sampler:
         K.sample(logits, out, chunks=self.chunks, inv_temperature=inv_t, seed=self.seed, rng_key=key,
                  rng_step=step, penalty_mask=self.mask if use_mask else None, row_seat=seat_t,
                  penalty=self.penalty)
-        tokens = out.cpu().numpy()
+        host[:n].copy_(out, non_blocking=True)
+        event.record()
         if self.mask is not None:
-            self.mark([r.seat for r in rows], tokens)
-        return tokens
+            seats = torch.from_numpy(np.asarray([r.seat for r in rows], dtype=np.int32)).to(self.device)
+            K.mark_tokens(self.mask, seats, out)
+        return PendingTokens(host, event, n)

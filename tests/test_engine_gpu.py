@@ -104,6 +104,47 @@ def test_eos_ends_generation_and_is_not_returned(model_dirs, gpu):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_running_ahead_of_the_device_changes_nothing_that_is_emitted(dtype, model_dirs, gpu):
+    """The serving loop launches a step before it has seen the previous step's tokens (they stay
+    on the device).  Same requests with and without that: same tokens, same reasons - with
+    end-of-sequence tokens arriving at different times, more requests than seats, a repetition
+    penalty and a temperature."""
+    name = "C"
+    prompts = prompts_for(name, [12, 3, 40, 25, 7, 18], seed=11)
+    d = json.load(open(os.path.join(model_dirs[name], "config.json")))
+    import shutil
+    import tempfile
+    with tempfile.TemporaryDirectory() as tmp:
+        shutil.copy(os.path.join(model_dirs[name], "model.safetensors"), tmp)
+        json.dump(d, open(os.path.join(tmp, "config.json"), "w"))
+        probe = LLM(tmp, EngineOptions(dtype=dtype, max_seqs=3, max_seq_len=128), ServeOptions(run_ahead=False))
+        free = probe.generate(prompts, max_new_tokens=24, ignore_eos=True)
+        # end-of-sequence ids that some requests meet early, some late and some never
+        d["eos_token_id"] = [free[0][5], free[2][14], free[4][1]]
+        json.dump(d, open(os.path.join(tmp, "config.json"), "w"))
+        results = {}
+        for ahead in (False, True):
+            llm = LLM(tmp, EngineOptions(dtype=dtype, max_seqs=3, max_seq_len=128),
+                      ServeOptions(run_ahead=ahead, max_batch_tokens=32, chunk_size=16))
+            results[ahead] = [
+                llm.generate(prompts, max_new_tokens=24, return_reasons=True),
+                llm.generate(prompts, max_new_tokens=24, return_reasons=True, temperature=0.9, seed=3,
+                             repetition_penalty=1.15),
+            ]
+            llm.engine.cache.check()
+            assert llm.engine.cache.free_seats == 3
+        assert results[True] == results[False]
+        got, reasons = results[True][0]
+        assert "eos" in reasons and "length" in reasons
+        eos = set(d["eos_token_id"])
+        for g, f, r in zip(got, free, reasons):
+            stop = next((i for i, t in enumerate(f) if t in eos), None)
+            if dtype == "float32":
+                assert g == (f if stop is None else f[:stop]) and r == ("length" if stop is None else "eos")
+            assert not eos & set(g)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_and_first_tokens(dtype, model_dirs, gpu):
     """300 tokens decoded one by one from a one-token start: crosses many pages and several
     context buckets of the graphs; every position is compared with the plain logits."""

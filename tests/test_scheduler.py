@@ -195,3 +195,120 @@ def test_contiguous_mode_blocks_at_the_head_never_preempts_and_stops_at_the_rese
     s.add(Request(0, [9] * 60, 100))
     out, reasons, _, _ = run(s)
     assert reasons[(0, 0)] == "sequence_too_long" and len(out[(0, 0)]) == 5
+
+
+# ----------------------------------------------------------------------------------------------
+# Running ahead: a step is booked before its tokens are known and resolved one step later.
+
+def run_ahead(s, max_steps=10000):
+    """Like ``run``, but the tokens of a step reach the scheduler only after the NEXT step has been
+    planned and booked, and a decode entry may name its token by feedback row."""
+    from kv_cache_optimization_for_llm_amd.engine.scheduler import UnresolvedTokens
+    out, reasons, events = {}, {}, []
+    in_flight = None                       # (ticket, sampled values)
+    resolved_early = 0
+    feedback = []                          # what "the device" holds: the last sampling's tokens
+
+    def resolve():
+        nonlocal in_flight
+        evs = s.resolve(*in_flight) if in_flight else []
+        in_flight = None
+        return evs
+
+    for _ in range(max_steps):
+        if s.idle() and in_flight is None:
+            break
+        evs = []
+        try:
+            plan = s.plan()
+        except UnresolvedTokens:
+            resolved_early += 1
+            evs += resolve()
+            plan = s.plan()
+        s.cache.check()
+        launched = None
+        if plan.entries:
+            sampled = []
+            for e in plan.entries:
+                assert s.cache.grow(e.seq.seat, e.start + len(e.tokens)), "the plan promised pages it cannot get"
+                toks = [feedback[-1 - t] if t < 0 else t for t in e.tokens]
+                if len(e.tokens) == 1 and e.start >= len(e.seq.prompt):
+                    # a decoded token is the one "the model" sampled for this position
+                    assert toks[0] == fake_token(e.seq.request.id, e.start), "a stale feedback row was named"
+                assert all(t >= 0 for t in toks[1:]) and (toks[0] >= 0)
+                if e.sample:
+                    sampled.append(fake_token(e.seq.request.id, e.start + len(e.tokens)))
+            launched = (s.book(plan), sampled)
+            feedback = sampled
+        evs += resolve()
+        evs += plan.events
+        in_flight = launched
+        s.cache.check()
+        for ev in evs:
+            key = (ev.request_id, ev.seq_index)
+            if ev.kind == "token":
+                out.setdefault(key, []).append(ev.token)
+            elif ev.kind in ("done", "rejected"):
+                assert key not in reasons, "a request finished twice"
+                reasons[key] = ev.reason
+        events += evs
+    assert s.idle() and in_flight is None, "the scheduler did not finish"
+    return out, reasons, events, resolved_early
+
+
+def eos_position(request_id, start, limit=400):
+    for p in range(start, limit):
+        if fake_token(request_id, p) == EOS + 8:
+            return p
+    return None
+
+
+@pytest.mark.parametrize("pages", [64, 8])
+def test_running_ahead_gives_the_tokens_and_reasons_of_the_synchronous_loop(pages):
+    """Same requests, same made-up model: booking a step before its tokens are seen changes when
+    things are known, not what is emitted - with end-of-sequence tokens (a token computed for a
+    request that had already ended is dropped) and, with few pages, preemptions (which wait for
+    the values)."""
+    eos = EOS + 8                                     # a value fake_token does produce
+    lens = [5, 17, 33, 40, 1, 9, 21]
+
+    def make():
+        s = Scheduler(cache(pages=pages, seqs=4), max_batch_tokens=48, chunk_size=16, eos_token_ids=[eos])
+        for i, n in enumerate(lens):
+            s.add(Request(i, [20 + (j % 50) for j in range(n)], 30 + i))
+        return s
+
+    want_out, want_reasons, _, _ = run(make())
+    s = make()
+    out, reasons, events, early = run_ahead(s)
+    assert out == want_out and reasons == want_reasons
+    assert any(r == "eos" for r in reasons.values()) and any(r == "length" for r in reasons.values())
+    if pages == 8:
+        assert s.preemptions > 0 and early > 0
+    assert all(g.free_pages() == g.num_pages for g in s.cache.groups) and s.cache.free_seats == 4
+
+
+def test_planning_refuses_to_preempt_while_tokens_are_unseen_and_changes_nothing():
+    from kv_cache_optimization_for_llm_amd.engine.scheduler import UnresolvedTokens
+    s = Scheduler(cache(pages=4, seqs=4), max_batch_tokens=64, ignore_eos=True)
+    s.add(Request(0, list(range(8, 8 + 31)), 40))
+    s.add(Request(1, list(range(8, 8 + 31)), 40))
+    p = s.plan()                                       # both prompts: 2 pages each, pool is full
+    for e in p.entries:
+        assert s.cache.grow(e.seq.seat, e.start + len(e.tokens))
+    t1 = s.book(p)
+    p2 = s.plan()                                      # position 31 still fits the second page
+    assert [e.tokens for e in p2.entries] == [[-1], [-2]]
+    for e in p2.entries:
+        assert s.cache.grow(e.seq.seat, e.start + 1)
+    s.resolve(t1, [fake_token(0, 31), fake_token(1, 31)])
+    t2 = s.book(p2)
+    before = (len(s.running), len(s.waiting), s.preemptions, [g.free_pages() for g in s.cache.groups])
+    with pytest.raises(UnresolvedTokens):
+        s.plan()                                       # position 32 needs a third page each: none free
+    assert before == (len(s.running), len(s.waiting), s.preemptions, [g.free_pages() for g in s.cache.groups])
+    evs = s.resolve(t2, [fake_token(0, 32), fake_token(1, 32)])
+    assert [e.kind for e in evs] == ["token", "token"]
+    p3 = s.plan()
+    assert [e.kind for e in p3.events] == ["preempted"] and p3.events[0].request_id == 1
+    assert s.waiting[0].tokens[-2:] == [fake_token(1, 31), fake_token(1, 32)]
