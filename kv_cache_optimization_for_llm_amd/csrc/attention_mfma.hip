@@ -32,6 +32,7 @@
 // Reference: same recurrence as paged_attention/src/kernels.cu:150-219 and the tiled prefill
 // kernel base/src/kernels.cu:361-466, which work one key at a time on CUDA cores.
 #include "common.h"
+#include <type_traits>
 #include <math.h>
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -59,20 +60,19 @@ union Frag4 {
 };
 
 template <int D, int RT, bool FAST>
-__global__ void __launch_bounds__(KVA_WAVE)
-attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
+__device__ __forceinline__ void
+attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
                       const bf16_t *__restrict__ q, int q_row_stride,
                       const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
                       const int *__restrict__ block_table, int max_blocks,
                       const int *__restrict__ item_entry, const int *__restrict__ item_row0,
                       const int *__restrict__ entry_seat, const int *__restrict__ entry_q_start,
                       const int *__restrict__ entry_start_pos, int num_q_heads, int num_kv_heads,
-                      int page_size, float scale, int window, int splits, int keys_per_split) {
+                      int page_size, float scale, int window, int splits, int keys_per_split, const int item, const int kvh, const int split) {
     constexpr int KSTEP = (D % 32 == 0) ? 32 : 16;   // head-dim slice per S^T product
     constexpr int NKS = D / KSTEP;
     constexpr int NDT = D / 16;                      // 16-wide tiles of the value dimension
 
-    const int item = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
     const int lane = threadIdx.x, r = lane & 15, g = lane >> 4;
     const int G = num_q_heads / num_kv_heads;
 
@@ -87,7 +87,7 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
 
     // per row tile: this lane's query row
     bool row_valid[RT];
-    int tq[RT], head[RT], my_pos[RT], my_lo[RT], tile_hi[RT];
+    int tq[RT], head[RT], my_pos[RT], my_lo[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         const int row = row0 + rt * 16 + r;
@@ -96,8 +96,6 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
         head[rt] = kvh * G + (row_valid[rt] ? row % G : 0);
         my_pos[rt] = start_pos + tq[rt];
         my_lo[rt] = (window > 0 && my_pos[rt] - window + 1 > 0) ? my_pos[rt] - window + 1 : 0;
-        const int last = (row0 + rt * 16 + 15 < M - 1) ? row0 + rt * 16 + 15 : M - 1;
-        tile_hi[rt] = (row0 + rt * 16 < M) ? start_pos + last / G : -1;   // last key the tile sees
     }
 
     // keys any row of this item may see
@@ -159,12 +157,18 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
     constexpr uint32_t v_tile_stride = 16u * 16u * 2u;                         // 16 value dims
     auto load_block = [&](BlockFrags &f, int kstart) {
         if constexpr (FAST) {
+            // the index is uniform: said so explicitly, the lookups are scalar loads (both issued
+            // before either is waited for) and do not stand in the queue of the vector loads
+            int pg[2];
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
                 int tile0 = kstart + t * 16;
                 tile0 = tile0 < lo_tile ? lo_tile : (tile0 > hi_tile ? hi_tile : tile0);
-                const int pg = __builtin_amdgcn_readfirstlane(bt[tile0 >> 4]);
-                const size_t page_bytes = ((size_t)pg * num_kv_heads + kvh) * (size_t)(16 * D * 2);
+                pg[t] = bt[__builtin_amdgcn_readfirstlane(tile0 >> 4)];
+            }
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const size_t page_bytes = ((size_t)pg[t] * num_kv_heads + kvh) * (size_t)(16 * D * 2);
                 const char *kb = reinterpret_cast<const char *>(k_cache) + page_bytes;
                 const char *vb = reinterpret_cast<const char *>(v_cache) + page_bytes;
 #pragma unroll
@@ -211,88 +215,117 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
         }
     };
 
-    // scores are kept in the base-2 domain: exp(x) = exp2(x * log2(e))
+    // exponentials are taken in base 2: exp(x * scale) = exp2(x * scale * log2(e))
     const float scale2 = scale * 1.44269504088896340736f;
     const int first_pos = start_pos + row0 / G;          // smallest position among the item's rows
     const bool all_rows = row0 + 16 * RT <= M;
 
-    auto compute_block = [&](const BlockFrags &f, int kstart) {
-        // blocks wholly visible to every row of the item need no mask
-        const bool masked = window > 0 || kstart + 31 > first_pos || !all_rows;   // incl. redirected tiles
+    // One 32-key block for all row tiles of the item, as straight-line code: first every S^T
+    // product, then the softmax updates, then every P V product, so that the independent chains
+    // of the row tiles overlap (matrix-core latency behind vector work and the other way round).
+    // MASKED is decided per block (wave-uniform): blocks wholly visible to every row need no mask.
+    auto compute_block_as = [&](auto masked_tag, const BlockFrags &f, int kstart) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        f32x4 s[RT][2];
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-            if (RT > 1 && kstart > tile_hi[rt]) continue;               // wave-uniform
-            // ---- S^T for two 16-key tiles
-            f32x4 s[2];
+        for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-                s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+                s[rt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ks = 0; ks < NKS; ++ks) {
                     if (KSTEP == 32)
-                        s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k8[t][ks].v, qf8[rt][ks].v, s[t], 0, 0, 0);
+                        s[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k8[t][ks].v, qf8[rt][ks].v, s[rt][t], 0, 0, 0);
                     else
-                        s[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(f.k4[t][ks].v, qf4[rt][ks].v, s[t], 0, 0, 0);
+                        s[rt][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(f.k4[t][ks].v, qf4[rt][ks].v, s[rt][t], 0, 0, 0);
                 }
             }
-            // ---- scale, mask, online softmax for query row r (its keys are spread over 4 lane groups)
-            float sv[8];
-            float mloc = -INFINITY;
+        // ---- mask, online softmax for query row r (its keys are spread over 4 lane groups).
+        // m and the maxima are kept in the domain of the raw products q.k; the scale (times
+        // log2 e, for exp2) goes into the one fused multiply-add in front of every exponential.
+        float sv[RT][8], mloc[RT];
+        Frag8 pf[RT];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            float mx = -INFINITY;
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    float x = s[t][i] * scale2;
-                    if (masked) {
+                    float x = s[rt][t][i];
+                    if (MASKED) {
                         const int key = kstart + t * 16 + 4 * g + i;
                         const bool vis = row_valid[rt] && key <= my_pos[rt] && key >= my_lo[rt];
                         x = vis ? x : -INFINITY;
                     }
-                    sv[t * 4 + i] = x;
-                    mloc = fmaxf(mloc, x);
+                    sv[rt][t * 4 + i] = x;
+                    mx = fmaxf(mx, x);
                 }
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 16, KVA_WAVE));
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, KVA_WAVE));
-            const float m_new = fmaxf(m[rt], mloc);
-            // a row that has seen no key yet keeps m = -inf: use 0 as the reference instead
-            const float m_ref = (m_new == -INFINITY) ? 0.f : m_new;
-            const float corr = __builtin_amdgcn_exp2f(m[rt] - m_ref);
-            float lsum = 0.f;
-            Frag8 pf;
+            mloc[rt] = quad_rows_max(mx);
+        }
+        // m[rt] is the reference the row's exponentials are taken against.  It follows the
+        // running maximum lazily: only when a row's maximum has outgrown it by more than
+        // 2^REBASE (after scaling) does the wave re-base (multiply l and O by
+        // exp2((old - new) * scale2)), which costs as much as the rest of the block.  In between,
+        // p = exp2((s - m) * scale2) may reach 2^REBASE, which fp32 sums and bf16 products hold
+        // without loss; o / l does not depend on the reference.
+        constexpr float REBASE = 8.f;
+        const float rebase_raw = REBASE / scale2;
+        bool rebase = false;
 #pragma unroll
-            for (int j = 0; j < 8; j += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(sv[j] - m_ref);   // exp2(-inf) = 0
-                const float p1 = __builtin_amdgcn_exp2f(sv[j + 1] - m_ref);
-                lsum += p0 + p1;
-                pf.p2[j / 2] = pack_bf16(p0, p1);
-            }
-            lsum += __shfl_xor(lsum, 16, KVA_WAVE);
-            lsum += __shfl_xor(lsum, 32, KVA_WAVE);
-            l[rt] = l[rt] * corr + lsum;
-            m[rt] = m_new;
-            // ---- O^T += V^T * P^T
-            if (__builtin_amdgcn_ballot_w64(corr != 1.f) != 0) {           // some row's maximum moved
+        for (int rt = 0; rt < RT; ++rt) rebase = rebase || mloc[rt] > m[rt] + rebase_raw;
+        if (__builtin_amdgcn_ballot_w64(rebase) != 0) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                const float m_new = fmaxf(m[rt], mloc[rt]);
+                // a row that has seen no key yet keeps m = -inf (exp2(-inf) = 0 clears nothing that counts)
+                const float c = __builtin_amdgcn_exp2f((m[rt] - ((m_new == -INFINITY) ? 0.f : m_new)) * scale2);
+                l[rt] *= c;
 #pragma unroll
                 for (int dt = 0; dt < NDT; ++dt) {
-                    o[rt][dt][0] *= corr; o[rt][dt][1] *= corr; o[rt][dt][2] *= corr; o[rt][dt][3] *= corr;
+                    o[rt][dt][0] *= c; o[rt][dt][1] *= c; o[rt][dt][2] *= c; o[rt][dt][3] *= c;
                 }
+                m[rt] = m_new;
             }
+        }
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            const float neg_ref = (MASKED && m[rt] == -INFINITY) ? 0.f : -m[rt] * scale2;
+            float lsum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; j += 2) {
+                const float p0 = __builtin_amdgcn_exp2f(fmaf(sv[rt][j], scale2, neg_ref));   // exp2(-inf) = 0
+                const float p1 = __builtin_amdgcn_exp2f(fmaf(sv[rt][j + 1], scale2, neg_ref));
+                lsum += p0 + p1;
+                pf[rt].p2[j / 2] = pack_bf16(p0, p1);
+            }
+            l[rt] += quad_rows_sum(lsum);
+        }
+        // ---- O^T += V^T * P^T
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt)
-                o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.v[dt].v, pf.v, o[rt][dt], 0, 0, 0);
-        }
+                o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.v[dt].v, pf[rt].v, o[rt][dt], 0, 0, 0);
+    };
+    auto compute_block = [&](const BlockFrags &f, int kstart) {
+        // incl. redirected tiles and items whose last row tile is cut short
+        const bool masked = window > 0 || kstart + 31 > first_pos || !all_rows;
+        if (masked) compute_block_as(std::true_type{}, f, kstart);
+        else compute_block_as(std::false_type{}, f, kstart);
     };
 
+    // Two blocks in flight (a third does not pay: the waits are for bandwidth, not latency).  The
+    // loads are issued unconditionally (a block past the end is
+    // redirected or predicated off inside load_block and its values are never used): a load
+    // under a branch would make the wait before the next product a wait for everything.
     BlockFrags fa, fb;
-    if (k_begin < k_end) load_block(fa, k_begin);
+    load_block(fa, k_begin);
     for (int kstart = k_begin; kstart < k_end; kstart += 64) {
-        const bool second = kstart + 32 < k_end;
-        if (second) load_block(fb, kstart + 32);
+        load_block(fb, kstart + 32);
         compute_block(fa, kstart);
-        if (second) {
-            if (kstart + 64 < k_end) load_block(fa, kstart + 64);
-            compute_block(fb, kstart + 32);
-        }
+        load_block(fa, kstart + 64);
+        if (kstart + 32 < k_end) compute_block(fb, kstart + 32);
     }
 
     // lane (r, g) holds O[row r][dt * 16 + 4g + i]
@@ -317,11 +350,38 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
                 *reinterpret_cast<float4 *>(dst + dt * 16 + 4 * g) =
                     make_float4(o[rt][dt][0], o[rt][dt][1], o[rt][dt][2], o[rt][dt][3]);
             if (g == 0) {
-                part_ml[(orow * splits + split) * 2] = m[rt];
+                part_ml[(orow * splits + split) * 2] = m[rt] * scale2;   // the merge works in the base-2 domain
                 part_ml[(orow * splits + split) * 2 + 1] = l[rt];
             }
         }
     }
+}
+
+// One wavefront per (item or pair of items, kv head, key split).  Workgroups are handed to the 8
+// dies in turn, each die with its own L2: the kv head varies fastest, so a die keeps meeting the
+// same heads' keys and values.  With `pair`, a wavefront takes item w and then item n-1-w of the
+// list: the caller orders the list by the number of keys an item visits (most first), so every
+// wavefront gets about the same work - rows late in a prompt visit many keys, early rows few.
+template <int D, int RT, bool FAST>
+__global__ void __launch_bounds__(KVA_WAVE)
+attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
+                      const bf16_t *__restrict__ q, int q_row_stride,
+                      const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
+                      const int *__restrict__ block_table, int max_blocks,
+                      const int *__restrict__ item_entry, const int *__restrict__ item_row0,
+                      const int *__restrict__ entry_seat, const int *__restrict__ entry_q_start,
+                      const int *__restrict__ entry_start_pos, int num_q_heads, int num_kv_heads,
+                      int page_size, float scale, int window, int splits, int keys_per_split, int num_items, int pair) {
+    const int kvh = blockIdx.x % num_kv_heads, split = blockIdx.z;
+    const int w = blockIdx.x / num_kv_heads;
+    attention_item<D, RT, FAST>(out, part_o, part_ml, q, q_row_stride, k_cache, v_cache, block_table, max_blocks,
+                                item_entry, item_row0, entry_seat, entry_q_start, entry_start_pos, num_q_heads,
+                                num_kv_heads, page_size, scale, window, splits, keys_per_split, w, kvh, split);
+    const int other = num_items - 1 - w;
+    if (pair && other > w)
+        attention_item<D, RT, FAST>(out, part_o, part_ml, q, q_row_stride, k_cache, v_cache, block_table, max_blocks,
+                                    item_entry, item_row0, entry_seat, entry_q_start, entry_start_pos, num_q_heads,
+                                    num_kv_heads, page_size, scale, window, splits, keys_per_split, other, kvh, split);
 }
 
 // out[row, :] = sum_s o_s * exp(m_s - M) / sum_s l_s * exp(m_s - M),  M = max_s m_s.
@@ -381,7 +441,7 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
                                   const int *entry_seat, const int *entry_q_start,
                                   const int *entry_start_pos, int total_rows, int num_q_heads,
                                   int num_kv_heads, int head_dim, int page_size, float scale, int window,
-                                  int splits, int keys_per_split, hipStream_t stream) {
+                                  int splits, int keys_per_split, int pair, hipStream_t stream) {
     KVA_REQUIRE(num_items >= 0 && num_q_heads > 0 && num_kv_heads > 0 && max_blocks > 0,
                 "attention_mfma: bad sizes");
     KVA_REQUIRE(num_q_heads % num_kv_heads == 0, "attention_mfma: %d query heads is not a multiple of %d kv heads",
@@ -395,17 +455,20 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
     KVA_REQUIRE(splits == 1 || (keys_per_split > 0 && keys_per_split % 32 == 0 && part_o && part_ml),
                 "attention_mfma: splits need a key count that is a multiple of 32 and a workspace");
     KVA_REQUIRE(window >= 0, "attention_mfma: negative window");
+    KVA_REQUIRE(scale > 0.f, "attention_mfma: the score scale must be positive");
     KVA_REQUIRE(row_tiles == 1 || row_tiles == kva_attention_mfma_row_tiles(head_dim, 1),
                 "attention_mfma: %d row tiles per item is not what head_dim %d is built with", row_tiles, head_dim);
     if (num_items == 0) return KVA_OK;
-    dim3 grid(num_items, num_kv_heads, splits), block(KVA_WAVE);
+    KVA_REQUIRE((long)num_items * num_kv_heads < (1L << 31), "attention_mfma: too many work items");
+    const int waves_x = pair ? (num_items + 1) / 2 : num_items;
+    dim3 grid(waves_x * num_kv_heads, 1, splits), block(KVA_WAVE);
     const bool fast = page_size == 16;
 #define LAUNCH(DD, RR, FF)                                                                      \
     hipLaunchKernelGGL((attention_mfma_kernel<DD, RR, FF>), grid, block, 0, stream, (bf16_t *)out, \
                        part_o, part_ml, (const bf16_t *)q, q_row_stride, (const bf16_t *)k_cache, \
                        (const bf16_t *)v_cache, block_table, max_blocks, item_entry, item_row0,  \
                        entry_seat, entry_q_start, entry_start_pos, num_q_heads, num_kv_heads,    \
-                       page_size, scale, window, splits, keys_per_split)
+                       page_size, scale, window, splits, keys_per_split, num_items, pair)
 #define CASE(DD, WIDE)                                                                          \
     case DD:                                                                                    \
         if (row_tiles == 1) {                                                                   \

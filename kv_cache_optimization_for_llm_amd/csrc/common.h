@@ -78,6 +78,28 @@ __device__ inline float wave_max(float v) {
     return v;
 }
 
+// Reductions over the four lanes {r, r + 16, r + 32, r + 48} (r = lane % 16), every one of them
+// getting the result.  v_permlane16_swap / v_permlane32_swap exchange 16- and 32-lane halves
+// between two registers in the vector ALU (no trip through LDS as a wave shuffle takes): from two
+// copies of x they leave (x of the lower half, x of the upper half) in every lane.
+__device__ inline float quad_rows_sum(float x) {
+    const unsigned u = __float_as_uint(x);
+    auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const float y = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    const unsigned v = __float_as_uint(y);
+    auto b = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+__device__ inline float quad_rows_max(float x) {
+    const unsigned u = __float_as_uint(x);
+    auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const float y = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    const unsigned v = __float_as_uint(y);
+    auto b = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
 // Sum over a whole workgroup of `nwaves` wavefronts; `scratch` holds at least nwaves floats.
 // Every thread gets the result.  The order of the additions is fixed.
 __device__ inline float block_sum(float v, float *scratch, int nwaves) {

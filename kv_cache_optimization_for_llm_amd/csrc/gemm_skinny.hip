@@ -266,8 +266,7 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
         rinv[mt] = 1.f;
         if (a.sumsq != nullptr) {
             float s = ssum[mt];
-            s += __shfl_xor(s, 16, KVA_WAVE);
-            s += __shfl_xor(s, 32, KVA_WAVE);
+            s = quad_rows_sum(s);
             rinv[mt] = 1.f / sqrtf(s / (float)a.norm_width + a.eps);
         }
     }
@@ -408,8 +407,7 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
                         }
                     }
                 }
-                ss += __shfl_xor(ss, 16, KVA_WAVE);
-                ss += __shfl_xor(ss, 32, KVA_WAVE);
+                ss = quad_rows_sum(ss);
                 if (m_ok && g == 0) a.sumsq_out[(size_t)m * n_tiles + tile] = ss;
                 continue;
             }

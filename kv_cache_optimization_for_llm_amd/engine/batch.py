@@ -58,7 +58,8 @@ class StepBatch:
     def attention_items(self, group: int, row_tiles: int = 1):
         """Work items of the matrix-core attention kernel for a query-head group size: (entry,
         first row) of every ``16 * row_tiles`` query rows, row = token_in_step * group +
-        head_in_group."""
+        head_in_group; ordered by the number of keys an item visits, most first (when the
+        entries' start positions are known on the host)."""
         key = (group, row_tiles)
         if key not in self._items:
             lens = np.diff(self.h_entry_q_start)
@@ -67,7 +68,15 @@ class StepBatch:
                 starts = np.arange(0, int(n) * group, 16 * row_tiles, dtype=np.int32)
                 ent.append(np.full(starts.shape[0], e, dtype=np.int32))
                 row0.append(starts)
-            both = np.concatenate([np.concatenate(ent), np.concatenate(row0)])
+            ent, row0 = np.concatenate(ent), np.concatenate(row0)
+            if self.h_entry_start_pos is not None and ent.shape[0] > 1:
+                # most keys first: the kernel hands out items in list order (and may give a
+                # wavefront the i-th and the i-th last), so the long ones should start early
+                last_row = np.minimum(row0 + 16 * row_tiles, lens[ent] * group) - 1
+                keys = self.h_entry_start_pos[ent] + last_row // group + 1
+                order = np.argsort(-keys, kind="stable")
+                ent, row0 = ent[order], row0[order]
+            both = np.concatenate([ent, row0])
             dev = torch.from_numpy(both).to(self.token_ids.device, non_blocking=True)
             n = both.shape[0] // 2
             self._items[key] = (dev[:n], dev[n:])

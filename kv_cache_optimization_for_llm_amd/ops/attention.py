@@ -15,6 +15,7 @@ _TARGET_WAVES = 2048
 _MIN_KEYS_PER_SPLIT = 128
 # wide items (two row tiles per wave) are used when they alone give this many waves
 _WIDE_MIN_WAVES = 1024
+_PAIR_MIN_WAVES = 2048      # two items per wavefront once that still leaves a wavefront per SIMD
 
 
 def choose_splits(num_items: int, num_kv_heads: int, max_context: int) -> tuple:
@@ -41,7 +42,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
     if qkv.dtype == torch.bfloat16 and K.attention_mfma_supported(head_dim, kv.page_size) \
             and qkv.shape[1] % 8 == 0:
         group = num_q_heads // num_kv_heads
-        tiles, splits, per = 1, 1, 0
+        tiles, splits, per, pair = 1, 1, 0, False
         if batch.max_q_len * group > 16:
             # prompt portions: two row tiles per wave, so each key and value loaded serves 32
             # query rows; whole key ranges as long as that still gives a wave per SIMD
@@ -49,13 +50,17 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
             item_entry, item_row0 = batch.attention_items(group, tiles)
             if item_entry.shape[0] * num_kv_heads < _WIDE_MIN_WAVES:
                 tiles = 1
+            else:
+                # items come ordered by work: a wavefront that takes the i-th and the i-th last
+                # does about the average; worth it while every SIMD still gets a wavefront
+                pair = item_entry.shape[0] * num_kv_heads >= _PAIR_MIN_WAVES
         if tiles == 1:
             item_entry, item_row0 = batch.attention_items(group, 1)
             splits, per = choose_splits(item_entry.shape[0], num_kv_heads, batch.max_context)
         return K.attention_mfma(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table,
                                 item_entry, item_row0, batch.entry_seat, batch.entry_q_start,
                                 batch.entry_start_pos, num_q_heads, num_kv_heads, head_dim, scale,
-                                window, splits, per, tiles)
+                                window, splits, per, tiles, pair)
     return K.attention_rowwise(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table,
                                batch.tok_seat, batch.positions, num_q_heads, num_kv_heads,
                                head_dim, scale, window)

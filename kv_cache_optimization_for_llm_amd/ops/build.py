@@ -28,6 +28,9 @@ HIP_FLAGS = [
     f"--offload-arch={GPU_ARCH}", "-O3", "-fPIC", "-std=c++17",
     # packed fp32 arithmetic is kept off for every kernel of this package
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # matrix-core results go to ordinary vector registers: the kernels work on them at once
+    # (softmax, epilogues) and would otherwise copy every value out of the accumulation registers
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wno-unused-result", "-Wno-unknown-attributes",
 ]
 HOST_FLAGS = ["-O2", "-fPIC", "-std=c++17", "-shared"]

@@ -250,9 +250,11 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
                    item_row0: torch.Tensor, entry_seat: torch.Tensor, entry_q_start: torch.Tensor,
                    entry_start_pos: torch.Tensor, num_q_heads: int, num_kv_heads: int, head_dim: int,
                    scale: float, window: int = 0, splits: int = 1, keys_per_split: int = 0,
-                   row_tiles: int = 1) -> torch.Tensor:
+                   row_tiles: int = 1, pair: bool = False) -> torch.Tensor:
     """bf16 matrix-core attention over the paged cache.  Items are (entry, first query row) pairs
-    of ``16 * row_tiles`` query rows each, row = token_in_step * (nq / nkv) + head_in_group."""
+    of ``16 * row_tiles`` query rows each, row = token_in_step * (nq / nkv) + head_in_group.
+    With ``pair`` one wavefront takes item i and item n-1-i of the list (give the list ordered by
+    keys visited, most first, and every wavefront has about the same work)."""
     tokens = out.shape[0]
     if out.dtype != torch.bfloat16 or q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16:
         raise KernelError("attention_mfma: bfloat16 only")
@@ -278,7 +280,7 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
         int(row_tiles), _dev(entry_seat, "entry_seat", torch.int32), _dev(entry_q_start, "entry_q_start", torch.int32),
         _dev(entry_start_pos, "entry_start_pos", torch.int32), tokens * num_q_heads, num_q_heads,
         num_kv_heads, head_dim, k_cache.shape[2], float(scale), int(window), int(splits),
-        int(keys_per_split), _stream()), "attention_mfma")
+        int(keys_per_split), 1 if pair else 0, _stream()), "attention_mfma")
     return out
 
 

@@ -218,8 +218,9 @@ def items_for(lens, group, gpu, row_tiles=1):
 @pytest.mark.parametrize("nq, nkv, d, page, window", [
     (4, 2, 16, 16, 0), (6, 2, 48, 8, 0), (3, 3, 32, 4, 0), (8, 2, 64, 16, 45), (32, 8, 64, 16, 0),
     (5, 1, 80, 16, 0), (24, 8, 128, 16, 0), (4, 4, 96, 32, 33), (2, 1, 256, 16, 0), (14, 2, 112, 16, 0)])
-@pytest.mark.parametrize("splits, wide", [(1, False), (3, False), (1, True), (2, True)])
-def test_attention_mfma(nq, nkv, d, page, window, splits, wide, gpu):
+@pytest.mark.parametrize("splits, wide, pair", [(1, False, False), (3, False, False), (1, True, False),
+                                                (2, True, False), (1, True, True), (2, False, True)])
+def test_attention_mfma(nq, nkv, d, page, window, splits, wide, pair, gpu):
     assert K.attention_mfma_supported(d, page)
     dev, want, T, stride, scale, lens = attention_case("bfloat16", nq, nkv, d, page, window, ENTRIES, 11, gpu)
     tiles = K.attention_mfma_row_tiles(d, wide)
@@ -232,8 +233,42 @@ def test_attention_mfma(nq, nkv, d, page, window, splits, wide, gpu):
         per = (per + 31) // 32 * 32
     K.attention_mfma(dev["qkv"], stride, out, dev["kc"], dev["vc"], dev["table"], ent, row0,
                      dev["entry_seat"], dev["q_start"], dev["start_pos"], nq, nkv, d, scale, window,
-                     splits, per, tiles)
-    close(out, want, torch.bfloat16, f"attention_mfma splits={splits} tiles={tiles}", tol16=8e-3)
+                     splits, per, tiles, pair)
+    close(out, want, torch.bfloat16, f"attention_mfma splits={splits} tiles={tiles} pair={pair}", tol16=8e-3)
+
+
+@pytest.mark.parametrize("slope", [0.0, 0.35, -0.35, 3.0])
+def test_attention_with_scores_that_keep_rising_or_falling(slope, gpu):
+    """The kernel re-bases its running softmax only when a row's maximum has moved far; scores
+    that climb a little with every key (many small moves), fall, or jump must all give the plain
+    softmax.  Keys are made so that q.k grows by ``slope`` per position."""
+    nq, nkv, d, page, ctx = 4, 2, 64, 16, 600
+    g = torch.Generator().manual_seed(5)
+    q = torch.zeros(1, nq, d)
+    q[..., 0] = 8.0                                    # scale 1/8: the score is k[..., 0]
+    q[..., 1:] = torch.randn(nq, d - 1, generator=g) * 0.05
+    k = torch.randn(ctx, nkv, d, generator=g) * 0.05
+    k[..., 0] = (torch.arange(ctx, dtype=torch.float32) * slope)[:, None]
+    v = torch.randn(ctx, nkv, d, generator=g)
+    q, k, v = (t.to(torch.bfloat16) for t in (q, k, v))
+    want = torch.zeros(1, nq, d, dtype=torch.float64)
+    for h in range(nq):
+        kh = h // (nq // nkv)
+        p = torch.softmax((k[:, kh].double() @ q[0, h].double()) / 8.0, dim=0)
+        want[0, h] = p @ v[:, kh].double()
+    pages = (ctx + page - 1) // page
+    kc = torch.zeros(pages, nkv, page, d, dtype=torch.bfloat16)
+    vc = torch.zeros(pages, nkv, d, page, dtype=torch.bfloat16)
+    for t in range(ctx):
+        kc[t // page, :, t % page, :] = k[t]
+        vc[t // page, :, :, t % page] = v[t]
+    table = torch.arange(pages, dtype=torch.int32).view(1, pages).to(gpu)
+    i32 = lambda *x: torch.tensor(x, dtype=torch.int32, device=gpu)
+    for splits, per in ((1, 0), (4, 160)):
+        out = torch.full((1, nq * d), float("nan"), dtype=torch.bfloat16, device=gpu)
+        K.attention_mfma(q.view(1, nq * d).to(gpu), nq * d, out, kc.to(gpu), vc.to(gpu), table, i32(0), i32(0),
+                         i32(0), i32(0, 1), i32(ctx - 1), nq, nkv, d, 1 / 8.0, 0, splits, per, 1)
+        close(out.view(1, nq, d), want, torch.bfloat16, f"slope {slope} splits {splits}", tol16=1e-2)
 
 
 def test_attention_finds_one_far_key_among_hundreds(gpu):
