@@ -84,3 +84,27 @@ def write_random_model(model_dir: str, config_dict: Mapping[str, Any], seed: int
     state = random_state_dict(specs, seed, _DTYPES[dtype_name])
     save_file(state, os.path.join(model_dir, "model.safetensors"), metadata={"format": "pt"})
     return model_dir
+
+
+def main(argv=None) -> int:
+    """``python -m kv_cache_optimization_for_llm_amd.weights.random_init --config config.json
+    --out DIR --seed 0``: writes a model folder with random weights for a configuration."""
+    import argparse
+    import json
+
+    ap = argparse.ArgumentParser(description="write a model folder (config.json, model.safetensors) "
+                                             "with seeded random weights")
+    ap.add_argument("--config", required=True, help="a config.json of the architecture (its own keys)")
+    ap.add_argument("--out", required=True, help="folder to create")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--dtype", choices=sorted(_DTYPES), default=None,
+                    help="storage type of the tensors (default: the configuration's torch_dtype)")
+    args = ap.parse_args(argv)
+    with open(args.config) as f:
+        cfg = json.load(f)
+    print(write_random_model(args.out, cfg, args.seed, args.dtype))
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())

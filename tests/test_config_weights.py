@@ -161,3 +161,14 @@ def test_dtype_rule():
     assert target_dtype(bf, "matrix", f32) == f32        # widened exactly for the 32-bit path
     assert target_dtype(f32, "vector", bf) == f32        # stored in 32-bit stays so
     assert target_dtype(torch.int64, "table", bf) == torch.int32
+
+
+def test_random_weights_command_writes_the_same_folder_as_the_function(tmp_path):
+    from kv_cache_optimization_for_llm_amd.weights import random_init
+    cfg_file = tmp_path / "c.json"
+    cfg_file.write_text(json.dumps(TINY_B))
+    assert random_init.main(["--config", str(cfg_file), "--out", str(tmp_path / "cmd"), "--seed", "5"]) == 0
+    write_random_model(str(tmp_path / "fn"), TINY_B, 5)
+    a = (tmp_path / "cmd" / "model.safetensors").read_bytes()
+    b = (tmp_path / "fn" / "model.safetensors").read_bytes()
+    assert a == b and read_config_json(str(tmp_path / "cmd")) == read_config_json(str(tmp_path / "fn"))
