@@ -65,6 +65,7 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
                       const bf16_t *__restrict__ q, int q_row_stride,
                       const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
                       const int *__restrict__ block_table, int max_blocks,
+                      const int *__restrict__ item_meta,
                       const int *__restrict__ item_entry, const int *__restrict__ item_row0,
                       const int *__restrict__ entry_seat, const int *__restrict__ entry_q_start,
                       const int *__restrict__ entry_start_pos, int num_q_heads, int num_kv_heads,
@@ -76,13 +77,27 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
     const int lane = threadIdx.x, r = lane & 15, g = lane >> 4;
     const int G = num_q_heads / num_kv_heads;
 
-    // everything about the item is uniform over the wavefront: keep it in scalar registers
-    const int e = __builtin_amdgcn_readfirstlane(item_entry[item]);
-    const int row0 = __builtin_amdgcn_readfirstlane(item_row0[item]);
-    const int q_start = __builtin_amdgcn_readfirstlane(entry_q_start[e]);
-    const int q_len = __builtin_amdgcn_readfirstlane(entry_q_start[e + 1]) - q_start;
-    const int start_pos = __builtin_amdgcn_readfirstlane(entry_start_pos[e]);
-    const int *bt = block_table + (size_t)__builtin_amdgcn_readfirstlane(entry_seat[e]) * max_blocks;
+    // Everything about the item is uniform over the wavefront: keep it in scalar registers.  Every
+    // dependent load at the start of a short kernel costs a trip to memory, so the caller may
+    // hand over all of it in one record per item (item_meta: q_start, q_len, start_pos, seat,
+    // row0, 3 unused) instead of the chain item -> entry -> entry's arrays.
+    int row0, q_start, q_len, start_pos, seat;
+    if (item_meta != nullptr) {
+        const int *meta = item_meta + (size_t)__builtin_amdgcn_readfirstlane(item) * 8;
+        q_start = __builtin_amdgcn_readfirstlane(meta[0]);
+        q_len = __builtin_amdgcn_readfirstlane(meta[1]);
+        start_pos = __builtin_amdgcn_readfirstlane(meta[2]);
+        seat = __builtin_amdgcn_readfirstlane(meta[3]);
+        row0 = __builtin_amdgcn_readfirstlane(meta[4]);
+    } else {
+        const int e = __builtin_amdgcn_readfirstlane(item_entry[item]);
+        row0 = __builtin_amdgcn_readfirstlane(item_row0[item]);
+        q_start = __builtin_amdgcn_readfirstlane(entry_q_start[e]);
+        q_len = __builtin_amdgcn_readfirstlane(entry_q_start[e + 1]) - q_start;
+        start_pos = __builtin_amdgcn_readfirstlane(entry_start_pos[e]);
+        seat = __builtin_amdgcn_readfirstlane(entry_seat[e]);
+    }
+    const int *bt = block_table + (size_t)seat * max_blocks;
     const int M = q_len * G;
 
     // per row tile: this lane's query row
@@ -368,6 +383,7 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
                       const bf16_t *__restrict__ q, int q_row_stride,
                       const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
                       const int *__restrict__ block_table, int max_blocks,
+                      const int *__restrict__ item_meta,
                       const int *__restrict__ item_entry, const int *__restrict__ item_row0,
                       const int *__restrict__ entry_seat, const int *__restrict__ entry_q_start,
                       const int *__restrict__ entry_start_pos, int num_q_heads, int num_kv_heads,
@@ -375,19 +391,22 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
     const int kvh = blockIdx.x % num_kv_heads, split = blockIdx.z;
     const int w = blockIdx.x / num_kv_heads;
     attention_item<D, RT, FAST>(out, part_o, part_ml, q, q_row_stride, k_cache, v_cache, block_table, max_blocks,
-                                item_entry, item_row0, entry_seat, entry_q_start, entry_start_pos, num_q_heads,
+                                item_meta, item_entry, item_row0, entry_seat, entry_q_start, entry_start_pos, num_q_heads,
                                 num_kv_heads, page_size, scale, window, splits, keys_per_split, w, kvh, split);
     const int other = num_items - 1 - w;
     if (pair && other > w)
         attention_item<D, RT, FAST>(out, part_o, part_ml, q, q_row_stride, k_cache, v_cache, block_table, max_blocks,
-                                    item_entry, item_row0, entry_seat, entry_q_start, entry_start_pos, num_q_heads,
+                                    item_meta, item_entry, item_row0, entry_seat, entry_q_start, entry_start_pos, num_q_heads,
                                     num_kv_heads, page_size, scale, window, splits, keys_per_split, other, kvh, split);
 }
 
 // out[row, :] = sum_s o_s * exp(m_s - M) / sum_s l_s * exp(m_s - M),  M = max_s m_s.
 // One wavefront per row: lanes first own splits (max and denominator by wave reduction, the
-// weights go to LDS), then own value dimensions and add the weighted partials.
+// weights go to LDS), then own value dimensions and add the weighted partials.  The partials of
+// the first MERGE_EARLY splits are loaded before the weights are known, so that the kernel makes
+// one trip to memory, not two.
 #define MERGE_MAX_SPLITS 256
+#define MERGE_EARLY 32
 __global__ void __launch_bounds__(KVA_WAVE)
 attention_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o,
                        const float *__restrict__ part_ml, int head_dim, int splits) {
@@ -395,6 +414,12 @@ attention_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_
     const size_t row = blockIdx.x;
     const int lane = threadIdx.x;
     const float2 *ml = reinterpret_cast<const float2 *>(part_ml) + row * splits;
+    const float *po = part_o + row * splits * head_dim;
+    float early[MERGE_EARLY];
+    const bool j0_ok = lane < head_dim;
+#pragma unroll
+    for (int s = 0; s < MERGE_EARLY; ++s)
+        early[s] = (j0_ok && s < splits) ? po[(size_t)s * head_dim + lane] : 0.f;
     float M = -INFINITY;
     for (int s = lane; s < splits; s += KVA_WAVE) M = fmaxf(M, ml[s].x);
     M = wave_max(M);
@@ -408,11 +433,18 @@ attention_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_
     denom = wave_sum(denom);
     __syncthreads();
     const float inv = 1.f / denom;
-    const float *po = part_o + row * splits * head_dim;
     for (int j = lane; j < head_dim; j += KVA_WAVE) {
         float acc = 0.f;
+        int s0 = 0;
+        if (j == lane) {                                   // this lane's first dimension: loaded already
+            const int n = splits < MERGE_EARLY ? splits : MERGE_EARLY;
+#pragma unroll
+            for (int s = 0; s < MERGE_EARLY; ++s)
+                if (s < n) acc += early[s] * w_s[s];
+            s0 = n;
+        }
 #pragma unroll 8
-        for (int s = 0; s < splits; ++s) acc += po[(size_t)s * head_dim + j] * w_s[s];
+        for (int s = s0; s < splits; ++s) acc += po[(size_t)s * head_dim + j] * w_s[s];
         out[row * head_dim + j].bits = float_to_bf16_bits(acc * inv);
     }
 }
@@ -436,8 +468,8 @@ extern "C" int kva_attention_mfma_row_tiles(int head_dim, int wide) {
 
 extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, const void *q,
                                   int q_row_stride, const void *k_cache, const void *v_cache,
-                                  const int *block_table, int max_blocks, const int *item_entry,
-                                  const int *item_row0, int num_items, int row_tiles,
+                                  const int *block_table, int max_blocks, const int *item_meta,
+                                  const int *item_entry, const int *item_row0, int num_items, int row_tiles,
                                   const int *entry_seat, const int *entry_q_start,
                                   const int *entry_start_pos, int total_rows, int num_q_heads,
                                   int num_kv_heads, int head_dim, int page_size, float scale, int window,
@@ -466,7 +498,8 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
 #define LAUNCH(DD, RR, FF)                                                                      \
     hipLaunchKernelGGL((attention_mfma_kernel<DD, RR, FF>), grid, block, 0, stream, (bf16_t *)out, \
                        part_o, part_ml, (const bf16_t *)q, q_row_stride, (const bf16_t *)k_cache, \
-                       (const bf16_t *)v_cache, block_table, max_blocks, item_entry, item_row0,  \
+                       (const bf16_t *)v_cache, block_table, max_blocks, item_meta, item_entry,  \
+                       item_row0,                                                               \
                        entry_seat, entry_q_start, entry_start_pos, num_q_heads, num_kv_heads,    \
                        page_size, scale, window, splits, keys_per_split, num_items, pair)
 #define CASE(DD, WIDE)                                                                          \

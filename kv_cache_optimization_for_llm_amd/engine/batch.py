@@ -53,15 +53,24 @@ class StepBatch:
     max_context: int = 0
     logits_for_all_rows: bool = False    # logit_rows is exactly 0, 1, ..., T-1
     feedback: torch.Tensor = None        # device int32: tokens that negative token_ids stand for
+    meta_provider: object = None         # callable(group, row_tiles) -> attention items, or None
     _items: Dict[tuple, tuple] = field(default_factory=dict, repr=False)
 
     def attention_items(self, group: int, row_tiles: int = 1):
         """Work items of the matrix-core attention kernel for a query-head group size: (entry,
         first row) of every ``16 * row_tiles`` query rows, row = token_in_step * group +
         head_in_group; ordered by the number of keys an item visits, most first (when the
-        entries' start positions are known on the host)."""
+        entries' start positions are known on the host).  Returns ``(entry, row0, meta)``;
+        ``meta`` ``[items, 8]`` repeats per item what the kernel would otherwise look up through
+        the entry (q_start, q_len, start_pos, seat, row0), or is ``None`` when the host does not
+        know it."""
         key = (group, row_tiles)
         if key not in self._items:
+            if self.meta_provider is not None:
+                made = self.meta_provider(group, row_tiles)
+                if made is not None:
+                    self._items[key] = made
+                    return made
             lens = np.diff(self.h_entry_q_start)
             ent, row0 = [], []
             for e, n in enumerate(lens):
@@ -69,17 +78,27 @@ class StepBatch:
                 ent.append(np.full(starts.shape[0], e, dtype=np.int32))
                 row0.append(starts)
             ent, row0 = np.concatenate(ent), np.concatenate(row0)
-            if self.h_entry_start_pos is not None and ent.shape[0] > 1:
-                # most keys first: the kernel hands out items in list order (and may give a
-                # wavefront the i-th and the i-th last), so the long ones should start early
-                last_row = np.minimum(row0 + 16 * row_tiles, lens[ent] * group) - 1
-                keys = self.h_entry_start_pos[ent] + last_row // group + 1
-                order = np.argsort(-keys, kind="stable")
-                ent, row0 = ent[order], row0[order]
-            both = np.concatenate([ent, row0])
-            dev = torch.from_numpy(both).to(self.token_ids.device, non_blocking=True)
-            n = both.shape[0] // 2
-            self._items[key] = (dev[:n], dev[n:])
+            n = ent.shape[0]
+            parts = [ent, row0]
+            known = self.h_entry_start_pos is not None and self.h_entry_seat is not None
+            if known:
+                if n > 1:
+                    # most keys first: the kernel hands out items in list order (and may give a
+                    # wavefront the i-th and the i-th last), so the long ones should start early
+                    last_row = np.minimum(row0 + 16 * row_tiles, lens[ent] * group) - 1
+                    keys = self.h_entry_start_pos[ent] + last_row // group + 1
+                    order = np.argsort(-keys, kind="stable")
+                    ent, row0 = ent[order], row0[order]
+                    parts = [ent, row0]
+                meta = np.zeros((n, 8), dtype=np.int32)
+                meta[:, 0] = self.h_entry_q_start[:-1][ent]
+                meta[:, 1] = lens[ent]
+                meta[:, 2] = self.h_entry_start_pos[ent]
+                meta[:, 3] = self.h_entry_seat[ent]
+                meta[:, 4] = row0
+                parts.append(meta.reshape(-1))
+            dev = torch.from_numpy(np.concatenate(parts)).to(self.token_ids.device, non_blocking=True)
+            self._items[key] = (dev[:n], dev[n:2 * n], dev[2 * n:].view(n, 8) if known else None)
         return self._items[key]
 
 

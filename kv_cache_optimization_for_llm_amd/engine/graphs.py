@@ -37,9 +37,13 @@ class _DecodeSlot:
         self.n, self.bucket = n, bucket
         # layout of the int32 staging buffer: token_ids, positions, tok_seat, entry_start_pos,
         # then one slot mapping per cache group; each n long
-        self.fields = 4 + num_groups
+        # ... and, last, one record of 8 per entry for the attention kernel (q_start, q_len,
+        # start_pos, seat, row0, 0, 0, 0): with at most 16 query heads per kv head a decoded
+        # token is one work item, so the records can be written here every step
+        self.fields = 4 + num_groups + 8
         self.staging = torch.zeros(self.fields * n, dtype=torch.int32, pin_memory=True)
         self.dev = torch.zeros(self.fields * n, dtype=torch.int32, device=device)
+        self.meta_at = (4 + num_groups) * n
         self.const = torch.cat([torch.arange(n + 1, dtype=torch.int32),          # entry_q_start
                                 torch.arange(n, dtype=torch.int32)]).to(device)   # logit rows
         v = lambda i: self.dev[i * n:(i + 1) * n]
@@ -52,6 +56,13 @@ class _DecodeSlot:
         # attention work items depend on this array only, so they are the same every step; the
         # eager warm-up run uploads them, the captured run finds them cached
         self.batch.h_entry_q_start = np.arange(n + 1, dtype=np.int32)
+        items = torch.arange(n, dtype=torch.int32).to(device)
+        zeros = torch.zeros(n, dtype=torch.int32, device=device)
+        meta = self.dev[self.meta_at:self.meta_at + 8 * n].view(n, 8)
+        self.batch.meta_provider = lambda group, row_tiles: \
+            (items, zeros, meta) if group <= 16 and row_tiles == 1 else None
+        m = self.staging.numpy()[self.meta_at:self.meta_at + 8 * n].reshape(n, 8)
+        m[:, 0], m[:, 1] = np.arange(n), 1
         self.copied = torch.cuda.Event()
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None
@@ -65,6 +76,8 @@ class _DecodeSlot:
         st[0:n], st[n:2 * n], st[2 * n:3 * n], st[3 * n:4 * n] = tokens, positions, seats, positions
         for g, sm in enumerate(slot_maps):
             st[(4 + g) * n:(5 + g) * n] = sm
+        m = st[self.meta_at:self.meta_at + 8 * n].reshape(n, 8)
+        m[:, 2], m[:, 3] = positions, seats
         self.dev.copy_(self.staging, non_blocking=True)
         self.copied.record()
 

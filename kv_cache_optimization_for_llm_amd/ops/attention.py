@@ -47,7 +47,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
             # prompt portions: two row tiles per wave, so each key and value loaded serves 32
             # query rows; whole key ranges as long as that still gives a wave per SIMD
             tiles = K.attention_mfma_row_tiles(head_dim, True)
-            item_entry, item_row0 = batch.attention_items(group, tiles)
+            item_entry, item_row0, meta = batch.attention_items(group, tiles)
             if item_entry.shape[0] * num_kv_heads < _WIDE_MIN_WAVES:
                 tiles = 1
             else:
@@ -55,12 +55,12 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
                 # does about the average; worth it while every SIMD still gets a wavefront
                 pair = item_entry.shape[0] * num_kv_heads >= _PAIR_MIN_WAVES
         if tiles == 1:
-            item_entry, item_row0 = batch.attention_items(group, 1)
+            item_entry, item_row0, meta = batch.attention_items(group, 1)
             splits, per = choose_splits(item_entry.shape[0], num_kv_heads, batch.max_context)
         return K.attention_mfma(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table,
                                 item_entry, item_row0, batch.entry_seat, batch.entry_q_start,
                                 batch.entry_start_pos, num_q_heads, num_kv_heads, head_dim, scale,
-                                window, splits, per, tiles, pair)
+                                window, splits, per, tiles, pair, meta)
     return K.attention_rowwise(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table,
                                batch.tok_seat, batch.positions, num_q_heads, num_kv_heads,
                                head_dim, scale, window)

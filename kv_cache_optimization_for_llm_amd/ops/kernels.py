@@ -250,11 +250,14 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
                    item_row0: torch.Tensor, entry_seat: torch.Tensor, entry_q_start: torch.Tensor,
                    entry_start_pos: torch.Tensor, num_q_heads: int, num_kv_heads: int, head_dim: int,
                    scale: float, window: int = 0, splits: int = 1, keys_per_split: int = 0,
-                   row_tiles: int = 1, pair: bool = False) -> torch.Tensor:
+                   row_tiles: int = 1, pair: bool = False,
+                   item_meta: Optional[torch.Tensor] = None) -> torch.Tensor:
     """bf16 matrix-core attention over the paged cache.  Items are (entry, first query row) pairs
     of ``16 * row_tiles`` query rows each, row = token_in_step * (nq / nkv) + head_in_group.
     With ``pair`` one wavefront takes item i and item n-1-i of the list (give the list ordered by
-    keys visited, most first, and every wavefront has about the same work)."""
+    keys visited, most first, and every wavefront has about the same work).  ``item_meta``
+    ``[items, 8]`` int32 (q_start, q_len, start_pos, seat, row0, 0, 0, 0 per item) saves the
+    kernel the chain of lookups item -> entry -> entry arrays; it must say the same as they do."""
     tokens = out.shape[0]
     if out.dtype != torch.bfloat16 or q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16:
         raise KernelError("attention_mfma: bfloat16 only")
@@ -268,6 +271,8 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
         raise KernelError("attention_mfma: index arrays do not fit each other")
     if q.data_ptr() % 16 or q_row_stride < num_q_heads * head_dim:
         raise KernelError("attention_mfma: q view is misaligned or its stride is too small")
+    if item_meta is not None and item_meta.shape != (n_items, 8):
+        raise KernelError("attention_mfma: item_meta must be [items, 8]")
     part_o = part_ml = None
     if splits > 1:
         part_o = torch.empty((tokens * num_q_heads, splits, head_dim), dtype=torch.float32, device=out.device)
@@ -276,6 +281,7 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
         _dev(out, "out"), _opt(part_o, "part_o"), _opt(part_ml, "part_ml"),
         _dev(q, "q", contiguous=False), q_row_stride, _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
         _dev(block_table, "block_table", torch.int32), block_table.shape[1],
+        _opt(item_meta, "item_meta", torch.int32),
         _dev(item_entry, "item_entry", torch.int32), _dev(item_row0, "item_row0", torch.int32), n_items,
         int(row_tiles), _dev(entry_seat, "entry_seat", torch.int32), _dev(entry_q_start, "entry_q_start", torch.int32),
         _dev(entry_start_pos, "entry_start_pos", torch.int32), tokens * num_q_heads, num_q_heads,

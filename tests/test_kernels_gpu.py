@@ -235,6 +235,16 @@ def test_attention_mfma(nq, nkv, d, page, window, splits, wide, pair, gpu):
                      dev["entry_seat"], dev["q_start"], dev["start_pos"], nq, nkv, d, scale, window,
                      splits, per, tiles, pair)
     close(out, want, torch.bfloat16, f"attention_mfma splits={splits} tiles={tiles} pair={pair}", tol16=8e-3)
+    # the same with one record per item instead of the lookups through the entry: bitwise equal
+    e = ent.cpu().long()
+    qs, sp, seat = dev["q_start"].cpu(), dev["start_pos"].cpu(), dev["entry_seat"].cpu()
+    meta = torch.zeros((e.shape[0], 8), dtype=torch.int32)
+    meta[:, 0], meta[:, 1], meta[:, 2], meta[:, 3], meta[:, 4] = qs[e], qs[e + 1] - qs[e], sp[e], seat[e], row0.cpu()
+    out2 = torch.full_like(out, float("nan"))
+    K.attention_mfma(dev["qkv"], stride, out2, dev["kc"], dev["vc"], dev["table"], ent, row0,
+                     dev["entry_seat"], dev["q_start"], dev["start_pos"], nq, nkv, d, scale, window,
+                     splits, per, tiles, pair, meta.to(gpu))
+    assert torch.equal(out2, out)
 
 
 @pytest.mark.parametrize("slope", [0.0, 0.35, -0.35, 3.0])
