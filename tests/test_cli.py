@@ -50,3 +50,25 @@ def test_served_tokens_are_the_same_in_both_cache_modes(model_dirs, tmp_path, gp
     assert results["paged"]["checksums"] == results["contiguous"]["checksums"]
     assert results["paged"]["engine_config"]["mechanism"] == "paged"
     assert results["contiguous"]["engine_config"]["reserve_policy"] == "oracle"
+
+
+@pytest.mark.gpu
+def test_sweep_reports_both_cache_modes_on_a_small_shape(model_dirs, tmp_path, gpu, capsys):
+    """The sweep command on a tiny configuration: every request finishes with its budget, the
+    contiguous cache reserves more than it holds (whole reservations), the paged cache about what
+    it holds, and with a small pool pages are used again."""
+    from kv_cache_optimization_for_llm_amd.cli import sweep
+    cfg = os.path.join(model_dirs["A"], "config.json")
+    out = tmp_path / "sweep.jsonl"
+    assert sweep.main(["--shapes", cfg, "--batches", "3,6", "--cache-modes", "paged,contiguous", "--prompt-len", "40",
+                       "--prompt-min", "5", "--workload", "mixed", "--new-tokens", "12", "--max-seqs", "3",
+                       "--reserve-policy", "pow2", "--out", str(out)]) == 0
+    lines = [json.loads(l) for l in out.read_text().splitlines()]
+    assert [(l["cache_mode"], l["batch"]) for l in lines] == [("paged", 3), ("paged", 6), ("contiguous", 3), ("contiguous", 6)]
+    for l in lines:
+        assert l["requests_done"] == l["batch"] and l["tokens_emitted"] == 12 * l["batch"]
+        assert l["finish_reasons"] == {"length": l["batch"]} and l["decode_tok_s"] > 0
+        assert l["peak_kv_tokens_reserved"] >= l["peak_kv_tokens_live"] > 0
+    paged, contiguous = lines[1], lines[3]
+    assert paged["reserved_over_live"] < contiguous["reserved_over_live"]
+    assert paged["pages_reused"] > 0                  # six requests through three seats
