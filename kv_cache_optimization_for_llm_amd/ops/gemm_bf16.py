@@ -1,9 +1,10 @@
 """bf16 matrix products: picks the kernel for a shape.
 
 ``linear_bf16(x, w, out)`` computes ``out = x @ w^T`` with fp32 accumulation.  ``out`` may be
-bf16 or fp32.  Up to 16 rows (decode steps, short portions) take the hand-written matrix-core
-kernel that streams a tiled copy of the weight once (``csrc/gemm_skinny.hip``).  Other shapes go to the vendor
-GEMM library through ``torch.matmul``, which is where the reference's engine uses cuBLAS.
+bf16 or fp32.  Few rows (decode steps, short portions; how few depends on the matrix, see
+``use_skinny``) take the hand-written matrix-core kernel that streams a tiled copy of the weight
+once (``csrc/gemm_skinny.hip``).  Other shapes go to the vendor GEMM library through
+``torch.matmul``, which is where the reference's engine uses cuBLAS.
 """
 from __future__ import annotations
 
@@ -12,14 +13,32 @@ import torch
 from . import kernels as K
 
 
-# Measured on MI355X at the Llama-3.2-1B shapes: up to 16 rows the few-rows kernel beats the vendor
-# GEMM (weights streamed at 5+ TB/s, norms and activation fused); from 32 rows on the vendor
-# GEMM's tiles win because the few-rows kernel re-reads X once per 16 rows of W.
-SKINNY_MAX_ROWS = 16
+# Measured on MI355X at the Llama-3.2-1B shapes with weights that are not in any cache, whole
+# decode steps timed:
+# * up to 16 rows the few-rows kernel beats the vendor GEMM everywhere (weights streamed once at
+#   5+ TB/s, norms, rotation, activation and residual fused);
+# * up to 32 rows it still wins for small matrices (the Q/K/V and output projections), where a
+#   launch costs more than the product and its epilogues replace 5 us kernels, and for matrices
+#   with many more rows than columns (the joined gate/up matrix: many workgroups, SwiGLU fused);
+#   not for the down projection (few row tiles, long K: the vendor GEMM's split wins), and at 64
+#   rows the vendor GEMM wins everywhere because the few-rows kernel re-reads X once per 16 rows of W;
+# * the vocabulary-sized product (4 row tiles of W per wave share each X fragment, fp32 output
+#   without a cast) wins up to 48 rows.
+SKINNY_MAX_ROWS = 16            # every shape
+SKINNY_MID_ROWS = 32            # small or tall matrices
+SKINNY_MID_ELEMENTS = 1 << 23
+SKINNY_WIDE_ROWS = 48           # vocabulary-sized matrices
+SKINNY_WIDE_N = 32768
 
 
 def use_skinny(m: int, n: int, k: int) -> bool:
-    return m <= SKINNY_MAX_ROWS and K.gemm_skinny_supported(m, n, k)
+    if not K.gemm_skinny_supported(m, n, k):
+        return False
+    if m <= SKINNY_MAX_ROWS:
+        return True
+    if m <= SKINNY_MID_ROWS and (n * k <= SKINNY_MID_ELEMENTS or n >= 4 * k):
+        return True
+    return m <= SKINNY_WIDE_ROWS and n >= SKINNY_WIDE_N
 
 
 def linear_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, tiled=None) -> torch.Tensor:
