@@ -1,0 +1,30 @@
+// Register fragments of the bf16 matrix-core attention kernels (gfx950).
+#pragma once
+#include "common.h"
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 b16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 b16x2 __attribute__((ext_vector_type(2)));
+
+// 8 bf16 = one operand of mfma_f32_16x16x32_bf16
+union Frag8 {
+    b16x8 v;
+    uint4 u4;
+    uint2 u2[2];
+    uint16_t h[8];
+    b16x2 p2[4];
+};
+
+// 4 bf16 = one operand of mfma_f32_16x16x16bf16_1k
+union Frag4 {
+    s16x4 v;
+    uint2 u2;
+    uint16_t h[4];
+};
+
+// two floats -> two bf16, round to nearest even (one v_cvt_pk_bf16_f32)
+__device__ inline b16x2 pack_bf16(float a, float b) {
+    return __builtin_convertvector(f32x2{a, b}, b16x2);
+}

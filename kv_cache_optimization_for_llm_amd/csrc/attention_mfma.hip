@@ -32,32 +32,9 @@
 // Reference: same recurrence as paged_attention/src/kernels.cu:150-219 and the tiled prefill
 // kernel base/src/kernels.cu:361-466, which work one key at a time on CUDA cores.
 #include "common.h"
+#include "attention_frag.h"
 #include <type_traits>
 #include <math.h>
-
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef __bf16 b16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef __bf16 b16x2 __attribute__((ext_vector_type(2)));
-
-union Frag8 {
-    b16x8 v;
-    uint4 u4;
-    uint2 u2[2];
-    uint16_t h[8];
-    b16x2 p2[4];
-};
-
-// two floats -> two bf16, round to nearest even (one v_cvt_pk_bf16_f32)
-__device__ inline b16x2 pack_bf16(float a, float b) {
-    return __builtin_convertvector(f32x2{a, b}, b16x2);
-}
-union Frag4 {
-    s16x4 v;
-    uint2 u2;
-    uint16_t h[4];
-};
 
 template <int D, int RT, bool FAST>
 __device__ __forceinline__ void

@@ -50,30 +50,34 @@ class StepBatch:
     h_entry_q_start: np.ndarray = field(repr=False, default=None)
     h_entry_start_pos: np.ndarray = field(repr=False, default=None)
     max_q_len: int = 0
+    min_q_len: int = 0
     max_context: int = 0
     logits_for_all_rows: bool = False    # logit_rows is exactly 0, 1, ..., T-1
     feedback: torch.Tensor = None        # device int32: tokens that negative token_ids stand for
     meta_provider: object = None         # callable(group, row_tiles) -> attention items, or None
     _items: Dict[tuple, tuple] = field(default_factory=dict, repr=False)
 
-    def attention_items(self, group: int, row_tiles: int = 1):
-        """Work items of the matrix-core attention kernel for a query-head group size: (entry,
+    def attention_items(self, group: int, row_tiles: int = 1, which: str = "all"):
+        """Work items of the matrix-core attention kernels for a query-head group size: (entry,
         first row) of every ``16 * row_tiles`` query rows, row = token_in_step * group +
         head_in_group; ordered by the number of keys an item visits, most first (when the
-        entries' start positions are known on the host).  Returns ``(entry, row0, meta)``;
-        ``meta`` ``[items, 8]`` repeats per item what the kernel would otherwise look up through
-        the entry (q_start, q_len, start_pos, seat, row0), or is ``None`` when the host does not
-        know it."""
-        key = (group, row_tiles)
+        entries' start positions are known on the host).  ``which`` takes all entries, only the
+        ``"long"`` ones (more than 16 query rows: prompt portions) or only the ``"short"`` ones
+        (decoded tokens).  Returns ``(entry, row0, meta)``; ``meta`` ``[items, 8]`` repeats per
+        item what the kernel would otherwise look up through the entry (q_start, q_len,
+        start_pos, seat, row0), or is ``None`` when the host does not know it."""
+        key = (group, row_tiles, which)
         if key not in self._items:
-            if self.meta_provider is not None:
+            if self.meta_provider is not None and which == "all":
                 made = self.meta_provider(group, row_tiles)
                 if made is not None:
                     self._items[key] = made
                     return made
             lens = np.diff(self.h_entry_q_start)
-            ent, row0 = [], []
+            ent, row0 = [np.zeros(0, np.int32)], [np.zeros(0, np.int32)]
             for e, n in enumerate(lens):
+                if which != "all" and (int(n) * group > 16) != (which == "long"):
+                    continue
                 starts = np.arange(0, int(n) * group, 16 * row_tiles, dtype=np.int32)
                 ent.append(np.full(starts.shape[0], e, dtype=np.int32))
                 row0.append(starts)
@@ -100,6 +104,16 @@ class StepBatch:
             dev = torch.from_numpy(np.concatenate(parts)).to(self.token_ids.device, non_blocking=True)
             self._items[key] = (dev[:n], dev[n:2 * n], dev[2 * n:].view(n, 8) if known else None)
         return self._items[key]
+
+    def mean_keys_of_long_entries(self) -> float:
+        """Average number of keys a query token of the prompt portions visits (host estimate)."""
+        lens = np.diff(self.h_entry_q_start).astype(np.float64)
+        if self.h_entry_start_pos is None:
+            return float(self.max_context)
+        long = lens > 1
+        if not long.any():
+            return 0.0
+        return float(((self.h_entry_start_pos[long] + (lens[long] + 1) / 2) * lens[long]).sum() / lens[long].sum())
 
 
 def _align(n: int, a: int = 4) -> int:
@@ -158,6 +172,6 @@ def build_batch(seats: Sequence[int], starts: Sequence[int], token_lists: Sequen
         h_positions=positions, h_tok_seat=tok_seat, h_entry_seat=segs["entry_seat"],
         h_entry_q_start=q_start, h_entry_start_pos=segs["entry_start_pos"],
         logits_for_all_rows=rows == list(range(T)),
-        max_q_len=max(lens) if lens else 0,
+        max_q_len=max(lens) if lens else 0, min_q_len=min(lens) if lens else 0,
         max_context=max((s + n for s, n in zip(starts, lens)), default=0),
     )

@@ -52,7 +52,7 @@ class _DecodeSlot:
             token_ids=v(0), positions=v(1), tok_seat=v(2), logit_rows=self.const[n + 1:],
             slot_mapping=[v(4 + g) for g in range(num_groups)],
             entry_seat=v(2), entry_q_start=self.const[:n + 1], entry_start_pos=v(3),
-            max_q_len=1, max_context=bucket, logits_for_all_rows=True, feedback=feedback)
+            max_q_len=1, min_q_len=1, max_context=bucket, logits_for_all_rows=True, feedback=feedback)
         # attention work items depend on this array only, so they are the same every step; the
         # eager warm-up run uploads them, the captured run finds them cached
         self.batch.h_entry_q_start = np.arange(n + 1, dtype=np.int32)

@@ -16,6 +16,12 @@ _MIN_KEYS_PER_SPLIT = 128
 # wide items (two row tiles per wave) are used when they alone give this many waves
 _WIDE_MIN_WAVES = 1024
 _PAIR_MIN_WAVES = 2048      # two items per wavefront once that still leaves a wavefront per SIMD
+# The workgroup kernel (128 query rows share each key block through LDS) pays one barrier per key
+# block: it wins once there are three workgroups per compute unit, or one per unit when the rows
+# visit thousands of keys each (measured: 2,048-token prompt from position 0 a tie, 4,096 1.5x).
+_LDS_MIN_GROUPS = 256
+_LDS_MANY_GROUPS = 768
+_LDS_MIN_MEAN_KEYS = 2048
 
 
 def choose_splits(num_items: int, num_kv_heads: int, max_context: int) -> tuple:
@@ -35,32 +41,61 @@ def choose_splits(num_items: int, num_kv_heads: int, max_context: int) -> tuple:
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads: int,
                     num_kv_heads: int, head_dim: int, scale: float, window: int = 0) -> torch.Tensor:
     """Causal GQA attention of the step's tokens over the paged cache.  ``qkv`` is the fused
-    projection output ``[T, (nq + 2 nkv) d]`` whose first ``nq * d`` columns are the (already
-    position-encoded) queries; keys and values are read from ``kv``."""
+    projection output ``[T, (nq + 2 nkv) d]`` (or just its Q part) whose first ``nq * d`` columns
+    are the (already position-encoded) queries; keys and values are read from ``kv``.
+
+    bf16 runs on the matrix cores.  Decoded tokens (at most 16 query rows per kv head) take the
+    one-wavefront kernel with their keys split over wavefronts; prompt portions take the
+    workgroup kernel that shares key blocks through LDS when there is enough of them to fill the
+    chip, else the one-wavefront kernel with two row tiles.  A step that holds both is two
+    launches, each over its own entries."""
     if kv is None:
         raise K.KernelError("paged_attention: the mixer has no cache view")
-    if qkv.dtype == torch.bfloat16 and K.attention_mfma_supported(head_dim, kv.page_size) \
-            and qkv.shape[1] % 8 == 0:
-        group = num_q_heads // num_kv_heads
-        tiles, splits, per, pair = 1, 1, 0, False
-        if batch.max_q_len * group > 16:
-            # prompt portions: two row tiles per wave, so each key and value loaded serves 32
-            # query rows; whole key ranges as long as that still gives a wave per SIMD
-            tiles = K.attention_mfma_row_tiles(head_dim, True)
-            item_entry, item_row0, meta = batch.attention_items(group, tiles)
-            if item_entry.shape[0] * num_kv_heads < _WIDE_MIN_WAVES:
-                tiles = 1
-            else:
-                # items come ordered by work: a wavefront that takes the i-th and the i-th last
-                # does about the average; worth it while every SIMD still gets a wavefront
-                pair = item_entry.shape[0] * num_kv_heads >= _PAIR_MIN_WAVES
-        if tiles == 1:
-            item_entry, item_row0, meta = batch.attention_items(group, 1)
-            splits, per = choose_splits(item_entry.shape[0], num_kv_heads, batch.max_context)
-        return K.attention_mfma(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table,
-                                item_entry, item_row0, batch.entry_seat, batch.entry_q_start,
-                                batch.entry_start_pos, num_q_heads, num_kv_heads, head_dim, scale,
-                                window, splits, per, tiles, pair, meta)
-    return K.attention_rowwise(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table,
-                               batch.tok_seat, batch.positions, num_q_heads, num_kv_heads,
-                               head_dim, scale, window)
+    if not (qkv.dtype == torch.bfloat16 and K.attention_mfma_supported(head_dim, kv.page_size)
+            and qkv.shape[1] % 8 == 0):
+        return K.attention_rowwise(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table,
+                                   batch.tok_seat, batch.positions, num_q_heads, num_kv_heads,
+                                   head_dim, scale, window)
+    group = num_q_heads // num_kv_heads
+    stride = qkv.shape[1]
+
+    def wave_kernel(items, tiles, splits, per, pair):
+        item_entry, item_row0, meta = items
+        K.attention_mfma(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table, item_entry, item_row0,
+                         batch.entry_seat, batch.entry_q_start, batch.entry_start_pos, num_q_heads,
+                         num_kv_heads, head_dim, scale, window, splits, per, tiles, pair, meta)
+
+    def decoded(which):
+        items = batch.attention_items(group, 1, which)
+        splits, per = choose_splits(items[0].shape[0], num_kv_heads, batch.max_context)
+        wave_kernel(items, 1, splits, per, False)
+
+    if batch.max_q_len * group <= 16:
+        decoded("all")
+        return out
+    mixed = batch.min_q_len * group <= 16
+    which = "long" if mixed else "all"
+    done = False
+    if K.attention_lds_supported(head_dim, kv.page_size):
+        items = batch.attention_items(group, 8, which)
+        groups = items[0].shape[0] * num_kv_heads
+        if items[2] is not None and groups >= _LDS_MIN_GROUPS and (
+                groups >= _LDS_MANY_GROUPS or batch.mean_keys_of_long_entries() >= _LDS_MIN_MEAN_KEYS):
+            K.attention_lds(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table, items[2], num_q_heads,
+                            num_kv_heads, head_dim, scale, window, False)
+            done = True
+    if not done:
+        # two row tiles per wave, so each key and value loaded serves 32 query rows; whole key
+        # ranges as long as that still gives a wave per SIMD
+        tiles = K.attention_mfma_row_tiles(head_dim, True)
+        items = batch.attention_items(group, tiles, which)
+        waves = items[0].shape[0] * num_kv_heads
+        if waves >= _WIDE_MIN_WAVES:
+            # items come ordered by work: a wavefront that takes the i-th and the i-th last does
+            # about the average; worth it while every SIMD still gets a wavefront
+            wave_kernel(items, tiles, 1, 0, waves >= _PAIR_MIN_WAVES)
+        else:
+            decoded(which)
+    if mixed:
+        decoded("short")
+    return out

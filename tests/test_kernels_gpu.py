@@ -247,6 +247,32 @@ def test_attention_mfma(nq, nkv, d, page, window, splits, wide, pair, gpu):
     assert torch.equal(out2, out)
 
 
+LONG_ENTRIES = [(0, 300), (40, 1), (200, 131), (5, 64), (0, 33)]
+
+
+@pytest.mark.parametrize("nq, nkv, d, window", [(4, 2, 32, 0), (32, 8, 64, 0), (8, 2, 64, 70), (6, 2, 96, 0),
+                                                (24, 8, 128, 0), (5, 1, 64, 0), (3, 3, 128, 150)])
+@pytest.mark.parametrize("pair", [False, True])
+def test_attention_with_keys_shared_through_lds(nq, nkv, d, window, pair, gpu):
+    """The workgroup kernel for prompt portions (128 query rows share each key block): long and
+    short entries, entries that start deep in their request, groups that do not divide 128,
+    windows, and work items taken in pairs."""
+    assert K.attention_lds_supported(d, 16) and not K.attention_lds_supported(d, 8)
+    assert not K.attention_lds_supported(48, 16)
+    dev, want, T, stride, scale, lens = attention_case("bfloat16", nq, nkv, d, 16, window, LONG_ENTRIES, 3, gpu)
+    group = nq // nkv
+    qs, sp, seat = dev["q_start"].cpu(), dev["start_pos"].cpu(), dev["entry_seat"].cpu()
+    rows = []
+    for e, n in enumerate(lens):
+        for r0 in range(0, n * group, 128):
+            rows.append((int(qs[e]), n, int(sp[e]), int(seat[e]), r0, 0, 0, 0))
+    rows.sort(key=lambda m: -(m[2] + (min(m[4] + 128, m[1] * group) - 1) // group))     # most keys first
+    meta = torch.tensor(rows, dtype=torch.int32, device=gpu)
+    out = torch.full((T, nq * d), float("nan"), dtype=torch.bfloat16, device=gpu)
+    K.attention_lds(dev["qkv"], stride, out, dev["kc"], dev["vc"], dev["table"], meta, nq, nkv, d, scale, window, pair)
+    close(out, want, torch.bfloat16, f"attention_lds pair={pair}", tol16=8e-3)
+
+
 @pytest.mark.parametrize("slope", [0.0, 0.35, -0.35, 3.0])
 def test_attention_with_scores_that_keep_rising_or_falling(slope, gpu):
     """The kernel re-bases its running softmax only when a row's maximum has moved far; scores
