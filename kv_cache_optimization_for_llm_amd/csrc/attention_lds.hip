@@ -31,6 +31,9 @@ struct LdsGeom {
     static constexpr int VBYTES = D * VROW;
     static constexpr int CHUNKS = 4 * D;             // 16-byte chunks of a K tile (and of a V^T tile)
     static constexpr int PER_THREAD = (CHUNKS + 255) / 256;
+    static constexpr int SB = 1;                     // 32-key blocks per stage (per barrier); 2 measured slower
+    static constexpr int BLOCK_BYTES = KBYTES + VBYTES;
+    static constexpr int STAGE_BYTES = SB * BLOCK_BYTES;
 };
 
 template <int D>
@@ -109,8 +112,8 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, const bf16_t *__restrict
     // chunk c of the V^T tile is 8 keys of value dimension (c % 2D) / 2 in page c / 2D.  A tile
     // outside the keys the workgroup needs is redirected to the nearest needed one (its page is
     // certainly mapped); its scores are masked away.
-    uint4 stage_k[Geo::PER_THREAD], stage_v[Geo::PER_THREAD];
-    auto fetch = [&](int kstart) {
+    uint4 stage_k[Geo::SB][Geo::PER_THREAD], stage_v[Geo::SB][Geo::PER_THREAD];
+    auto fetch = [&](int b, int kstart) {
         int pg[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -124,21 +127,21 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, const bf16_t *__restrict
             if (Geo::CHUNKS % 256 != 0 && c >= Geo::CHUNKS) break;
             const int key = c / (D / 8), kc = c % (D / 8);
             const size_t kpage = ((size_t)pg[key >> 4] * num_kv_heads + kvh) * (size_t)(16 * D);
-            stage_k[i] = *reinterpret_cast<const uint4 *>(k_cache + kpage + (size_t)(key & 15) * D + kc * 8);
+            stage_k[b][i] = *reinterpret_cast<const uint4 *>(k_cache + kpage + (size_t)(key & 15) * D + kc * 8);
             const int t = c / (2 * D), rem = c % (2 * D);
             const size_t vpage = ((size_t)pg[t] * num_kv_heads + kvh) * (size_t)(16 * D);
-            stage_v[i] = *reinterpret_cast<const uint4 *>(v_cache + vpage + (size_t)(rem >> 1) * 16 + (rem & 1) * 8);
+            stage_v[b][i] = *reinterpret_cast<const uint4 *>(v_cache + vpage + (size_t)(rem >> 1) * 16 + (rem & 1) * 8);
         }
     };
-    auto stash = [&](char *buf) {
+    auto stash = [&](int b, char *buf) {
 #pragma unroll
         for (int i = 0; i < Geo::PER_THREAD; ++i) {
             const int c = tid + i * 256;
             if (Geo::CHUNKS % 256 != 0 && c >= Geo::CHUNKS) break;
             const int key = c / (D / 8), kc = c % (D / 8);
-            *reinterpret_cast<uint4 *>(buf + key * Geo::KROW + kc * 16) = stage_k[i];
+            *reinterpret_cast<uint4 *>(buf + key * Geo::KROW + kc * 16) = stage_k[b][i];
             const int t = c / (2 * D), rem = c % (2 * D);
-            *reinterpret_cast<uint4 *>(buf + Geo::KBYTES + (rem >> 1) * Geo::VROW + (t * 16 + (rem & 1) * 8) * 2) = stage_v[i];
+            *reinterpret_cast<uint4 *>(buf + Geo::KBYTES + (rem >> 1) * Geo::VROW + (t * 16 + (rem & 1) * 8) * 2) = stage_v[b][i];
         }
     };
 
@@ -229,21 +232,33 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, const bf16_t *__restrict
                 o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf[rt].v, o[rt][dt], 0, 0, 0);
     };
 
-    // ---- the key loop: one barrier per block, two LDS buffers
-    constexpr int BUF = Geo::KBYTES + Geo::VBYTES;
-    fetch(k_begin);
-    stash(lds);
+    // ---- the key loop: a stage is SB blocks of 32 keys; one barrier per stage, two LDS buffers.
+    // Loads past the end are redirected inside fetch (never out of the mapped pages) and unused.
+    auto compute = [&](const char *buf, int kstart) {
+        if (wave_valid && kstart < k_end && kstart <= w_hi && kstart + 31 >= w_lo) {
+            const bool masked = window > 0 || kstart + 31 > w_first_pos || !all_rows;
+            if (masked) compute_as(std::true_type{}, buf, kstart);
+            else compute_as(std::false_type{}, buf, kstart);
+        }
+    };
+#pragma unroll
+    for (int b = 0; b < Geo::SB; ++b) fetch(b, k_begin + 32 * b);
+#pragma unroll
+    for (int b = 0; b < Geo::SB; ++b) stash(b, lds + b * Geo::BLOCK_BYTES);
     __syncthreads();
     int which = 0;
-    for (int kstart = k_begin; kstart < k_end; kstart += 32) {
-        const bool more = kstart + 32 < k_end;                 // uniform over the workgroup
-        if (more) fetch(kstart + 32);
-        if (wave_valid && kstart <= w_hi && kstart + 31 >= w_lo) {
-            const bool masked = window > 0 || kstart + 31 > w_first_pos || !all_rows;
-            if (masked) compute_as(std::true_type{}, lds + which * BUF, kstart);
-            else compute_as(std::false_type{}, lds + which * BUF, kstart);
+    for (int kstart = k_begin; kstart < k_end; kstart += 32 * Geo::SB) {
+        const bool more = kstart + 32 * Geo::SB < k_end;       // uniform over the workgroup
+        if (more) {
+#pragma unroll
+            for (int b = 0; b < Geo::SB; ++b) fetch(b, kstart + 32 * (Geo::SB + b));
         }
-        if (more) stash(lds + (which ^ 1) * BUF);
+#pragma unroll
+        for (int b = 0; b < Geo::SB; ++b) compute(lds + which * Geo::STAGE_BYTES + b * Geo::BLOCK_BYTES, kstart + 32 * b);
+        if (more) {
+#pragma unroll
+            for (int b = 0; b < Geo::SB; ++b) stash(b, lds + (which ^ 1) * Geo::STAGE_BYTES + b * Geo::BLOCK_BYTES);
+        }
         __syncthreads();
         which ^= 1;
     }
@@ -276,7 +291,7 @@ attention_lds_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q, int
                      const int *__restrict__ item_meta, int num_items, int pair, int num_q_heads,
                      int num_kv_heads, float scale, int window) {
     using Geo = LdsGeom<D>;
-    __shared__ __align__(16) char lds[2 * (Geo::KBYTES + Geo::VBYTES)];
+    __shared__ __align__(16) char lds[2 * Geo::STAGE_BYTES];
     const int kvh = blockIdx.x % num_kv_heads;
     const int w = blockIdx.x / num_kv_heads;
     attention_lds_item<D>(lds, out, q, q_row_stride, k_cache, v_cache, block_table, max_blocks, item_meta,
