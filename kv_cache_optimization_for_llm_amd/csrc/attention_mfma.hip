@@ -27,7 +27,8 @@
 // rounded to bf16 for the second product, the accumulator stays fp32.  Keys
 // are visited in blocks of 32 aligned to absolute positions.  With `splits` > 1 each split
 // writes an un-normalised partial (o, m, l) and attention_merge combines them (flash-decoding);
-// with one split the normalised result is written directly.
+// with one split the normalised result is written directly.  The merge runs over every row of the
+// output when the launch covered them all (`all_rows`), else over the rows the items name.
 //
 // Reference: same recurrence as paged_attention/src/kernels.cu:150-219 and the tiled prefill
 // kernel base/src/kernels.cu:361-466, which work one key at a time on CUDA cores.
@@ -386,9 +387,31 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
 #define MERGE_EARLY 32
 __global__ void __launch_bounds__(KVA_WAVE)
 attention_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o,
-                       const float *__restrict__ part_ml, int head_dim, int splits) {
+                       const float *__restrict__ part_ml, int head_dim, int splits,
+                       const int *__restrict__ item_meta, const int *__restrict__ item_entry,
+                       const int *__restrict__ item_row0, const int *__restrict__ entry_q_start,
+                       int num_q_heads, int num_kv_heads) {
     __shared__ float w_s[MERGE_MAX_SPLITS];
-    const size_t row = blockIdx.x;
+    // Either one workgroup per row of `out` (the launch covered every row: item arrays null), or
+    // one per (item, kv head, row of the item): then only the rows the items name are touched.
+    size_t row = blockIdx.x;
+    if (item_entry != nullptr) {
+        const int kvh = blockIdx.x % num_kv_heads, item = blockIdx.x / num_kv_heads;
+        int row0, q_start, q_len;
+        if (item_meta != nullptr) {
+            const int *meta = item_meta + (size_t)item * 8;
+            q_start = meta[0]; q_len = meta[1]; row0 = meta[4];
+        } else {
+            const int e = item_entry[item];
+            row0 = item_row0[item];
+            q_start = entry_q_start[e];
+            q_len = entry_q_start[e + 1] - q_start;
+        }
+        const int G = num_q_heads / num_kv_heads;
+        const int r = row0 + (int)blockIdx.y;
+        if (r >= q_len * G) return;
+        row = (size_t)(q_start + r / G) * num_q_heads + kvh * G + r % G;
+    }
     const int lane = threadIdx.x;
     const float2 *ml = reinterpret_cast<const float2 *>(part_ml) + row * splits;
     const float *po = part_o + row * splits * head_dim;
@@ -450,7 +473,8 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
                                   const int *entry_seat, const int *entry_q_start,
                                   const int *entry_start_pos, int total_rows, int num_q_heads,
                                   int num_kv_heads, int head_dim, int page_size, float scale, int window,
-                                  int splits, int keys_per_split, int pair, hipStream_t stream) {
+                                  int splits, int keys_per_split, int pair, int all_rows,
+                                  hipStream_t stream) {
     KVA_REQUIRE(num_items >= 0 && num_q_heads > 0 && num_kv_heads > 0 && max_blocks > 0,
                 "attention_mfma: bad sizes");
     KVA_REQUIRE(num_q_heads % num_kv_heads == 0, "attention_mfma: %d query heads is not a multiple of %d kv heads",
@@ -497,8 +521,14 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
 #undef LAUNCH
     KVA_CHECK_LAUNCH("attention_mfma");
     if (splits > 1) {
-        hipLaunchKernelGGL(attention_merge_kernel, dim3(total_rows), dim3(64), 0, stream, (bf16_t *)out,
-                           part_o, part_ml, head_dim, splits);
+        if (all_rows)
+            hipLaunchKernelGGL(attention_merge_kernel, dim3(total_rows), dim3(64), 0, stream, (bf16_t *)out,
+                               part_o, part_ml, head_dim, splits, nullptr, nullptr, nullptr, nullptr,
+                               num_q_heads, num_kv_heads);
+        else
+            hipLaunchKernelGGL(attention_merge_kernel, dim3(num_items * num_kv_heads, 16 * row_tiles), dim3(64),
+                               0, stream, (bf16_t *)out, part_o, part_ml, head_dim, splits, item_meta,
+                               item_entry, item_row0, entry_q_start, num_q_heads, num_kv_heads);
         KVA_CHECK_LAUNCH("attention_merge");
     }
     return KVA_OK;

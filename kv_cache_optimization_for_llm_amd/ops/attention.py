@@ -59,16 +59,17 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
     group = num_q_heads // num_kv_heads
     stride = qkv.shape[1]
 
-    def wave_kernel(items, tiles, splits, per, pair):
+    def wave_kernel(items, tiles, splits, per, pair, which):
         item_entry, item_row0, meta = items
         K.attention_mfma(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table, item_entry, item_row0,
                          batch.entry_seat, batch.entry_q_start, batch.entry_start_pos, num_q_heads,
-                         num_kv_heads, head_dim, scale, window, splits, per, tiles, pair, meta)
+                         num_kv_heads, head_dim, scale, window, splits, per, tiles, pair, meta,
+                         covers_all_rows=which == "all")
 
     def decoded(which):
         items = batch.attention_items(group, 1, which)
         splits, per = choose_splits(items[0].shape[0], num_kv_heads, batch.max_context)
-        wave_kernel(items, 1, splits, per, False)
+        wave_kernel(items, 1, splits, per, False, which)
 
     if batch.max_q_len * group <= 16:
         decoded("all")
@@ -93,7 +94,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
         if waves >= _WIDE_MIN_WAVES:
             # items come ordered by work: a wavefront that takes the i-th and the i-th last does
             # about the average; worth it while every SIMD still gets a wavefront
-            wave_kernel(items, tiles, 1, 0, waves >= _PAIR_MIN_WAVES)
+            wave_kernel(items, tiles, 1, 0, waves >= _PAIR_MIN_WAVES, which)
         else:
             decoded(which)
     if mixed:

@@ -39,7 +39,17 @@ TINY_C = dict(
                       original_max_position_embeddings=128),
     tie_word_embeddings=False, hidden_act="silu", torch_dtype="bfloat16",
 )
-TINY = {"A": (TINY_A, 11), "B": (TINY_B, 23), "C": (TINY_C, 37)}
+# head size 32: the sizes at which the product epilogues and the workgroup attention kernel that
+# need multiples of 32 take part (the other three have 16, 24 and 48)
+TINY_D = dict(
+    architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=301, hidden_size=160,
+    intermediate_size=208, num_hidden_layers=2, num_attention_heads=5, num_key_value_heads=1,
+    head_dim=32, rms_norm_eps=2e-5, rope_theta=300000.0, max_position_embeddings=512,
+    rope_scaling=dict(rope_type="llama3", factor=16.0, low_freq_factor=1.0, high_freq_factor=8.0,
+                      original_max_position_embeddings=256),
+    tie_word_embeddings=True, hidden_act="silu", torch_dtype="bfloat16",
+)
+TINY = {"A": (TINY_A, 11), "B": (TINY_B, 23), "C": (TINY_C, 37), "D": (TINY_D, 41)}
 
 
 @pytest.fixture(scope="session")

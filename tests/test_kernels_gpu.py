@@ -245,6 +245,20 @@ def test_attention_mfma(nq, nkv, d, page, window, splits, wide, pair, gpu):
                      dev["entry_seat"], dev["q_start"], dev["start_pos"], nq, nkv, d, scale, window,
                      splits, per, tiles, pair, meta.to(gpu))
     assert torch.equal(out2, out)
+    # a launch over some of the entries only (the others belong to another launch of the same
+    # step): their rows are right, every other row keeps what it held, split merge included
+    keep = (ent.cpu() % 2 == 0)
+    sub = keep.nonzero().flatten().to(gpu)
+    out3 = torch.full_like(out, 7.0)
+    K.attention_mfma(dev["qkv"], stride, out3, dev["kc"], dev["vc"], dev["table"], ent[sub], row0[sub],
+                     dev["entry_seat"], dev["q_start"], dev["start_pos"], nq, nkv, d, scale, window,
+                     splits, per, tiles, False, meta.to(gpu)[sub] if pair else None, covers_all_rows=False)
+    for e in range(len(lens)):
+        rows = slice(int(qs[e]), int(qs[e + 1]))
+        if e % 2 == 0:
+            assert torch.equal(out3[rows], out[rows])
+        else:
+            assert (out3[rows] == 7.0).all()
 
 
 LONG_ENTRIES = [(0, 300), (40, 1), (200, 131), (5, 64), (0, 33)]
