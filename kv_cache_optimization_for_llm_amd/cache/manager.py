@@ -45,6 +45,7 @@ class _Seat:
     next_block: List[int] = field(default_factory=list)  # per group: first logical block not mapped yet
     first_block: List[int] = field(default_factory=list)  # per group: first logical block still mapped
     run: List[Optional[Tuple[int, int]]] = field(default_factory=list)  # contiguous: (start, pages)
+    mapped_tokens: int = 0                              # paged: positions below this have a page in every group
 
 
 class CacheGroup:
@@ -94,6 +95,7 @@ class CacheManager:
         self._seats: List[Optional[_Seat]] = [None] * max_seqs
         self._free_seats = list(range(max_seqs - 1, -1, -1))   # popped from the back: lowest first
         self.peak_held_pages = 0
+        self._no_pages = [0] * len(self.groups)     # shared answer of pages_needed; never modified
         self._flush_event = None     # set while an upload of table spans may still be reading the host table
         if device is not None:
             self._allocate_device()
@@ -237,8 +239,8 @@ class CacheManager:
     def pages_needed(self, seat: int, new_len: int) -> List[int]:
         """Pages each group must still map so that positions ``< new_len`` have a place."""
         s = self.seat(seat)
-        if self.mode == "contiguous":
-            return [0] * len(self.groups)
+        if self.mode == "contiguous" or new_len <= s.mapped_tokens:
+            return self._no_pages
         blocks = (new_len + self.page_size - 1) // self.page_size
         return [max(0, blocks - s.next_block[g.index]) for g in self.groups]
 
@@ -252,11 +254,13 @@ class CacheManager:
 
     def grow(self, seat: int, new_len: int) -> bool:
         """Maps pages so positions ``< new_len`` can be written.  All groups or none."""
+        s = self.seat(seat)
+        if self.mode == "paged" and new_len <= s.mapped_tokens:
+            return True         # the common decode step: the page is there already
         if new_len > self.capacity_tokens(seat):
             return False
         if self.mode == "contiguous":
             return True
-        s = self.seat(seat)
         need = self.pages_needed(seat, new_len)
         if any(n > g.free_pages() for n, g in zip(need, self.groups)):
             return False
@@ -274,6 +278,7 @@ class CacheManager:
             g.table_host[seat, lo:lo + n] = np.asarray(pages, dtype=np.int32)
             g.mark_dirty(seat, lo, lo + n)
             s.next_block[g.index] = lo + n
+        s.mapped_tokens = min(min(s.next_block) * self.page_size, self.capacity_tokens(seat))   # never past the longest sequence
         self._note_peak()
         return True
 
@@ -286,6 +291,15 @@ class CacheManager:
             raise CacheError(f"seat {seat}: positions {start}..{start + count - 1} are not all mapped "
                              f"in group {group}")
         return (pages * self.page_size + pos % self.page_size).astype(np.int32)
+
+    def slot_mapping_each(self, seats: np.ndarray, positions: np.ndarray, group: int) -> np.ndarray:
+        """Cache slots of one position per seat (a decode step), in one go."""
+        g = self.groups[group]
+        pages = g.table_host[seats, positions // self.page_size].astype(np.int64)
+        if (pages < 0).any():
+            bad = int(np.nonzero(pages < 0)[0][0])
+            raise CacheError(f"seat {int(seats[bad])}: position {int(positions[bad])} is not mapped in group {group}")
+        return (pages * self.page_size + positions % self.page_size).astype(np.int32)
 
     def commit(self, seat: int, new_len: int) -> None:
         """The step wrote positions up to ``new_len``; window groups give back what lies behind."""

@@ -153,8 +153,6 @@ def run_one(args, shape: str, batch: int, mode: str) -> dict:
         gbs = step_bytes / (decode_time / decode_steps) / 1e9
         out["decode_hbm_gbs"] = round(gbs, 1)
         out["decode_hbm_frac"] = round(gbs / HBM_PEAK_GBS, 4)
-    del runner, engine
-    torch.cuda.empty_cache()
     return out
 
 

@@ -166,18 +166,23 @@ class Engine:
     def _run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         seats, starts, toks, wants = self._place(entries)
         groups = self.cache.groups
-        slot_maps = [[self.cache.slot_mapping(seat, start, len(arr), g.index)
-                      for seat, start, arr in zip(seats, starts, toks)] for g in groups]
-        self.cache.flush_tables()
-        if self.graphs is not None and all(len(t) == 1 for t in toks):
-            logits = self.graphs.run(np.asarray([t[0] for t in toks], dtype=np.int32),
-                                     np.asarray(starts, dtype=np.int32), np.asarray(seats, dtype=np.int32),
-                                     [np.concatenate(m) for m in slot_maps])
-            rows = [e for e, w in enumerate(wants) for _ in w]
-            if rows != list(range(len(entries))):
-                logits = logits[torch.tensor(rows, dtype=torch.long, device=self.device)] if rows \
-                    else logits[:0]
-            return logits
+        if all(len(t) == 1 for t in toks):
+            # a decode step: one position per entry, everything in whole arrays
+            seats_a, starts_a = np.asarray(seats, dtype=np.int32), np.asarray(starts, dtype=np.int32)
+            slots = [self.cache.slot_mapping_each(seats_a, starts_a, g.index) for g in groups]
+            self.cache.flush_tables()
+            if self.graphs is not None:
+                logits = self.graphs.run(np.asarray([t[0] for t in toks], dtype=np.int32), starts_a, seats_a, slots)
+                rows = [e for e, w in enumerate(wants) for _ in w]
+                if rows != list(range(len(entries))):
+                    logits = logits[torch.tensor(rows, dtype=torch.long, device=self.device)] if rows \
+                        else logits[:0]
+                return logits
+            slot_maps = [[m[i:i + 1] for i in range(len(seats))] for m in slots]
+        else:
+            slot_maps = [[self.cache.slot_mapping(seat, start, len(arr), g.index)
+                          for seat, start, arr in zip(seats, starts, toks)] for g in groups]
+            self.cache.flush_tables()
         batch = build_batch(seats, starts, toks, wants, slot_maps, self.device)
         batch.feedback = self.feedback
         return self.model.forward(batch, self.cache)
@@ -188,37 +193,46 @@ class Engine:
             raise EngineError("a step needs at least one entry")
         seen = set()
         seats, starts, toks, wants = [], [], [], []
+        vocab, lowest_single = self.vocab_size, -self.feedback.shape[0]
         for e in entries:       # refuse a bad step before anything is admitted or mapped
             if e.request_id in seen:
                 raise EngineError(f"request {e.request_id!r} appears twice in one step")
             seen.add(e.request_id)
-            if len(e.tokens) == 0:
+            n = len(e.tokens)
+            if n == 0:
                 raise EngineError(f"request {e.request_id!r}: an entry needs at least one token")
-            arr = np.asarray(e.tokens, dtype=np.int64)
-            lowest = -self.feedback.shape[0] if len(arr) == 1 else 0     # a lone token may be a feedback row
-            if arr.min() < lowest or arr.max() >= self.vocab_size:
-                raise EngineError(f"request {e.request_id!r}: token id outside [0, {self.vocab_size})")
+            if n == 1:
+                arr = e.tokens if isinstance(e.tokens, list) else list(e.tokens)
+                lo = hi = int(arr[0])
+                lowest = lowest_single           # a lone token may be a feedback row
+            else:
+                arr = np.asarray(e.tokens, dtype=np.int64)
+                lo, hi, lowest = int(arr.min()), int(arr.max()), 0
+            if lo < lowest or hi >= vocab:
+                raise EngineError(f"request {e.request_id!r}: token id outside [0, {vocab})")
             for i in e.want:
-                if not 0 <= i < len(arr):
+                if not 0 <= i < n:
                     raise EngineError(f"request {e.request_id!r}: wanted place {i} is outside its "
-                                      f"{len(arr)} tokens")
+                                      f"{n} tokens")
             toks.append(arr)
-            wants.append(list(e.want))
+            wants.append(e.want if isinstance(e.want, list) else list(e.want))
+        seat_of, cache = self._seat_of, self.cache
         for e in entries:
-            if e.request_id not in self._seat_of:
+            seat = seat_of.get(e.request_id)
+            if seat is None:
                 if self.add_request(e.request_id) is None:
                     raise CacheExhausted(f"no seat (or reservation) for request {e.request_id!r}")
-            seat = self._seat_of[e.request_id]
+                seat = seat_of[e.request_id]
             seats.append(seat)
-            starts.append(self.cache.length(seat))
+            starts.append(cache.length(seat))
         # map the pages the step writes to
         for e, seat, start, arr in zip(entries, seats, starts, toks):
-            if not self.cache.grow(seat, start + len(arr)):
-                need = self.cache.pages_needed(seat, start + len(arr))
+            if not cache.grow(seat, start + len(arr)):
+                need = cache.pages_needed(seat, start + len(arr))
                 raise CacheExhausted(
                     f"request {e.request_id!r} needs {need} more pages for positions "
-                    f"{start}..{start + len(arr) - 1} (capacity {self.cache.capacity_tokens(seat)} "
-                    f"tokens, free pages {[g.free_pages() for g in self.cache.groups]})")
+                    f"{start}..{start + len(arr) - 1} (capacity {cache.capacity_tokens(seat)} "
+                    f"tokens, free pages {[g.free_pages() for g in cache.groups]})")
         return seats, starts, toks, wants
 
     def finish(self, entries: Sequence[StepEntry]) -> None:

@@ -203,3 +203,17 @@ def test_random_orders_keep_the_books(mode, seed):
     m.check()
     assert all(g.free_pages() == 24 for g in m.groups) and m.free_seats == 5
     assert admitted > 20
+
+
+def test_a_sequence_cannot_grow_past_the_longest_length_inside_its_last_page():
+    """The longest sequence need not be a multiple of the page size: the last page then has rows
+    that must never be used, also on the quick path that skips the books when a page is there."""
+    m = CacheManager([(KVCacheSpec(2, 16), [0])], {}, page_size=16, num_pages=8, max_seqs=2, max_seq_len=53)
+    seat = m.admit("r")
+    assert m.grow(seat, 50) and m.capacity_tokens(seat) == 53
+    m.commit(seat, 50)
+    assert m.pages_needed(seat, 53) == [0] and m.grow(seat, 53)
+    assert not m.grow(seat, 54) and not m.can_grow(seat, 54)
+    m.commit(seat, 53)
+    assert not m.grow(seat, 54)
+    m.check()
