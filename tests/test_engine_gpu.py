@@ -144,6 +144,45 @@ def test_running_ahead_of_the_device_changes_nothing_that_is_emitted(dtype, mode
             assert not eos & set(g)
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_random_workloads_emit_the_same_with_and_without_running_ahead(seed, model_dirs, gpu):
+    """Random prompt lengths and output budgets, more requests than seats, so few pages that
+    requests are preempted and recomputed, end-of-sequence ids that do occur, a temperature: the
+    loop that runs ahead of the device emits, per request, exactly what the synchronous loop does."""
+    from kv_cache_optimization_for_llm_amd.engine.runner import Runner
+    rng = np.random.default_rng(100 + seed)
+    cfg = TINY["A"][0]
+    eng = Engine(model_dirs["A"], EngineOptions(dtype="float32", max_seqs=3, max_seq_len=128, cache_tokens=160))
+    requests = [([int(t) for t in rng.integers(0, cfg["vocab_size"], int(rng.integers(1, 60)))],
+                 int(rng.integers(3, 40))) for _ in range(9)]
+    probe = Runner(eng, ServeOptions(run_ahead=False, ignore_eos=True, temperature=0.8, sampling_seed=seed))
+    for p, n in requests:
+        probe.submit(p, n)
+    seen = [ev.token for ev in probe.run_until_idle() if ev.kind == "token"]
+    eos = [int(t) for t in np.unique(seen)[:3]]               # ids that the requests do sample
+    results = {}
+    for ahead in (False, True):
+        runner = Runner(eng, ServeOptions(run_ahead=ahead, temperature=0.8, sampling_seed=seed,
+                                          max_batch_tokens=48, chunk_size=16))
+        runner.scheduler.eos = frozenset(eos)
+        ids = [runner.submit(p, n) for p, n in requests]
+        out = {i: [] for i in ids}
+        reasons = {}
+        for ev in runner.run_until_idle():
+            if ev.kind == "token":
+                assert ev.request_id not in reasons, "a token after the request was done"
+                out[ev.request_id].append(ev.token)
+            elif ev.kind in ("done", "rejected"):
+                reasons[ev.request_id] = ev.reason
+        results[ahead] = (out, reasons, runner.scheduler.preemptions)
+        eng.cache.check()
+        assert eng.cache.free_seats == 3 and all(g.free_pages() == g.num_pages for g in eng.cache.groups)
+    assert results[True][0] == results[False][0] and results[True][1] == results[False][1]
+    assert set(results[True][1].values()) <= {"eos", "length"} and len(results[True][1]) == len(requests)
+    assert not any(set(eos) & set(toks) for toks in results[True][0].values())
+    assert results[False][2] > 0 or results[True][2] > 0 or seed != 0     # pages do run out at least once
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_and_first_tokens(dtype, model_dirs, gpu):
     """300 tokens decoded one by one from a one-token start: crosses many pages and several
