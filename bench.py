@@ -23,7 +23,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "fp32": 157.3}
 
-# BASELINE.json configs[2]: Llama 3.2 1B shape
+# the benchmark configuration: Llama 3.2 1B shape
 CONFIG_1B = dict(
     architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=128256, hidden_size=2048,
     intermediate_size=8192, num_hidden_layers=16, num_attention_heads=32, num_key_value_heads=8,
@@ -154,7 +154,7 @@ def main():
             k = max(16, args.steps // 2)
             d, _ = decode_run(b, k, 8, ctx)
             points[f"decode_b{b}"] = round(b * k / d, 1)
-        # the workload BASELINE.json words: 512-token prompts, 256 generated tokens
+        # the serving workload of the comparison: 512-token prompts, 256 generated tokens
         for b in (1, 8, 64):
             d, _ = decode_run(b, 240, 8, 512 + 256)
             points[f"decode_b{b}_p512_g256"] = round(b * 240 / d, 1)
