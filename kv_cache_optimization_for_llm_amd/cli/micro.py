@@ -1,0 +1,158 @@
+"""Single kernels in a loop, for timing and for profilers.
+
+    python -m kv_cache_optimization_for_llm_amd.cli.micro attention --tokens 8192 --kernel lds
+    python -m kv_cache_optimization_for_llm_amd.cli.micro attention --batch 8 --context 8192 --splits 32
+    python -m kv_cache_optimization_for_llm_amd.cli.micro gemm --rows 8 --shape gate_up
+
+The reference keeps a harness that runs its attention kernels alone over made-up caches
+(``micro/harness.cuh``); this is the same idea for the kernels here.  Sizes default to the
+Llama-3.2-1B ones.  Every call works on its own copy of the weights or the cache, enough copies
+that nothing is served from a cache of the memory system, and one line is printed per case:
+microseconds per call, and TFLOP/s or TB/s of what the call has to compute or read.  Calls are
+launched one by one from the host: below some 15 us a figure shows the host's launch rate, not
+the kernel (inside a HIP graph, as decode steps run, the same kernels take less).
+"""
+from __future__ import annotations
+
+import argparse
+import sys
+import time
+
+GEMM_SHAPES = {          # name: (N, K, mode)   mode: plain | resid | swiglu | f32
+    "qkv": (3072, 2048, "plain"), "o": (2048, 2048, "resid"), "gate_up": (16384, 2048, "swiglu"),
+    "down": (2048, 8192, "resid"), "lm_head": (128256, 2048, "f32"),
+}
+
+
+def _time(calls, reps: int) -> float:
+    import torch
+    for f in calls:
+        f()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(reps):
+        calls[i % len(calls)]()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / reps * 1e6
+
+
+def attention(args) -> None:
+    import numpy as np
+    import torch
+    from ..ops import kernels as K
+
+    dev = torch.device("cuda:0")
+    nq, nkv, d, page = args.heads, args.kv_heads, args.head_dim, 16
+    group = nq // nkv
+    scale = d ** -0.5
+    if args.tokens:                                # one prompt of `tokens` tokens from position 0
+        entries = [(0, args.tokens)]
+    else:                                          # `batch` decoded tokens at the end of `context`
+        entries = [(args.context - 1, 1)] * args.batch
+    ctx = max(s + n for s, n in entries)
+    blocks = (ctx + page - 1) // page
+    copies = max(1, min(8, int(600e6 / (len(entries) * blocks * page * nkv * d * 4)) + 1))
+    caches = [(torch.randn(len(entries) * blocks, nkv, page, d, device=dev).bfloat16(),
+               torch.randn(len(entries) * blocks, nkv, d, page, device=dev).bfloat16()) for _ in range(copies)]
+    table = torch.arange(len(entries) * blocks, dtype=torch.int32).view(len(entries), blocks).to(dev)
+    lens = [n for _, n in entries]
+    T = sum(lens)
+    qkv = torch.randn(T, nq * d, device=dev).bfloat16()
+    out = torch.empty(T, nq * d, dtype=torch.bfloat16, device=dev)
+    q_start = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    rows_per_item = {"lds": 128, "wave": 32 if args.tokens else 16}[args.kernel]
+    meta = []
+    for e, (start, n) in enumerate(entries):
+        for r0 in range(0, n * group, rows_per_item):
+            meta.append((q_start[e], n, start, e, r0, 0, 0, 0))
+    meta.sort(key=lambda m: -(m[2] + (min(m[4] + rows_per_item, m[1] * group) - 1) // group))
+    meta_d = torch.tensor(meta, dtype=torch.int32, device=dev)
+    ent = meta_d[:, 3].contiguous()
+    row0 = meta_d[:, 4].contiguous()
+    seat = torch.arange(len(entries), dtype=torch.int32, device=dev)
+    qs = torch.from_numpy(q_start).to(dev)
+    sp = torch.tensor([s for s, _ in entries], dtype=torch.int32, device=dev)
+    splits, per = 1, 0
+    if not args.tokens:
+        splits = args.splits
+        per = ((ctx + splits - 1) // splits + 31) // 32 * 32
+    if args.kernel == "lds":
+        calls = [lambda c=c: K.attention_lds(qkv, nq * d, out, c[0], c[1], table, meta_d, nq, nkv, d, scale, 0, False)
+                 for c in caches]
+    else:
+        tiles = 2 if args.tokens else 1
+        pair = bool(args.tokens) and len(meta) * nkv >= 2048
+        calls = [lambda c=c: K.attention_mfma(qkv, nq * d, out, c[0], c[1], table, ent, row0, seat, qs, sp, nq, nkv,
+                                              d, scale, 0, splits, per, tiles, pair, meta_d) for c in caches]
+    us = _time(calls, args.reps)
+    flops = sum(4.0 * nq * d * n * (2 * s + n + 1) / 2 for s, n in entries)
+    kv_bytes = sum((s + n) * nkv * d * 4 for s, n in entries)
+    what = f"prompt of {args.tokens}" if args.tokens else f"batch {args.batch} at context {args.context}, {splits} splits"
+    print(f"attention {args.kernel:4s} {what}: {us:9.1f} us  {flops / us / 1e6:8.1f} TFLOP/s  "
+          f"{kv_bytes / us / 1e6:7.2f} TB/s of keys and values", flush=True)
+
+
+def gemm(args) -> None:
+    import torch
+    from ..ops import kernels as K
+
+    dev = torch.device("cuda:0")
+    n, k, mode = GEMM_SHAPES[args.shape]
+    m = args.rows
+    copies = min(48, max(4, int(600e6 / (n * k * 2)) + 1))
+    x = torch.randn(m, k, device=dev).bfloat16()
+    ws = [torch.randn(n, k, device=dev).bfloat16() * 0.02 for _ in range(copies)]
+    tiled = [K.TiledWeight(w, 2 if mode == "swiglu" else 1) for w in ws]
+    if mode == "resid":
+        hidden = torch.zeros(m, n, device=dev).bfloat16()
+        scaled = torch.empty_like(hidden)
+        ss = torch.empty(m, K.gemm_skinny_sumsq_parts(n), device=dev)
+        nw = torch.ones(n, device=dev).bfloat16()
+        calls = [lambda w=w: K.gemm_skinny(x, w, None, hidden=hidden, next_weight=nw, scaled_out=scaled, sumsq_out=ss)
+                 for w in tiled]
+    elif mode == "swiglu":
+        out = torch.empty(m, n // 2, device=dev).bfloat16()
+        calls = [lambda w=w: K.gemm_skinny(x, w, out, swiglu=True) for w in tiled]
+    else:
+        out = torch.empty(m, n, device=dev, dtype=torch.float32 if mode == "f32" else torch.bfloat16)
+        calls = [lambda w=w: K.gemm_skinny(x, w, out) for w in tiled]
+    us = _time(calls, args.reps)
+    line = f"gemm {args.shape:8s} rows {m:3d} [{n} x {k}] few-rows kernel {us:8.2f} us  {n * k * 2 / us / 1e6:6.2f} TB/s of weights"
+    if args.vendor:
+        out_v = torch.empty(m, n, device=dev, dtype=torch.bfloat16)
+        us_v = _time([lambda w=w: torch.matmul(x, w.t(), out=out_v) for w in ws], args.reps)
+        line += f"   vendor GEMM {us_v:8.2f} us"
+    print(line, flush=True)
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(description="one kernel in a loop")
+    sub = ap.add_subparsers(dest="what", required=True)
+    a = sub.add_parser("attention")
+    a.add_argument("--kernel", choices=["wave", "lds"], default="wave",
+                   help="one wavefront per work item, or a workgroup sharing key blocks through LDS")
+    a.add_argument("--tokens", type=int, default=0, help="a prompt of this many tokens (else decoded tokens)")
+    a.add_argument("--batch", type=int, default=8)
+    a.add_argument("--context", type=int, default=8192)
+    a.add_argument("--splits", type=int, default=32)
+    a.add_argument("--heads", type=int, default=32)
+    a.add_argument("--kv-heads", type=int, default=8)
+    a.add_argument("--head-dim", type=int, default=64)
+    a.add_argument("--reps", type=int, default=20)
+    g = sub.add_parser("gemm")
+    g.add_argument("--shape", choices=sorted(GEMM_SHAPES), default="gate_up")
+    g.add_argument("--rows", type=int, default=8)
+    g.add_argument("--vendor", action="store_true", help="also time the vendor GEMM on the plain weight")
+    g.add_argument("--reps", type=int, default=48)
+    args = ap.parse_args(argv)
+    if args.what == "attention":
+        if args.kernel == "lds" and not args.tokens:
+            ap.error("the workgroup kernel is for prompts: give --tokens")
+        attention(args)
+    else:
+        gemm(args)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
