@@ -98,12 +98,19 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, const bf16_t *__restrict
                                           : make_uint4(0, 0, 0, 0);
     }
 
-    float m[RT], l[RT];
-    f32x4 o[RT][NDT];
+    // Running maximum m, accumulator O^T and denominator per query row.  The denominator is one more
+    // tile of the second product: against a V^T tile of ones, O^T += V^T P^T adds up the row's P
+    // (every element of the tile ends up as the row's sum) - on the matrix cores, which have time
+    // to spare here, instead of 16 additions and a 4-lane reduction per block in the vector ALU,
+    // which has none.  It also makes the denominator the sum of exactly the rounded P the numerator uses.
+    float m[RT];
+    f32x4 o[RT][NDT], ol[RT];
+    Frag8 ones;
+    ones.u4 = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u);      // 8 x bf16 1.0
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         m[rt] = -INFINITY;
-        l[rt] = 0.f;
+        ol[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt) o[rt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
@@ -204,7 +211,7 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, const bf16_t *__restrict
             for (int rt = 0; rt < RT; ++rt) {
                 const float m_new = fmaxf(m[rt], mloc[rt]);
                 const float c = __builtin_amdgcn_exp2f((m[rt] - ((m_new == -INFINITY) ? 0.f : m_new)) * scale2);
-                l[rt] *= c;
+                ol[rt][0] *= c; ol[rt][1] *= c; ol[rt][2] *= c; ol[rt][3] *= c;
 #pragma unroll
                 for (int dt = 0; dt < NDT; ++dt) {
                     o[rt][dt][0] *= c; o[rt][dt][1] *= c; o[rt][dt][2] *= c; o[rt][dt][3] *= c;
@@ -215,21 +222,20 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, const bf16_t *__restrict
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
             const float neg_ref = (MASKED && m[rt] == -INFINITY) ? 0.f : -m[rt] * scale2;
-            float lsum = 0.f;
 #pragma unroll
             for (int j = 0; j < 8; j += 2) {
                 const float p0 = __builtin_amdgcn_exp2f(fmaf(sv[rt][j], scale2, neg_ref));
                 const float p1 = __builtin_amdgcn_exp2f(fmaf(sv[rt][j + 1], scale2, neg_ref));
-                lsum += p0 + p1;
                 pf[rt].p2[j / 2] = pack_bf16(p0, p1);
             }
-            l[rt] += quad_rows_sum(lsum);
         }
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
+        for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt)
                 o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf[rt].v, o[rt][dt], 0, 0, 0);
+            ol[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pf[rt].v, ol[rt], 0, 0, 0);
+        }
     };
 
     // ---- the key loop: a stage is SB blocks of 32 keys; one barrier per stage, two LDS buffers.
@@ -268,7 +274,7 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, const bf16_t *__restrict
     for (int rt = 0; rt < RT; ++rt) {
         if (!row_valid[rt]) continue;
         const size_t orow = (size_t)(q_start + tq[rt]) * num_q_heads + head[rt];
-        const float inv = 1.f / l[rt];
+        const float inv = 1.f / ol[rt][0];
         bf16_t *dst = out + orow * D;
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt) {
@@ -284,12 +290,12 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, const bf16_t *__restrict
 // head varies fastest so that a die's L2 keeps meeting the same heads.  With `pair` a workgroup
 // takes item w and then item n-1-w of the list, which the caller orders by keys visited.
 template <int D>
-__global__ void __launch_bounds__(256)
-attention_lds_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q, int q_row_stride,
-                     const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
-                     const int *__restrict__ block_table, int max_blocks,
-                     const int *__restrict__ item_meta, int num_items, int pair, int num_q_heads,
-                     int num_kv_heads, float scale, int window) {
+__device__ __forceinline__ void
+attention_lds_body(bf16_t *__restrict__ out, const bf16_t *__restrict__ q, int q_row_stride,
+                   const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
+                   const int *__restrict__ block_table, int max_blocks,
+                   const int *__restrict__ item_meta, int num_items, int pair, int num_q_heads,
+                   int num_kv_heads, float scale, int window) {
     using Geo = LdsGeom<D>;
     __shared__ __align__(16) char lds[2 * Geo::STAGE_BYTES];
     const int kvh = blockIdx.x % num_kv_heads;
@@ -300,6 +306,29 @@ attention_lds_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q, int
     if (pair && other > w)      // the last barrier of the first item has passed: LDS is free again
         attention_lds_item<D>(lds, out, q, q_row_stride, k_cache, v_cache, block_table, max_blocks, item_meta,
                               num_q_heads, num_kv_heads, scale, window, other, kvh);
+}
+
+#define LDS_KERNEL_PARAMS                                                                          \
+    bf16_t *__restrict__ out, const bf16_t *__restrict__ q, int q_row_stride,                      \
+    const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,                        \
+    const int *__restrict__ block_table, int max_blocks, const int *__restrict__ item_meta,        \
+    int num_items, int pair, int num_q_heads, int num_kv_heads, float scale, int window
+#define LDS_KERNEL_ARGS                                                                            \
+    out, q, q_row_stride, k_cache, v_cache, block_table, max_blocks, item_meta, num_items, pair,   \
+    num_q_heads, num_kv_heads, scale, window
+
+template <int D>
+__global__ void __launch_bounds__(256) attention_lds_kernel(LDS_KERNEL_PARAMS) {
+    attention_lds_body<D>(LDS_KERNEL_ARGS);
+}
+
+// Head sizes up to 64 need a few registers more than three wavefronts per SIMD leave each (168):
+// held to that, the compiler spills a handful of values, and three wavefronts instead of two are
+// worth far more than those cost (the kernel is bound by vector work the wavefronts overlap).
+template <int D>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3)))
+attention_lds_kernel_3(LDS_KERNEL_PARAMS) {
+    attention_lds_body<D>(LDS_KERNEL_ARGS);
 }
 
 extern "C" int kva_attention_lds_supported(int head_dim, int page_size) {
@@ -326,15 +355,15 @@ extern "C" int kva_attention_lds(void *out, const void *q, int q_row_stride, con
     const int groups = pair ? (num_items + 1) / 2 : num_items;
     KVA_REQUIRE((long)groups * num_kv_heads < (1L << 31), "attention_lds: too many work items");
     dim3 grid(groups * num_kv_heads), block(256);
-#define LAUNCH(DD)                                                                                  \
-    hipLaunchKernelGGL((attention_lds_kernel<DD>), grid, block, 0, stream, (bf16_t *)out,          \
-                       (const bf16_t *)q, q_row_stride, (const bf16_t *)k_cache, (const bf16_t *)v_cache, \
-                       block_table, max_blocks, item_meta, num_items, pair, num_q_heads, num_kv_heads, scale, window)
+#define LAUNCH(KERNEL, DD)                                                                          \
+    hipLaunchKernelGGL((KERNEL<DD>), grid, block, 0, stream, (bf16_t *)out, (const bf16_t *)q,      \
+                       q_row_stride, (const bf16_t *)k_cache, (const bf16_t *)v_cache, block_table, \
+                       max_blocks, item_meta, num_items, pair, num_q_heads, num_kv_heads, scale, window)
     switch (head_dim) {
-    case 32: LAUNCH(32); break;
-    case 64: LAUNCH(64); break;
-    case 96: LAUNCH(96); break;
-    default: LAUNCH(128); break;
+    case 32: LAUNCH(attention_lds_kernel_3, 32); break;
+    case 64: LAUNCH(attention_lds_kernel_3, 64); break;
+    case 96: LAUNCH(attention_lds_kernel, 96); break;
+    default: LAUNCH(attention_lds_kernel, 128); break;
     }
 #undef LAUNCH
     KVA_CHECK_LAUNCH("attention_lds");
