@@ -120,6 +120,20 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, const bf16_t *__restrict
     // outside the keys the workgroup needs is redirected to the nearest needed one (its page is
     // certainly mapped); its scores are masked away.
     uint4 stage_k[Geo::SB][Geo::PER_THREAD], stage_v[Geo::SB][Geo::PER_THREAD];
+    // which of the block's two pages a thread's chunk lies in is the same for a whole wavefront
+    // (said explicitly, so that the page's address stays scalar arithmetic); its place inside the
+    // page never changes
+    int k_sel[Geo::PER_THREAD], v_sel[Geo::PER_THREAD], k_off[Geo::PER_THREAD], v_off[Geo::PER_THREAD];
+#pragma unroll
+    for (int i = 0; i < Geo::PER_THREAD; ++i) {
+        const int c = tid + i * 256;
+        const int key = c / (D / 8), kc = c % (D / 8);
+        k_sel[i] = __builtin_amdgcn_readfirstlane(key >> 4);
+        k_off[i] = (key & 15) * D + kc * 8;
+        const int rem = c % (2 * D);
+        v_sel[i] = __builtin_amdgcn_readfirstlane(c / (2 * D));
+        v_off[i] = (rem >> 1) * 16 + (rem & 1) * 8;
+    }
     auto fetch = [&](int b, int kstart) {
         int pg[2];
 #pragma unroll
@@ -131,24 +145,24 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, const bf16_t *__restrict
 #pragma unroll
         for (int i = 0; i < Geo::PER_THREAD; ++i) {
             const int c = tid + i * 256;
-            if (Geo::CHUNKS % 256 != 0 && c >= Geo::CHUNKS) break;
-            const int key = c / (D / 8), kc = c % (D / 8);
-            const size_t kpage = ((size_t)pg[key >> 4] * num_kv_heads + kvh) * (size_t)(16 * D);
-            stage_k[b][i] = *reinterpret_cast<const uint4 *>(k_cache + kpage + (size_t)(key & 15) * D + kc * 8);
-            const int t = c / (2 * D), rem = c % (2 * D);
-            const size_t vpage = ((size_t)pg[t] * num_kv_heads + kvh) * (size_t)(16 * D);
-            stage_v[b][i] = *reinterpret_cast<const uint4 *>(v_cache + vpage + (size_t)(rem >> 1) * 16 + (rem & 1) * 8);
+            if (Geo::CHUNKS % 256 == 0 || c < Geo::CHUNKS) {
+                const size_t kpage = ((size_t)(k_sel[i] ? pg[1] : pg[0]) * num_kv_heads + kvh) * (size_t)(16 * D);
+                stage_k[b][i] = *reinterpret_cast<const uint4 *>(k_cache + kpage + k_off[i]);
+                const size_t vpage = ((size_t)(v_sel[i] ? pg[1] : pg[0]) * num_kv_heads + kvh) * (size_t)(16 * D);
+                stage_v[b][i] = *reinterpret_cast<const uint4 *>(v_cache + vpage + v_off[i]);
+            }
         }
     };
     auto stash = [&](int b, char *buf) {
 #pragma unroll
         for (int i = 0; i < Geo::PER_THREAD; ++i) {
             const int c = tid + i * 256;
-            if (Geo::CHUNKS % 256 != 0 && c >= Geo::CHUNKS) break;
-            const int key = c / (D / 8), kc = c % (D / 8);
-            *reinterpret_cast<uint4 *>(buf + key * Geo::KROW + kc * 16) = stage_k[b][i];
-            const int t = c / (2 * D), rem = c % (2 * D);
-            *reinterpret_cast<uint4 *>(buf + Geo::KBYTES + (rem >> 1) * Geo::VROW + (t * 16 + (rem & 1) * 8) * 2) = stage_v[b][i];
+            if (Geo::CHUNKS % 256 == 0 || c < Geo::CHUNKS) {
+                const int key = c / (D / 8), kc = c % (D / 8);
+                *reinterpret_cast<uint4 *>(buf + key * Geo::KROW + kc * 16) = stage_k[b][i];
+                const int t = c / (2 * D), rem = c % (2 * D);
+                *reinterpret_cast<uint4 *>(buf + Geo::KBYTES + (rem >> 1) * Geo::VROW + (t * 16 + (rem & 1) * 8) * 2) = stage_v[b][i];
+            }
         }
     };
 
