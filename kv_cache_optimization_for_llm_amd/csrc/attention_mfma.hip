@@ -415,21 +415,26 @@ attention_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_
     const int lane = threadIdx.x;
     const float2 *ml = reinterpret_cast<const float2 *>(part_ml) + row * splits;
     const float *po = part_o + row * splits * head_dim;
+    // Every load whose address is known goes out before anything is waited for: this lane's
+    // (max, sum) pairs and the first partial outputs of its first dimension.
+    float2 first = make_float2(-INFINITY, 0.f);
+    if (lane < splits) first = ml[lane];
     float early[MERGE_EARLY];
     const bool j0_ok = lane < head_dim;
 #pragma unroll
     for (int s = 0; s < MERGE_EARLY; ++s)
         early[s] = (j0_ok && s < splits) ? po[(size_t)s * head_dim + lane] : 0.f;
-    float M = -INFINITY;
-    for (int s = lane; s < splits; s += KVA_WAVE) M = fmaxf(M, ml[s].x);
+    float M = first.x;
+    for (int s = lane + KVA_WAVE; s < splits; s += KVA_WAVE) M = fmaxf(M, ml[s].x);
     M = wave_max(M);
     float denom = 0.f;
-    for (int s = lane; s < splits; s += KVA_WAVE) {
-        const float2 v = ml[s];
+    auto weigh = [&](int s, float2 v) {
         const float w = (v.x == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(v.x - M);   // m is kept in the base-2 domain
         w_s[s] = w;
         denom += v.y * w;
-    }
+    };
+    if (lane < splits) weigh(lane, first);
+    for (int s = lane + KVA_WAVE; s < splits; s += KVA_WAVE) weigh(s, ml[s]);
     denom = wave_sum(denom);
     __syncthreads();
     const float inv = 1.f / denom;

@@ -75,18 +75,30 @@ struct SkinnyArgs {
     const int *slots;             // [M] cache slot per token (negative: no write), null: no cache write
     bf16_t *k_cache, *v_cache;    // [pages, nkv, page, d] and [pages, nkv, d, page]
     int nq, nkv, head_dim, page_size;
+    // half tiles: a tile group takes 8 of its tiles' 16 rows (see choose_half_tiles)
+    int half;
 };
 
-template <int MT, int NTW, int EPI>
-__global__ void gemm_skinny_kernel(const SkinnyArgs a) {
-    extern __shared__ float red[];
+// XL: the waves of a workgroup that work on the same K range (one per tile group) share X through
+// LDS instead of each loading it (see the main loop).
+template <int MT, int NTW, int EPI, bool XL = false>
+__global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const SkinnyArgs a) {
+    extern __shared__ __align__(16) float red[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int waves = blockDim.x >> 6;
     const int k_waves = a.k_waves;
     const int groups_per_wg = waves / k_waves;                 // tile groups (NTW tiles) per workgroup
-    const int group = blockIdx.x * groups_per_wg + wave / k_waves;
     const int kpart = wave % k_waves;
     const int r = lane & 15, g = lane >> 4;
+    // With half tiles two waves (of different workgroups) share a tile group: each takes 8 of the
+    // 16 rows of its tiles.  The upper 8 lanes-rows of the matrix-core operand repeat the lower
+    // ones, so lane groups 2 and 3 end up with copies of the results and store nothing.
+    const int unit = blockIdx.x * groups_per_wg + wave / k_waves;
+    const int group = a.half ? unit >> 1 : unit;
+    const int hrow = a.half ? (unit & 1) * 8 : 0;
+    const int wrow = a.half ? hrow + (r & 7) : r;               // row of a tile that lane (r, g) loads
+    const int orow = a.half ? hrow + 4 * (g & 1) : 4 * g;       // first of the 4 rows whose results it holds
+    const bool lane_on = !a.half || g < 2;
     const int rows = EPI == EPI_SWIGLU ? a.inter : a.N;        // output columns
     const int n_tiles = (rows + 15) / 16;
     // EPI_SWIGLU: a wave's two tiles are the gate tile and the up tile of the same columns
@@ -119,7 +131,7 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
         }
         const int last = (EPI == EPI_SWIGLU ? 2 * n_tiles : n_tiles) - 1;
         if (tile > last) tile = last;
-        wp[t] = a.W + (size_t)tile * (size_t)(K / 32) * 512 + (4 * r + g) * 8;
+        wp[t] = a.W + (size_t)tile * (size_t)(K / 32) * 512 + (4 * wrow + g) * 8;
     }
     const bf16_t *xr[MT];
 #pragma unroll
@@ -135,11 +147,16 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
         for (int mt = 0; mt < MT; ++mt) acc[t][mt] = gf32x4{0.f, 0.f, 0.f, 0.f};
 
     // The first wave of a tile group also needs, per token, the sum of squares that finishes the
-    // input norm.  The loads are issued here, ahead of the main loop, so their latency is hidden
-    // behind the stream of W: lane group g adds a contiguous quarter of the partial sums.
+    // input norm: lane group g adds a contiguous quarter of the partial sums.  The loads are
+    // issued here, ahead of the main loop, and (for up to 32 tokens) their values are only added
+    // after it, so this wave starts streaming W as early as the others; with more token tiles
+    // there are no registers to hold them and they are added at once.
+    constexpr int DV = (MT == 1 && NTW <= 2) ? 16 : ((MT == 1 || (MT == 2 && NTW <= 2)) ? 8 : 0);   // vectors of 4 sums held per token tile
+    float4 dv[MT][DV > 0 ? DV : 1];
+    int dv_end[MT];
     float ssum[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) ssum[mt] = 0.f;
+    for (int mt = 0; mt < MT; ++mt) { ssum[mt] = 0.f; dv_end[mt] = 0; }
     if (a.sumsq != nullptr && kpart == 0 && group_ok) {
         const int parts = a.sumsq_parts;
         const int q = (parts + 3) / 4;
@@ -148,9 +165,19 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
             const int m = mt * 16 + r;
             if (m >= a.M) continue;
             const float *sp = a.sumsq + (size_t)m * parts;
-            const int lo = g * q, hi = (lo + q < parts) ? lo + q : parts;
+            int lo = g * q;
+            const int hi = (lo + q < parts) ? lo + q : parts;
             float s = 0.f;
             if ((parts & 15) == 0) {
+                if (DV > 0) {
+                    dv_end[mt] = hi - lo;
+#pragma unroll
+                    for (int j = 0; j < DV; ++j) {
+                        const int p = lo + 4 * j;
+                        dv[mt][j] = *reinterpret_cast<const float4 *>(sp + (p < hi ? p : hi - 4));
+                    }
+                    lo += 4 * DV;
+                }
                 // 8 vectors of 4 at a time, all loaded before any is added (a load past the
                 // lane's quarter repeats its last vector and is not counted)
                 for (int base = lo; base < hi; base += 32) {
@@ -177,7 +204,9 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
     int pre_slot[MT];
     float4 pre_cos[MT], pre_sin[MT];
     uint2 pre_hidden[MT];
-    float pre_wn[4] = {1.f, 1.f, 1.f, 1.f};
+    // the next norm's weight as loaded (converted in the epilogue: a conversion here would wait for the load)
+    float4 pre_wn_f = make_float4(1.f, 1.f, 1.f, 1.f);
+    uint2 pre_wn_b = make_uint2(0x3f803f80u, 0x3f803f80u);
     constexpr bool kPreRope = EPI == EPI_ROPE && MT <= 2;
     constexpr bool kPreResid = EPI == EPI_RESID && NTW == 1 && MT <= 2;
 #pragma unroll
@@ -187,47 +216,147 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
         pre_sin[mt] = make_float4(0.f, 0.f, 0.f, 0.f);
         pre_hidden[mt] = make_uint2(0u, 0u);
     }
+    int pre_pos[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) pre_pos[mt] = 0;
     if (kPreRope && kpart == 0 && group_ok) {
+        // slot and position now; the cos/sin entries, whose address needs the position, after the
+        // main loop (a wait here would hold back this wave's stream of W)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             const int m = mt * 16 + r;
             if (m >= a.M) continue;
             if (a.slots != nullptr && rope_head >= a.nq) pre_slot[mt] = a.slots[m];
-            if (rope_rotated && a.cos_t != nullptr) {
-                const size_t at = (size_t)a.positions[m] * (a.head_dim / 2) + rope_j * 16 + 4 * g;
-                pre_cos[mt] = *reinterpret_cast<const float4 *>(a.cos_t + at);
-                pre_sin[mt] = *reinterpret_cast<const float4 *>(a.sin_t + at);
-            }
+            if (rope_rotated && a.cos_t != nullptr) pre_pos[mt] = a.positions[m];
         }
     }
-    const bool resid_vec = kPreResid && (a.N % 4 == 0) && tile0 * 16 + 4 * g + 3 < rows;
+    const bool resid_vec = kPreResid && (a.N % 4 == 0) && tile0 * 16 + orow + 3 < rows;
     if (kPreResid && kpart == 0 && group_ok && resid_vec) {
-        const int n = tile0 * 16 + 4 * g;
+        const int n = tile0 * 16 + orow;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             const int m = mt * 16 + r;
             if (m < a.M) pre_hidden[mt] = *reinterpret_cast<const uint2 *>(a.hidden + (size_t)m * a.N + n);
         }
-        if (a.next_w != nullptr) {
-            if (a.next_w_f32) {
-                const float4 wv = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(a.next_w) + n);
-                pre_wn[0] = wv.x; pre_wn[1] = wv.y; pre_wn[2] = wv.z; pre_wn[3] = wv.w;
-            } else {
-                const uint2 wv = *reinterpret_cast<const uint2 *>(reinterpret_cast<const bf16_t *>(a.next_w) + n);
-                pre_wn[0] = bf16_bits_to_float((uint16_t)(wv.x & 0xffffu));
-                pre_wn[1] = bf16_bits_to_float((uint16_t)(wv.x >> 16));
-                pre_wn[2] = bf16_bits_to_float((uint16_t)(wv.y & 0xffffu));
-                pre_wn[3] = bf16_bits_to_float((uint16_t)(wv.y >> 16));
-            }
-        }
+        // both forms are loaded, one of them from a place that is always there (X), so that no
+        // branch joins here with a load in flight
+        const bool wf = a.next_w != nullptr && a.next_w_f32, wb = a.next_w != nullptr && !a.next_w_f32;
+        pre_wn_f = *(wf ? reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(a.next_w) + n)
+                        : reinterpret_cast<const float4 *>(a.X));
+        pre_wn_b = *(wb ? reinterpret_cast<const uint2 *>(reinterpret_cast<const bf16_t *>(a.next_w) + n)
+                        : reinterpret_cast<const uint2 *>(a.X));
     }
 
     // ---- the main loop.  Rows of X past M are read from row 0 instead (their columns of the
-    // result are never stored), so the loop body has no branch.  Left rolled: the compiler
-    // pipelines it by one step, which streams long K ranges best (straight-line chunks of 4-8
-    // steps with all loads up front were measured equal for short ranges and 10-20 % slower for
-    // the vocabulary-sized product).
-    if (group_ok) {
+    // result are never stored), so the loop body has no branch.  One step per turn and wave: what
+    // bounds these products is how much a compute unit can have in flight (about 32 KiB, or
+    // 33 GB/s per unit at the latency seen here), which its 16 waves reach with one step each;
+    // chunks of 2-8 steps with all loads up front were measured equal for the per-layer matrices
+    // and 10-20 % slower for the vocabulary-sized one.  What counts is that every compute unit
+    // has a workgroup.
+    if constexpr (XL) {
+        // More than 16 tokens: every wave needs MT fragments of X per fragment of W, and loading
+        // them per wave makes X (from L2, in half-used cache lines) the larger stream.  Here the
+        // waves of the workgroup that share a K range stage X through LDS: chunks of 64 of K,
+        // each loaded once per workgroup in full 128-byte lines, double-buffered, one barrier per
+        // chunk.  A token's row of a chunk is 128 bytes; tokens r and r + 8 of a tile lie next to
+        // each other and the 16-byte units of a row are XOR-swizzled with the token, so that the
+        // operand reads (16 tokens x 16 bytes at the same K) touch every bank once.  W is
+        // fetched two chunks ahead into two register buffers.  All waves run the loop (barriers);
+        // a wave past the last tile group computes a copy of the last one and stores nothing.
+        constexpr int KC = 64, ROWS = MT * 16, UNITS = ROWS * (KC / 8);
+        const int J = groups_per_wg;
+        const int sj = wave / k_waves;                          // place among the waves of this K range
+        char *xbase = reinterpret_cast<char *>(red) + (size_t)kpart * 2 * ROWS * 128;
+        const int n_chunks = (kper + KC - 1) / KC;
+        // (named registers, not an array: an array here ends up in scratch memory)
+        uint4 xs0 = make_uint4(0, 0, 0, 0), xs1 = xs0, xs2 = xs0, xs3 = xs0;
+        auto load_unit = [&](int i, int c) -> uint4 {
+            int u = (i * J + sj) * 64 + lane;
+            if (u >= UNITS) u = 0;
+            const int q = u >> 3, c16 = u & 7;
+            const int row = (q & ~15) | ((q >> 1) & 7) | ((q & 1) << 3);
+            int k = kbeg + c * KC + c16 * 8;
+            if (k >= kend) k = kbeg;
+            return *reinterpret_cast<const uint4 *>(a.X + (size_t)(row < a.M ? row : 0) * a.ldx + k);
+        };
+        auto store_unit = [&](int i, int c, const uint4 &v) {
+            const int u = (i * J + sj) * 64 + lane;
+            const int q = u >> 3, c16 = u & 7;
+            const int row = (q & ~15) | ((q >> 1) & 7) | ((q & 1) << 3);
+            if (u < UNITS)
+                *reinterpret_cast<uint4 *>(xbase + (c & 1) * ROWS * 128 + q * 128 + ((c16 ^ (row & 7)) << 4)) = v;
+        };
+        auto load_x = [&](int c) {
+            xs0 = load_unit(0, c);
+            if constexpr (MT > 1) xs1 = load_unit(1, c);
+            if constexpr (MT > 2) xs2 = load_unit(2, c);
+            if constexpr (MT > 3) xs3 = load_unit(3, c);
+        };
+        auto store_x = [&](int c) {
+            store_unit(0, c, xs0);
+            if constexpr (MT > 1) store_unit(1, c, xs1);
+            if constexpr (MT > 2) store_unit(2, c, xs2);
+            if constexpr (MT > 3) store_unit(3, c, xs3);
+        };
+        // W of a chunk goes straight to registers, NB chunks ahead (four were measured no faster)
+        constexpr int NB = 2;
+        GFrag8 wbuf[NB][2][NTW];
+        auto load_w = [&](GFrag8 (&w)[2][NTW], int c) {
+#pragma unroll
+            for (int st = 0; st < 2; ++st) {
+                int k = kbeg + c * KC + st * 32;
+                if (k >= kend) k = kbeg;                        // half a chunk at the end: loaded from a valid place, not used
+#pragma unroll
+                for (int t = 0; t < NTW; ++t) w[st][t].u4 = *reinterpret_cast<const uint4 *>(wp[t] + (size_t)k * 16);
+            }
+        };
+        auto compute = [&](GFrag8 (&w)[2][NTW], int c) {
+            const char *buf = xbase + (c & 1) * ROWS * 128 + (((r & 7) << 1) + (r >> 3)) * 128;
+#pragma unroll
+            for (int st = 0; st < 2; ++st) {
+                if (kbeg + c * KC + st * 32 < kend) {
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) {
+                        GFrag8 x;
+                        x.u4 = *reinterpret_cast<const uint4 *>(buf + mt * 16 * 128 + (((st * 4 + g) ^ (r & 7)) << 4));
+#pragma unroll
+                        for (int t = 0; t < NTW; ++t)
+                            acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[st][t].v, x.v, acc[t][mt], 0, 0, 0);
+                    }
+                }
+            }
+        };
+        load_x(0);
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+            if (b < n_chunks) load_w(wbuf[b], b);
+        // NB chunks per turn while every load of the turn exists: no branch in the body, so the
+        // waits count exactly and the loads issued last stay in flight across them.
+        int c = 0;
+        for (; c + 2 * NB - 1 < n_chunks; c += NB) {
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                store_x(c + b);
+                __syncthreads();
+                load_x(c + b + 1);
+                compute(wbuf[b], c + b);
+                load_w(wbuf[b], c + b + NB);
+            }
+        }
+        // the last chunks (fewer than 2 NB): X of chunk c is loaded, W of c + b in buffer b
+#pragma unroll
+        for (int b = 0; b < 2 * NB - 1; ++b) {
+            if (c + b < n_chunks) {
+                store_x(c + b);
+                __syncthreads();
+                if (c + b + 1 < n_chunks) load_x(c + b + 1);
+                compute(wbuf[b % NB], c + b);
+                if (c + b + NB < n_chunks) load_w(wbuf[b % NB], c + b + NB);
+            }
+        }
+        __syncthreads();                                        // the sums below reuse the buffer
+    } else if (group_ok) {
 #pragma unroll 8
         for (int k = kbeg; k < kend; k += 32) {
             GFrag8 w[NTW];
@@ -241,6 +370,26 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
                 for (int t = 0; t < NTW; ++t)
                     acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[t].v, x.v, acc[t][mt], 0, 0, 0);
             }
+        }
+    }
+
+    if (kPreRope && kpart == 0 && group_ok && rope_rotated && a.cos_t != nullptr) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            if (mt * 16 + r >= a.M) continue;
+            const size_t at = (size_t)pre_pos[mt] * (a.head_dim / 2) + rope_j * 16 + orow;
+            pre_cos[mt] = *reinterpret_cast<const float4 *>(a.cos_t + at);
+            pre_sin[mt] = *reinterpret_cast<const float4 *>(a.sin_t + at);
+        }
+    }
+    if (DV > 0) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            float s = ssum[mt];
+#pragma unroll
+            for (int j = 0; j < DV; ++j)
+                s += (4 * j < dv_end[mt]) ? (dv[mt][j].x + dv[mt][j].y) + (dv[mt][j].z + dv[mt][j].w) : 0.f;
+            ssum[mt] = s;
         }
     }
 
@@ -289,7 +438,7 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             const int m = mt * 16 + r;
-            if (m >= a.M) continue;
+            if (m >= a.M || !lane_on) continue;
             float va[4], vb[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -302,7 +451,7 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
             const int page = slot >= 0 ? slot / a.page_size : 0;
             const int off = slot >= 0 ? slot - page * a.page_size : 0;
             if (rope_rotated) {
-                const int f = rope_j * 16 + 4 * g;             // feature in [0, d/2); partner f + d/2
+                const int f = rope_j * 16 + orow;              // feature in [0, d/2); partner f + d/2
                 float o1[4], o2[4];
                 if (a.cos_t != nullptr) {
                     float4 c4 = pre_cos[mt], s4 = pre_sin[mt];
@@ -336,7 +485,7 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
                                (uint32_t)float_to_bf16_bits(o2[2]) | ((uint32_t)float_to_bf16_bits(o2[3]) << 16));
             } else {
                 if (slot < 0) continue;
-                const int f = rope_j * 32 + 4 * g;             // value features f..f+3 and f+16..f+19
+                const int f = rope_j * 32 + orow;              // value features f..f+3 and f+16..f+19
                 bf16_t *dst = a.v_cache + (((size_t)page * a.nkv + (rope_head - a.nq - a.nkv)) * D + f) * a.page_size + off;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
@@ -352,7 +501,7 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
     for (int t = 0; t < out_tiles; ++t) {
         const int tile = tile0 + t;
         if (tile >= n_tiles) break;
-        const int n = tile * 16 + 4 * g;                   // first of this lane's 4 outputs
+        const int n = tile * 16 + orow;                    // first of this lane's 4 outputs
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             const int m = mt * 16 + r;
@@ -369,7 +518,7 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
             }
             if (EPI == EPI_RESID) {
                 float ss = 0.f;
-                if (m_ok) {
+                if (m_ok && lane_on) {
                     bf16_t *hp = a.hidden + (size_t)m * a.N + n;
                     bf16_t *sp = a.scaled_out + (size_t)m * a.N + n;
                     if (n + 3 < rows && (a.N % 4 == 0)) {
@@ -378,7 +527,15 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
                                              bf16_bits_to_float((uint16_t)(hv.x >> 16)),
                                              bf16_bits_to_float((uint16_t)(hv.y & 0xffffu)),
                                              bf16_bits_to_float((uint16_t)(hv.y >> 16))};
-                        float wn[4] = {pre_wn[0], pre_wn[1], pre_wn[2], pre_wn[3]};
+                        float wn[4] = {pre_wn_f.x, pre_wn_f.y, pre_wn_f.z, pre_wn_f.w};
+                        if (a.next_w == nullptr) {
+                            wn[0] = wn[1] = wn[2] = wn[3] = 1.f;
+                        } else if (kPreResid && !a.next_w_f32) {
+                            wn[0] = bf16_bits_to_float((uint16_t)(pre_wn_b.x & 0xffffu));
+                            wn[1] = bf16_bits_to_float((uint16_t)(pre_wn_b.x >> 16));
+                            wn[2] = bf16_bits_to_float((uint16_t)(pre_wn_b.y & 0xffffu));
+                            wn[3] = bf16_bits_to_float((uint16_t)(pre_wn_b.y >> 16));
+                        }
                         if (!kPreResid && a.next_w != nullptr) {
                             if (a.next_w_f32) {
                                 const float4 wv = *reinterpret_cast<const float4 *>(
@@ -421,10 +578,13 @@ __global__ void gemm_skinny_kernel(const SkinnyArgs a) {
                     }
                 }
                 ss = quad_rows_sum(ss);
-                if (m_ok && g == 0) a.sumsq_out[(size_t)m * n_tiles + tile] = ss;
+                if (m_ok && g == 0) {
+                    if (a.half) a.sumsq_out[(size_t)m * (2 * n_tiles) + 2 * tile + (hrow >> 3)] = ss;
+                    else a.sumsq_out[(size_t)m * n_tiles + tile] = ss;
+                }
                 continue;
             }
-            if (!m_ok) continue;
+            if (!m_ok || !lane_on) continue;
             if (a.out_f32) {
                 float *dst = reinterpret_cast<float *>(a.Y) + (size_t)m * a.ldy + n;
                 if (n + 3 < rows && (a.ldy % 4 == 0)) {
@@ -467,12 +627,40 @@ static int choose_k_waves(int groups, int K, int ntw) {
     return kw;
 }
 
+// A compute unit streams some 25 GB/s of weights whatever its waves do, so a matrix with at most
+// half as many tile groups as the chip has compute units is spread over twice as many workgroups:
+// each takes half (8) of the rows of its tiles.  Depends on the matrix only, never on M.
+static int compute_units() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cus = n;
+    }
+    return cus;
+}
+static int choose_half_tiles(int groups) { return groups * 2 <= compute_units() ? 1 : 0; }
+
 extern "C" int kva_gemm_skinny_supported(int M, int N, int K) {
     return (M >= 1 && M <= 64 && N >= 1 && K >= 32 && K % 32 == 0) ? 1 : 0;
 }
 
 // Number of partial sums of squares per token that an EPI_RESID product with N columns writes.
-extern "C" int kva_gemm_skinny_sumsq_parts(int N) { return (N + 15) / 16; }
+extern "C" int kva_gemm_skinny_sumsq_parts(int N) {
+    const int n_tiles = (N + 15) / 16;
+    return choose_half_tiles(n_tiles) ? 2 * n_tiles : n_tiles;
+}
+
+template <int NTW, int EPI>
+static void launch_xl(const SkinnyArgs &a, dim3 grid, dim3 block, size_t lds, hipStream_t stream) {
+    switch ((a.M + 15) / 16) {
+    case 2: hipLaunchKernelGGL((gemm_skinny_kernel<2, NTW, EPI, true>), grid, block, lds, stream, a); break;
+    case 3: hipLaunchKernelGGL((gemm_skinny_kernel<3, NTW, EPI, true>), grid, block, lds, stream, a); break;
+    default: hipLaunchKernelGGL((gemm_skinny_kernel<4, NTW, EPI, true>), grid, block, lds, stream, a); break;
+    }
+}
 
 template <int NTW, int EPI>
 static void launch_mt(const SkinnyArgs &a, dim3 grid, dim3 block, size_t lds, hipStream_t stream) {
@@ -521,15 +709,33 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
     else if (n_tiles >= 4096) ntw = 4;
     else if (n_tiles >= 2048) ntw = 2;
     const int out_tiles = mode == 2 ? 1 : ntw;
-    const int groups = (n_tiles + out_tiles - 1) / out_tiles;
+    int groups = (n_tiles + out_tiles - 1) / out_tiles;
+    a.half = mode == 3 ? choose_half_tiles(groups) : 0;
+    if (a.half) groups *= 2;
     int kw = choose_k_waves(groups, K, ntw);
+    int groups_per_wg = kw >= 4 ? 1 : 4 / kw;
+    // More than 16 tokens and several tiles per wave: workgroups of several tile groups that
+    // share X through LDS (at most 4 K ranges of 2 x 64 tokens x 128 bytes: 64 KiB).
+    const bool xl = M > 16 && ntw >= 2 && groups >= 2;
+    if (xl) {
+        kw = kw < 4 ? kw : 4;
+        groups_per_wg = kw == 4 ? 2 : 4;
+    }
     a.k_waves = kw;
-    const int groups_per_wg = kw >= 4 ? 1 : 4 / kw;
     const int waves = kw * groups_per_wg;
-    const size_t lds = kw > 1 ? (size_t)waves * ntw * 64 * 4 * sizeof(float) : 0;
-    KVA_REQUIRE(lds <= 64 * 1024, "gemm_skinny: reduction buffer of %zu bytes does not fit", lds);
+    size_t lds = kw > 1 ? (size_t)waves * ntw * 64 * 4 * sizeof(float) : 0;
+    if (xl) {
+        const size_t stage = (size_t)kw * 2 * ((M + 15) / 16 * 16) * 128;
+        lds = lds > stage ? lds : stage;
+    }
+    KVA_REQUIRE(lds <= 64 * 1024, "gemm_skinny: LDS buffer of %zu bytes does not fit", lds);
     dim3 grid((groups + groups_per_wg - 1) / groups_per_wg), block(64 * waves);
-    if (mode == 2) launch_mt<2, EPI_SWIGLU>(a, grid, block, lds, stream);
+    if (xl) {
+        if (mode == 2) launch_xl<2, EPI_SWIGLU>(a, grid, block, lds, stream);
+        else if (ntw == 4) launch_xl<4, EPI_PLAIN>(a, grid, block, lds, stream);
+        else launch_xl<2, EPI_PLAIN>(a, grid, block, lds, stream);
+    }
+    else if (mode == 2) launch_mt<2, EPI_SWIGLU>(a, grid, block, lds, stream);
     else if (mode == 3) launch_mt<1, EPI_RESID>(a, grid, block, lds, stream);
     else if (ntw == 4) launch_mt<4, EPI_PLAIN>(a, grid, block, lds, stream);
     else if (ntw == 2) launch_mt<2, EPI_PLAIN>(a, grid, block, lds, stream);
@@ -570,13 +776,15 @@ extern "C" int kva_gemm_skinny_qkv_rope(void *q_out, int ldq, const void *X, con
     a.cos_t = cos_t; a.sin_t = sin_t; a.positions = positions; a.slots = slots;
     a.k_cache = (bf16_t *)k_cache; a.v_cache = (bf16_t *)v_cache;
     a.nq = nq; a.nkv = nkv; a.head_dim = head_dim; a.page_size = page_size;
-    const int groups = a.N / 32;
+    int groups = a.N / 32;
+    a.half = choose_half_tiles(groups);
+    if (a.half) groups *= 2;
     const int kw = choose_k_waves(groups, K, 2);
     a.k_waves = kw;
     const int groups_per_wg = kw >= 4 ? 1 : 4 / kw;
     const int waves = kw * groups_per_wg;
-    const size_t lds = kw > 1 ? (size_t)waves * 2 * 64 * 4 * sizeof(float) : 0;
-    KVA_REQUIRE(lds <= 64 * 1024, "gemm_skinny_qkv_rope: reduction buffer of %zu bytes does not fit", lds);
+    size_t lds = kw > 1 ? (size_t)waves * 2 * 64 * 4 * sizeof(float) : 0;
+    KVA_REQUIRE(lds <= 64 * 1024, "gemm_skinny_qkv_rope: LDS buffer of %zu bytes does not fit", lds);
     dim3 grid((groups + groups_per_wg - 1) / groups_per_wg), block(64 * waves);
     launch_mt<2, EPI_ROPE>(a, grid, block, lds, stream);
     KVA_CHECK_LAUNCH("gemm_skinny_qkv_rope");

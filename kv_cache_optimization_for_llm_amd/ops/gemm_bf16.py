@@ -27,18 +27,23 @@ from . import kernels as K
 SKINNY_MAX_ROWS = 16            # every shape
 SKINNY_MID_ROWS = 32            # small or tall matrices
 SKINNY_MID_ELEMENTS = 1 << 23
-SKINNY_WIDE_ROWS = 48           # vocabulary-sized matrices
+SKINNY_WIDE_ROWS = 64           # matrices whose waves share X through LDS
 SKINNY_WIDE_N = 32768
 
 
-def use_skinny(m: int, n: int, k: int) -> bool:
+def use_skinny(m: int, n: int, k: int, gated: bool = False) -> bool:
+    """``gated``: the weight is a joined [gate; up] matrix whose product is taken with the
+    activation fused."""
     if not K.gemm_skinny_supported(m, n, k):
         return False
     if m <= SKINNY_MAX_ROWS:
         return True
     if m <= SKINNY_MID_ROWS and (n * k <= SKINNY_MID_ELEMENTS or n >= 4 * k):
         return True
-    return m <= SKINNY_WIDE_ROWS and n >= SKINNY_WIDE_N
+    import os
+    if os.environ.get("KVA_POLICY") == "old":
+        return m <= 48 and n >= SKINNY_WIDE_N
+    return m <= SKINNY_WIDE_ROWS and (n >= SKINNY_WIDE_N or (gated and n >= 4 * k))
 
 
 def linear_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, tiled=None) -> torch.Tensor:

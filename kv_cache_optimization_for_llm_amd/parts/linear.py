@@ -25,6 +25,7 @@ class Linear:
             raise ValueError(f"Linear weight must be 2-D, got {tuple(weight.shape)}")
         self.weight = weight.contiguous()
         self.out_features, self.in_features = weight.shape
+        self.halves = halves
         # a second, tiled copy for the few-rows kernel (decode); the plain layout serves prompts
         self.tiled = None
         if weight.is_cuda and weight.dtype == torch.bfloat16 and self.in_features % 32 == 0:
@@ -35,7 +36,7 @@ class Linear:
         in its epilogue for these rows (bf16 everywhere, few rows)."""
         from ..ops.gemm_bf16 import use_skinny
         return (self.tiled is not None and x.dtype == torch.bfloat16
-                and use_skinny(x.shape[0], self.out_features, self.in_features))
+                and use_skinny(x.shape[0], self.out_features, self.in_features, self.halves == 2))
 
     def into_residual(self, x, tail: BranchTail) -> Optional[NormedRows]:
         """hidden += x @ W^T in place and the sum prepared for ``tail.norm``; ``None`` when this
