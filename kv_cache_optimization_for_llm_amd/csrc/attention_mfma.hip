@@ -148,6 +148,10 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
     const uint32_t k_lane = (uint32_t)(r * D + g * (KSTEP / 4)) * 2u;          // bytes
     const uint32_t v_lane = (uint32_t)(r * 16 + 4 * g) * 2u;                   // bytes
     constexpr uint32_t v_tile_stride = 16u * 16u * 2u;                         // 16 value dims
+    // One row tile per item is how decoded tokens (and short portions) run: their keys and values
+    // are read once per step, by this wave alone, and go past the caches.  Prompt items share
+    // theirs with the other row tiles of the request, through L2.
+    constexpr bool STREAM = RT == 1;
     auto load_block = [&](BlockFrags &f, int kstart) {
         if constexpr (FAST) {
             // the index is uniform: said so explicitly, the lookups are scalar loads (both issued
@@ -167,13 +171,16 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
 #pragma unroll
                 for (int ks = 0; ks < NKS; ++ks) {
                     if (KSTEP == 32)
-                        f.k8[t][ks].u4 = *reinterpret_cast<const uint4 *>(kb + k_lane + ks * 64);
+                        f.k8[t][ks].u4 = STREAM ? load_streamed_u4(kb + k_lane + ks * 64)
+                                                : *reinterpret_cast<const uint4 *>(kb + k_lane + ks * 64);
                     else
-                        f.k4[t][ks].u2 = *reinterpret_cast<const uint2 *>(kb + k_lane + ks * 32);
+                        f.k4[t][ks].u2 = STREAM ? load_streamed_u2(kb + k_lane + ks * 32)
+                                                : *reinterpret_cast<const uint2 *>(kb + k_lane + ks * 32);
                 }
 #pragma unroll
                 for (int dt = 0; dt < NDT; ++dt)
-                    f.v[dt].u2[t] = *reinterpret_cast<const uint2 *>(vb + v_lane + dt * v_tile_stride);
+                    f.v[dt].u2[t] = STREAM ? load_streamed_u2(vb + v_lane + dt * v_tile_stride)
+                                           : *reinterpret_cast<const uint2 *>(vb + v_lane + dt * v_tile_stride);
             }
             return;
         }

@@ -78,6 +78,20 @@ __device__ inline float wave_max(float v) {
     return v;
 }
 
+// Loads with the non-temporal hint, for data that is read once per kernel and will have left the
+// caches before it is wanted again (weights at decode time, the KV pages of decoded tokens): what
+// else lives in L2 stays there.
+typedef unsigned int kva_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int kva_u32x2 __attribute__((ext_vector_type(2)));
+__device__ inline uint4 load_streamed_u4(const void *p) {
+    const kva_u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const kva_u32x4 *>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ inline uint2 load_streamed_u2(const void *p) {
+    const kva_u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const kva_u32x2 *>(p));
+    return make_uint2(v.x, v.y);
+}
+
 // Reductions over the four lanes {r, r + 16, r + 32, r + 48} (r = lane % 16), every one of them
 // getting the result.  v_permlane16_swap / v_permlane32_swap exchange 16- and 32-lane halves
 // between two registers in the vector ALU (no trip through LDS as a wave shuffle takes): from two

@@ -308,7 +308,7 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
                 int k = kbeg + c * KC + st * 32;
                 if (k >= kend) k = kbeg;                        // half a chunk at the end: loaded from a valid place, not used
 #pragma unroll
-                for (int t = 0; t < NTW; ++t) w[st][t].u4 = *reinterpret_cast<const uint4 *>(wp[t] + (size_t)k * 16);
+                for (int t = 0; t < NTW; ++t) w[st][t].u4 = load_streamed_u4(wp[t] + (size_t)k * 16);
             }
         };
         auto compute = [&](GFrag8 (&w)[2][NTW], int c) {
@@ -361,7 +361,7 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
         for (int k = kbeg; k < kend; k += 32) {
             GFrag8 w[NTW];
 #pragma unroll
-            for (int t = 0; t < NTW; ++t) w[t].u4 = *reinterpret_cast<const uint4 *>(wp[t] + (size_t)k * 16);
+            for (int t = 0; t < NTW; ++t) w[t].u4 = load_streamed_u4(wp[t] + (size_t)k * 16);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 GFrag8 x;
