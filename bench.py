@@ -160,7 +160,7 @@ def main():
             points[f"decode_b{b}_p512_g256"] = round(b * 240 / d, 1)
 
     out = {
-        "metric": "decode tok/s at batch 8 (context 8192), Llama-3.2-1B shape", "value": round(value, 1),
+        "metric": f"decode tok/s at batch {args.batch} (context {ctx}), Llama-3.2-1B shape", "value": round(value, 1),
         "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic: random weights N(0,0.02), seeded uniform token ids (prompts are prefilled, then decoded)",

@@ -81,7 +81,7 @@ def attention(args) -> None:
                  for c in caches]
     else:
         tiles = 2 if args.tokens else 1
-        pair = bool(args.tokens) and len(meta) * nkv >= 2048
+        pair = bool(args.tokens) and len(meta) * nkv >= 2048 and not args.no_pair
         calls = [lambda c=c: K.attention_mfma(qkv, nq * d, out, c[0], c[1], table, ent, row0, seat, qs, sp, nq, nkv,
                                               d, scale, 0, splits, per, tiles, pair, meta_d) for c in caches]
     us = _time(calls, args.reps)
@@ -139,6 +139,7 @@ def main(argv=None) -> int:
     a.add_argument("--kv-heads", type=int, default=8)
     a.add_argument("--head-dim", type=int, default=64)
     a.add_argument("--reps", type=int, default=20)
+    a.add_argument("--no-pair", action="store_true", help="wave kernel: never give a wave two items")
     g = sub.add_parser("gemm")
     g.add_argument("--shape", choices=sorted(GEMM_SHAPES), default="gate_up")
     g.add_argument("--rows", type=int, default=8)
