@@ -16,8 +16,15 @@
 // a workgroup (partials summed through LDS in a fixed order) so that narrow matrices still put
 // about 2048 waves on the 256 compute units.
 //
-// A column of the result depends only on its own token's row of X: results do not change with
-// the batch.
+// A column of the result depends only on its own token's row of X, and with at most 16 rows the
+// order of its sum does not depend on M: bitwise the same result in any batch that small.
+//
+// Two more shapes of the same loop.  Above 16 rows (gated and vocabulary-sized products) the waves
+// of a workgroup that work on the same K range stage X through LDS, once for all of them, instead
+// of each loading MT fragments of X per fragment of W.  Matrices with at most half as many tile
+// groups as the chip has compute units are cut into half tiles: two workgroups share a tile, each
+// taking 8 of its 16 rows, because a compute unit sustains only some 25 GB/s of a stream from
+// memory and the chip's bandwidth needs all of them.
 //
 // Row scaling.  With `sumsq` the rows of X are un-normalised norm inputs: X = round(h * w_norm)
 // and sumsq[m, 0..parts) are partial sums of h[m,:]^2; the product is multiplied by
@@ -610,7 +617,8 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
 }
 
 // k_waves: how many wavefronts share one tile group's K range.  Depends on N and K only, never
-// on M, so a token's result does not depend on the batch it is in.  These products are bound by
+// on M, so a token's result does not depend on the batch it is in (the launcher cuts it to 4 where
+// the waves share X through LDS, above 16 rows: that changes the order of the sum, not more).  These products are bound by
 // memory latency until the waves together keep tens of megabytes in flight, so K is cut as deep
 // as a workgroup allows (16 waves) while a wave keeps at least 4 steps of 32, the chip is not
 // oversubscribed (4096 waves) and the waves do not already cover the bandwidth-delay product.
