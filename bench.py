@@ -82,6 +82,7 @@ def main():
         cfg["num_hidden_layers"] = args.layers
     max_batch = 64 if not args.skip_points else args.batch
     ctx = args.context
+    cfg["max_position_embeddings"] = max(cfg["max_position_embeddings"], ctx)      # a longer --context
     # room for max_batch requests at the context, one more page each for the tokens decoded
     pool = max_batch * (ctx + 2 * PAGE)
     engine = Engine(None, EngineOptions(dtype="bfloat16", page_size=PAGE, cache_tokens=pool,
@@ -112,7 +113,10 @@ def main():
         for _ in range(warmup):
             runner.step()
         torch.cuda.synchronize()
-        assert len(sched.running) == batch and not any(s.prefilling for s in sched.running)
+        if len(sched.running) != batch or any(s.prefilling for s in sched.running):
+            raise SystemExit(f"bench: {len(sched.running)} of {batch} requests are decoding after the prompts "
+                             f"(waiting {len(sched.waiting)}, preemptions {sched.preemptions}): the pool or the "
+                             f"token budget does not fit context {context}")
         ctx0 = sum(s.computed for s in sched.running) / batch
         t0 = time.perf_counter()
         for _ in range(steps):
