@@ -1,0 +1,151 @@
+// Y[M,N] = X[M,K] * W[N,K]^T for many rows (prompt portions, large decode batches): the vendor
+// GEMM library, hipBLASLt, called directly.
+//
+// Stands where the reference calls cublasGemmEx (base/src/engine.cu:1040-1117).  bf16 operands,
+// fp32 accumulation, bf16 or fp32 result.  What this file adds to calling the library through a
+// tensor framework is only that everything that depends on the shape alone is looked up once:
+// the descriptors, the layouts and the algorithm the library's heuristic picks are kept per
+// (device, M, N, K, strides, result type), so a call costs a hash lookup and the launch, a few
+// microseconds of host time instead of some 17.  Steps that are not replayed from a graph (every
+// prompt portion) are bound by exactly that host time when they are short.
+//
+// Row-major Y = X W^T is, in the library's column-major terms, Y' [N x M] = op_T(W') op_N(X')
+// with W' = [K x N] (ld K), X' = [K x M] (ld ldx), Y' = [N x M] (ld ldy).
+//
+// One workspace of 32 MiB per device, allocated at the first call on it (kva_gemm_vendor_init
+// does that call ahead of any graph capture) and never freed; products on different streams of
+// one device would share it, the engine runs them on one stream.
+#include "common.h"
+#include <hipblaslt/hipblaslt.h>
+#include <mutex>
+#include <unordered_map>
+
+namespace {
+
+constexpr int kMaxDevices = 16;
+constexpr size_t kWorkspaceBytes = 32u << 20;
+
+struct Plan {
+    hipblasLtMatmulDesc_t desc = nullptr;
+    hipblasLtMatrixLayout_t a = nullptr, b = nullptr, c = nullptr;
+    hipblasLtMatmulAlgo_t algo;
+    bool found = false;
+};
+
+struct Key {
+    int dev, m, n, k, ldx, ldy, f32;
+    bool operator==(const Key &o) const {
+        return dev == o.dev && m == o.m && n == o.n && k == o.k && ldx == o.ldx && ldy == o.ldy && f32 == o.f32;
+    }
+};
+struct KeyHash {
+    size_t operator()(const Key &x) const {
+        size_t h = 1469598103934665603ull;
+        for (int v : {x.dev, x.m, x.n, x.k, x.ldx, x.ldy, x.f32}) h = (h ^ (size_t)(unsigned)v) * 1099511628211ull;
+        return h;
+    }
+};
+
+std::mutex g_mutex;
+hipblasLtHandle_t g_handle[kMaxDevices];
+void *g_workspace[kMaxDevices];
+std::unordered_map<Key, Plan, KeyHash> g_plans;
+
+// The handle and the workspace of a device; 0 on success.
+int device_state(int dev) {
+    if (g_handle[dev] != nullptr) return KVA_OK;
+    if (hipblasLtCreate(&g_handle[dev]) != HIPBLAS_STATUS_SUCCESS) {
+        g_handle[dev] = nullptr;
+        kva_set_error("gemm_vendor: the GEMM library could not be initialised on device %d", dev);
+        return KVA_ERR_LAUNCH;
+    }
+    if (hipMalloc(&g_workspace[dev], kWorkspaceBytes) != hipSuccess) {
+        (void)hipGetLastError();
+        hipblasLtDestroy(g_handle[dev]);
+        g_handle[dev] = nullptr;
+        kva_set_error("gemm_vendor: no memory for the library's workspace (%zu bytes)", kWorkspaceBytes);
+        return KVA_ERR_LAUNCH;
+    }
+    return KVA_OK;
+}
+
+bool make_plan(int dev, const Key &key, Plan &p) {
+    const hipblasOperation_t op_t = HIPBLAS_OP_T, op_n = HIPBLAS_OP_N;
+    const hipDataType out_type = key.f32 ? HIP_R_32F : HIP_R_16BF;
+    bool ok = hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &op_t, sizeof(op_t)) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &op_n, sizeof(op_n)) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && hipblasLtMatrixLayoutCreate(&p.a, HIP_R_16BF, key.k, key.n, key.k) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && hipblasLtMatrixLayoutCreate(&p.b, HIP_R_16BF, key.k, key.m, key.ldx) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && hipblasLtMatrixLayoutCreate(&p.c, out_type, key.n, key.m, key.ldy) == HIPBLAS_STATUS_SUCCESS;
+    hipblasLtMatmulPreference_t pref = nullptr;
+    ok = ok && hipblasLtMatmulPreferenceCreate(&pref) == HIPBLAS_STATUS_SUCCESS;
+    if (ok) {
+        const uint64_t ws = kWorkspaceBytes;
+        ok = hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof(ws)) ==
+             HIPBLAS_STATUS_SUCCESS;
+    }
+    if (ok) {
+        hipblasLtMatmulHeuristicResult_t result[1];
+        int returned = 0;
+        const hipblasStatus_t st = hipblasLtMatmulAlgoGetHeuristic(g_handle[dev], p.desc, p.a, p.b, p.c, p.c, pref, 1,
+                                                                   result, &returned);
+        if (st == HIPBLAS_STATUS_SUCCESS && returned > 0 && result[0].state == HIPBLAS_STATUS_SUCCESS &&
+            result[0].workspaceSize <= kWorkspaceBytes) {
+            p.algo = result[0].algo;
+            p.found = true;
+        }
+    }
+    if (pref) hipblasLtMatmulPreferenceDestroy(pref);
+    return ok;
+}
+
+}  // namespace
+
+// Makes the library handle and the workspace of the current device (no effect when they exist).
+extern "C" int kva_gemm_vendor_init() {
+    int dev = 0;
+    KVA_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDevices, "gemm_vendor: no current device");
+    std::lock_guard<std::mutex> lock(g_mutex);
+    return device_state(dev);
+}
+
+// Returns KVA_OK, an error, or 1 when the library offers no algorithm for the shape (nothing was
+// launched then and the caller takes another path).
+extern "C" int kva_gemm_vendor(void *Y, const void *X, const void *W, int M, int N, int K, int ldx, int ldy,
+                               int out_f32, hipStream_t stream) {
+    KVA_REQUIRE(M >= 1 && N >= 1 && K >= 1 && ldx >= K && ldy >= N, "gemm_vendor: bad sizes M=%d N=%d K=%d ldx=%d ldy=%d",
+                M, N, K, ldx, ldy);
+    int dev = 0;
+    KVA_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDevices, "gemm_vendor: no current device");
+    Plan plan;
+    hipblasLtHandle_t handle;
+    void *workspace;
+    {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        const int st = device_state(dev);
+        if (st != KVA_OK) return st;
+        const Key key{dev, M, N, K, ldx, ldy, out_f32 ? 1 : 0};
+        auto it = g_plans.find(key);
+        if (it == g_plans.end()) {
+            Plan fresh;
+            if (!make_plan(dev, key, fresh)) {
+                kva_set_error("gemm_vendor: the library refused the description of M=%d N=%d K=%d", M, N, K);
+                return KVA_ERR_LAUNCH;
+            }
+            it = g_plans.emplace(key, fresh).first;
+        }
+        plan = it->second;
+        handle = g_handle[dev];
+        workspace = g_workspace[dev];
+    }
+    if (!plan.found) return 1;
+    const float alpha = 1.f, beta = 0.f;
+    const hipblasStatus_t st = hipblasLtMatmul(handle, plan.desc, &alpha, W, plan.a, X, plan.b, &beta, Y, plan.c, Y,
+                                               plan.c, &plan.algo, workspace, kWorkspaceBytes, stream);
+    if (st != HIPBLAS_STATUS_SUCCESS) {
+        kva_set_error("gemm_vendor: the library failed on M=%d N=%d K=%d (status %d)", M, N, K, (int)st);
+        return KVA_ERR_LAUNCH;
+    }
+    return KVA_OK;
+}

@@ -33,6 +33,8 @@ HIP_FLAGS = [
     "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wno-unused-result", "-Wno-unknown-attributes",
 ]
+# the vendor GEMM library (csrc/gemm_vendor.hip); the process has torch's copy of it loaded already
+HIP_LINK_LIBS = ["-lhipblaslt"]
 HOST_FLAGS = ["-O2", "-fPIC", "-std=c++17", "-shared"]
 
 
@@ -114,7 +116,7 @@ def _hipcc() -> str:
 
 
 def hip_digest() -> str:
-    return _digest(_hip_sources() + _headers(), HIP_FLAGS)
+    return _digest(_hip_sources() + _headers(), HIP_FLAGS + HIP_LINK_LIBS)
 
 
 def host_digest() -> str:
@@ -159,7 +161,9 @@ def build_hip(force: bool = False) -> str:
             _say(f"compiled {os.path.basename(s)} ({dt:.0f} s) [{done}/{len(srcs)}]")
     lib = os.path.join(out_dir, name)
     tmp = lib + f".tmp{os.getpid()}"
-    _run([hipcc, f"--offload-arch={GPU_ARCH}", "-shared", "-fPIC", *objs, "-o", tmp], "linking " + name)
+    rocm_lib = os.path.join(os.path.dirname(os.path.dirname(os.path.realpath(hipcc))), "lib")
+    _run([hipcc, f"--offload-arch={GPU_ARCH}", "-shared", "-fPIC", *objs, "-L", rocm_lib, *HIP_LINK_LIBS, "-o", tmp],
+         "linking " + name)
     os.replace(tmp, lib)
     with open(lib + ".stamp", "w") as f:
         f.write(digest + "\n")

@@ -3,8 +3,9 @@
 ``linear_bf16(x, w, out)`` computes ``out = x @ w^T`` with fp32 accumulation.  ``out`` may be
 bf16 or fp32.  Few rows (decode steps, short portions; how few depends on the matrix, see
 ``use_skinny``) take the hand-written matrix-core kernel that streams a tiled copy of the weight
-once (``csrc/gemm_skinny.hip``).  Other shapes go to the vendor GEMM library through
-``torch.matmul``, which is where the reference's engine uses cuBLAS.
+once (``csrc/gemm_skinny.hip``).  Other shapes go to the vendor GEMM library (hipBLASLt, called
+directly with the algorithm of a shape looked up once: ``csrc/gemm_vendor.hip``), which is where
+the reference's engine uses cuBLAS.
 """
 from __future__ import annotations
 
@@ -57,6 +58,9 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, tiled=None)
         return out
     if tiled is not None and use_skinny(x.shape[0], w.shape[0], w.shape[1]):
         return K.gemm_skinny(x, tiled, out)
+    if K.gemm_vendor(x, w, out):
+        return out
+    # a shape the library's heuristic has nothing for: the framework's route to the same library
     if out.dtype == torch.bfloat16:
         torch.matmul(x, w.t(), out=out)
     else:

@@ -23,7 +23,16 @@ def dtype_code(dt: torch.dtype) -> int:
         raise KernelError(f"unsupported dtype {dt}; kernels take float32 and bfloat16") from None
 
 
+_RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_RAW_DEVICE = getattr(torch._C, "_cuda_getDevice", None) or torch.cuda.current_device
+
+
 def _stream() -> int:
+    """Handle of torch's current stream on the current device (also while a graph is captured).
+    The raw accessor costs a fraction of a microsecond; ``torch.cuda.current_stream()`` some ten,
+    once per launch."""
+    if _RAW_STREAM is not None:
+        return _RAW_STREAM(_RAW_DEVICE())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -321,6 +330,29 @@ def attention_lds(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cache
         _dev(item_meta, "item_meta", torch.int32), item_meta.shape[0], 1 if pair else 0, num_q_heads,
         num_kv_heads, head_dim, k_cache.shape[2], float(scale), int(window), _stream()), "attention_lds")
     return out
+
+
+def gemm_vendor_init() -> None:
+    """Makes the vendor GEMM library's handle and workspace on the current device; called when a
+    weight is loaded, so that no product makes them in the middle of a graph capture."""
+    check(hip_lib().kva_gemm_vendor_init(), "gemm_vendor_init")
+
+
+def gemm_vendor(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
+    """out = x @ w^T by the vendor GEMM library (bf16 operands, fp32 accumulation, bf16 or fp32
+    result).  False when the library has no algorithm for the shape: nothing was launched."""
+    m, k = x.shape
+    n = w.shape[0]
+    if w.shape[1] != k or out.shape != (m, n) or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 \
+            or out.dtype not in (torch.bfloat16, torch.float32):
+        raise KernelError(f"gemm_vendor: x {tuple(x.shape)} {x.dtype}, w {tuple(w.shape)} {w.dtype}, out "
+                          f"{tuple(out.shape)} {out.dtype} do not fit")
+    code = hip_lib().kva_gemm_vendor(_dev(out, "out"), _dev(x, "x"), _dev(w, "w"), m, n, k, k, n,
+                                     1 if out.dtype == torch.float32 else 0, _stream())
+    if code == 1:
+        return False
+    check(code, "gemm_vendor")
+    return True
 
 
 def gemm_skinny_supported(m: int, n: int, k: int) -> bool:

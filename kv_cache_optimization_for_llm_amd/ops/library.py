@@ -51,6 +51,8 @@ _HIP_SIGNATURES = {
     "kva_gemm_skinny_qkv_rope_supported": [I, I, I],
     "kva_gemm_skinny_qkv_rope": [P, I, P, P, I, I, I, I, I, I, P, I, I, F, P, P, P, P, P, P, I, P],
     "kva_gemm_nt_f32": [P, P, P, I, I, I, I, I, I, P],
+    "kva_gemm_vendor": [P, P, P, I, I, I, I, I, I, P],
+    "kva_gemm_vendor_init": [],
     "kva_sample": [P, P, I, I, I, P, P, F, P, U, P, P, I, P, P],
     "kva_mark_tokens": [P, P, P, I, I, P],
 }

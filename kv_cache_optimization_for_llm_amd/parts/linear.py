@@ -4,7 +4,7 @@ The reference calls cublasGemmEx for this (bf16 operands, fp32 accumulate,
 ``base/src/engine.cu:652-671``).  Here:
 
 * bf16 weight, bf16 activations: hand-written MFMA kernels where they exist for the shape,
-  otherwise the vendor GEMM library through ``torch.matmul`` (as the reference uses cuBLAS);
+  otherwise the vendor GEMM library (``ops.kernels.gemm_vendor``, as the reference uses cuBLAS);
 * fp32 weight: the true-fp32 kernel ``gemm_nt_f32``; bf16 activations are widened for it and
   the result is rounded back, so a tensor stored in 32-bit is used in 32-bit.
 """
@@ -28,8 +28,10 @@ class Linear:
         self.halves = halves
         # a second, tiled copy for the few-rows kernel (decode); the plain layout serves prompts
         self.tiled = None
-        if weight.is_cuda and weight.dtype == torch.bfloat16 and self.in_features % 32 == 0:
-            self.tiled = K.TiledWeight(self.weight, halves)
+        if weight.is_cuda and weight.dtype == torch.bfloat16:
+            K.gemm_vendor_init()            # the library's handle and workspace exist before any step
+            if self.in_features % 32 == 0:
+                self.tiled = K.TiledWeight(self.weight, halves)
 
     def fusable(self, x) -> bool:
         """Whether this product can finish a norm on its input and/or feed the residual stream

@@ -206,3 +206,21 @@ def test_qkv_product_refuses_head_sizes_it_cannot_pair(gpu):
     with pytest.raises(K.KernelError):
         K.gemm_skinny_qkv_rope(rnd(4, 64).to(gpu), w, torch.empty((4, 96), dtype=torch.bfloat16, device=gpu), 2, 1, 48,
                                torch.zeros(4, dtype=torch.int32, device=gpu), None, None, None, None, None, 0)
+
+
+@pytest.mark.parametrize("m", [1, 33, 64, 200, 2048])
+@pytest.mark.parametrize("n, k", [(2048, 2048), (3072, 1024), (389, 96), (100, 40), (8192, 256)])
+def test_vendor_product_bf16_and_fp32_results(m, n, k, gpu):
+    """The library product called directly (descriptors and algorithm kept per shape): against a
+    plain product, twice per shape (the second call takes the kept plan), bf16 and fp32 results.
+    A shape the library has no algorithm for returns False and launches nothing."""
+    x, w = rnd(m, k), rnd(n, k, scale=0.05, seed=4)
+    want = x.double() @ w.double().t()
+    for dt, tol in ((torch.bfloat16, 6e-3), (torch.float32, 2e-5)):
+        for _ in range(2):
+            out = torch.full((m, n), float("nan"), dtype=dt, device=gpu)
+            if not K.gemm_vendor(x.to(gpu), w.to(gpu), out):
+                assert torch.isnan(out).all()
+                continue
+            err = (out.double().cpu() - want).abs().max() / want.abs().max()
+            assert err <= tol, f"{dt}: {err:.3g}"
