@@ -12,6 +12,8 @@ memory with a memset node.
 """
 from __future__ import annotations
 
+import gc
+
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
@@ -107,8 +109,19 @@ class DecodeGraphs:
         if slot.graph is None:
             torch.cuda.synchronize()
             g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                slot.logits = self.model.forward(slot.batch, self.cache)
+            # No garbage collection while the stream captures: an unreachable engine of earlier
+            # (its pinned tables, events, graphs) freed in the middle of a capture makes calls that
+            # a capturing stream forbids, and the failure is raised inside a destructor, where it
+            # ends the process.  Collect first, then keep the collector off until the capture ends.
+            gc.collect()
+            gc_was_on = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(g):
+                    slot.logits = self.model.forward(slot.batch, self.cache)
+            finally:
+                if gc_was_on:
+                    gc.enable()
             slot.graph = g
             self.captures += 1
         slot.graph.replay()
