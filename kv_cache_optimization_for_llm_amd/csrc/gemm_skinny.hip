@@ -276,8 +276,12 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
         const int sj = wave / k_waves;                          // place among the waves of this K range
         char *xbase = reinterpret_cast<char *>(red) + (size_t)kpart * 2 * ROWS * 128;
         const int n_chunks = (kper + KC - 1) / KC;
-        // (named registers, not an array: an array here ends up in scratch memory)
-        uint4 xs0 = make_uint4(0, 0, 0, 0), xs1 = xs0, xs2 = xs0, xs3 = xs0;
+        // X of a chunk is requested two chunks ahead, like W (one chunk ahead left every turn of the
+        // loop waiting for L2): two sets of staging registers (named, not arrays: an array here
+        // ends up in scratch memory).
+        struct XRegs { uint4 v0, v1, v2, v3; };
+        XRegs xsa = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+        XRegs xsb = xsa;
         auto load_unit = [&](int i, int c) -> uint4 {
             int u = (i * J + sj) * 64 + lane;
             if (u >= UNITS) u = 0;
@@ -294,17 +298,17 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
             if (u < UNITS)
                 *reinterpret_cast<uint4 *>(xbase + (c & 1) * ROWS * 128 + q * 128 + ((c16 ^ (row & 7)) << 4)) = v;
         };
-        auto load_x = [&](int c) {
-            xs0 = load_unit(0, c);
-            if constexpr (MT > 1) xs1 = load_unit(1, c);
-            if constexpr (MT > 2) xs2 = load_unit(2, c);
-            if constexpr (MT > 3) xs3 = load_unit(3, c);
+        auto load_x = [&](XRegs &xs, int c) {
+            xs.v0 = load_unit(0, c);
+            if constexpr (MT > 1) xs.v1 = load_unit(1, c);
+            if constexpr (MT > 2) xs.v2 = load_unit(2, c);
+            if constexpr (MT > 3) xs.v3 = load_unit(3, c);
         };
-        auto store_x = [&](int c) {
-            store_unit(0, c, xs0);
-            if constexpr (MT > 1) store_unit(1, c, xs1);
-            if constexpr (MT > 2) store_unit(2, c, xs2);
-            if constexpr (MT > 3) store_unit(3, c, xs3);
+        auto store_x = [&](const XRegs &xs, int c) {
+            store_unit(0, c, xs.v0);
+            if constexpr (MT > 1) store_unit(1, c, xs.v1);
+            if constexpr (MT > 2) store_unit(2, c, xs.v2);
+            if constexpr (MT > 3) store_unit(3, c, xs.v3);
         };
         // W of a chunk goes straight to registers, NB chunks ahead (four were measured no faster)
         constexpr int NB = 2;
@@ -334,32 +338,40 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
                 }
             }
         };
-        load_x(0);
-#pragma unroll
-        for (int b = 0; b < NB; ++b)
-            if (b < n_chunks) load_w(wbuf[b], b);
-        // NB chunks per turn while every load of the turn exists: no branch in the body, so the
+        static_assert(NB == 2, "the turns below are written out for two buffers");
+        load_x(xsa, 0);
+        if (n_chunks > 1) load_x(xsb, 1);
+        load_w(wbuf[0], 0);
+        if (n_chunks > 1) load_w(wbuf[1], 1);
+        // Two chunks per turn while every load of the turn exists: no branch in the body, so the
         // waits count exactly and the loads issued last stay in flight across them.
         int c = 0;
-        for (; c + 2 * NB - 1 < n_chunks; c += NB) {
-#pragma unroll
-            for (int b = 0; b < NB; ++b) {
-                store_x(c + b);
-                __syncthreads();
-                load_x(c + b + 1);
-                compute(wbuf[b], c + b);
-                load_w(wbuf[b], c + b + NB);
-            }
+        for (; c + 3 < n_chunks; c += 2) {
+            store_x(xsa, c);
+            __syncthreads();
+            load_x(xsa, c + 2);
+            compute(wbuf[0], c);
+            load_w(wbuf[0], c + 2);
+            store_x(xsb, c + 1);
+            __syncthreads();
+            load_x(xsb, c + 3);
+            compute(wbuf[1], c + 1);
+            load_w(wbuf[1], c + 3);
         }
-        // the last chunks (fewer than 2 NB): X of chunk c is loaded, W of c + b in buffer b
-#pragma unroll
-        for (int b = 0; b < 2 * NB - 1; ++b) {
-            if (c + b < n_chunks) {
-                store_x(c + b);
+        // the last one to three chunks: chunk c in (xsa, wbuf[0]), c + 1 in (xsb, wbuf[1])
+        store_x(xsa, c);
+        __syncthreads();
+        if (c + 2 < n_chunks) load_x(xsa, c + 2);
+        compute(wbuf[0], c);
+        if (c + 2 < n_chunks) load_w(wbuf[0], c + 2);
+        if (c + 1 < n_chunks) {
+            store_x(xsb, c + 1);
+            __syncthreads();
+            compute(wbuf[1], c + 1);
+            if (c + 2 < n_chunks) {
+                store_x(xsa, c + 2);
                 __syncthreads();
-                if (c + b + 1 < n_chunks) load_x(c + b + 1);
-                compute(wbuf[b % NB], c + b);
-                if (c + b + NB < n_chunks) load_w(wbuf[b % NB], c + b + NB);
+                compute(wbuf[0], c + 2);
             }
         }
         __syncthreads();                                        // the sums below reuse the buffer
