@@ -67,6 +67,27 @@ def test_greedy_generation_through_the_entry_point(name, dtype, model_dirs, gpu)
     assert llm.engine.cache.free_seats == 4
 
 
+@pytest.mark.parametrize("name, batch", [("A", 20), ("C", 40), ("D", 64)])
+def test_many_requests_decoding_together(name, batch, model_dirs, gpu):
+    """17 to 64 decoded tokens per step: the shapes of the few-rows products whose waves share X
+    through LDS, of the vendor GEMM at few rows and of decode graphs for large batches.  Every
+    pick must be the plain model's (within bf16 rounding), for every request."""
+    cfg, W = plain.load_model_dir(model_dirs[name])
+    rng = np.random.default_rng(7)
+    lengths = [int(n) for n in rng.integers(1, 12, batch)]
+    prompts = prompts_for(name, lengths, seed=5)
+    llm = LLM(model_dirs[name], EngineOptions(dtype="bfloat16", page_size=16, max_seqs=batch, max_seq_len=64),
+              ServeOptions(max_batch_tokens=1024))
+    got, reasons = llm.generate(prompts, max_new_tokens=10, ignore_eos=True, return_reasons=True)
+    assert reasons == ["length"] * batch
+    for p, g in zip(prompts, got):
+        assert len(g) == 10
+        check_choices(cfg, W, p, g, "bfloat16")
+    assert llm.engine.graphs.replays > 0
+    llm.engine.cache.check()
+    assert llm.engine.cache.free_seats == batch
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_temperature_sampling_and_penalty_follow_the_plain_sampler(dtype, model_dirs, gpu):
     cfg, W = plain.load_model_dir(model_dirs["B"])
