@@ -427,7 +427,27 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
             }
             __syncthreads();
             if (kpart == 0) {
-                for (int p = 1; p < k_waves; ++p) {
+                // three slices are read at a time and then added in slice order (one read per
+                // turn leaves this wave waiting for LDS fifteen times in a row)
+                constexpr int RB = NTW * MT <= 2 ? 3 : 1;       // (where registers allow)
+                int p = 1;
+                for (; RB > 1 && p + RB - 1 < k_waves; p += RB) {
+                    float4 v[RB][NTW];
+#pragma unroll
+                    for (int j = 0; j < RB; ++j)
+#pragma unroll
+                        for (int t = 0; t < NTW; ++t)
+                            v[j][t] = *reinterpret_cast<const float4 *>(red + (size_t)(wave + p + j) * (NTW * 64 * 4) +
+                                                                        (t * 64 + lane) * 4);
+#pragma unroll
+                    for (int j = 0; j < RB; ++j)
+#pragma unroll
+                        for (int t = 0; t < NTW; ++t) {
+                            acc[t][mt][0] += v[j][t].x; acc[t][mt][1] += v[j][t].y;
+                            acc[t][mt][2] += v[j][t].z; acc[t][mt][3] += v[j][t].w;
+                        }
+                }
+                for (; p < k_waves; ++p) {
                     const float *other = red + (size_t)(wave + p) * (NTW * 64 * 4);
 #pragma unroll
                     for (int t = 0; t < NTW; ++t) {
