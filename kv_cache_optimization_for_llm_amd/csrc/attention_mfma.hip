@@ -112,13 +112,11 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
         const bf16_t *qrow = q + (size_t)(q_start + tq[rt]) * q_row_stride + (size_t)head[rt] * D;
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
-            if (KSTEP == 32) {
-                qf8[rt][ks].u4 = row_valid[rt] ? *reinterpret_cast<const uint4 *>(qrow + ks * 32 + g * 8)
-                                               : make_uint4(0, 0, 0, 0);
-            } else {
-                qf4[rt][ks].u2 = row_valid[rt] ? *reinterpret_cast<const uint2 *>(qrow + ks * 16 + g * 4)
-                                               : make_uint2(0, 0);
-            }
+            // rows past the item's last read the entry's first row (tq and head are clamped): no
+            // select on the loaded value, which would wait for it here, long before its first
+            // use; every score of such a row is masked below and nothing of it is stored
+            if (KSTEP == 32) qf8[rt][ks].u4 = *reinterpret_cast<const uint4 *>(qrow + ks * 32 + g * 8);
+            else qf4[rt][ks].u2 = *reinterpret_cast<const uint2 *>(qrow + ks * 16 + g * 4);
         }
     }
 
@@ -163,6 +161,7 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
                 tile0 = tile0 < lo_tile ? lo_tile : (tile0 > hi_tile ? hi_tile : tile0);
                 pg[t] = bt[__builtin_amdgcn_readfirstlane(tile0 >> 4)];
             }
+            __builtin_amdgcn_sched_barrier(0);                  // both lookups are out before either is used
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
                 const size_t page_bytes = ((size_t)pg[t] * num_kv_heads + kvh) * (size_t)(16 * D * 2);
