@@ -350,3 +350,43 @@ def test_another_position_encoding_and_a_routed_feed_forward(dtype, tol, tmp_pat
         i += n
     assert err(torch.cat(rows)[sure], ref[sure]) <= tol
     eng.cache.check()
+
+
+def test_garbage_of_an_earlier_engine_is_not_collected_inside_a_graph_capture(tmp_path, gpu):
+    """An engine that has become unreachable (pinned block tables, events, captured graphs) is
+    freed by Python's collector at some later allocation - also one made while the next engine
+    captures a decode graph, where freeing such things is forbidden and fails inside a destructor.
+    The capture collects first and keeps the collector off: with a collector set to run at every
+    few allocations, a second engine captures and replays its graphs next to the garbage of a first."""
+    import gc
+    from conftest import TINY
+    cfg = TINY["A"][0]
+    write_random_model(str(tmp_path / "m"), cfg, 2)
+    prompt = [3, 1, 4, 1, 5, 9, 2, 6]
+
+    def decode_some(engine, name):
+        logits = engine.step([StepEntry(name, prompt, [len(prompt) - 1])])
+        tok = int(logits[0].argmax())
+        out = [tok]
+        for _ in range(6):                                    # the same shape again and again: warm-up, capture, replays
+            logits = engine.step([StepEntry(name, [tok], [0])])
+            tok = int(logits[0].argmax())
+            out.append(tok)
+        engine.release(name)
+        return out
+
+    first = Engine(str(tmp_path / "m"), EngineOptions(dtype="bfloat16", max_seqs=2, max_seq_len=64))
+    want = decode_some(first, "a")
+    assert first.graphs.captures >= 1
+    ring = [first]
+    ring.append(ring)                                         # a cycle: only the collector can free it
+    del first, ring
+    old = gc.get_threshold()
+    gc.set_threshold(5, 2, 2)
+    try:
+        second = Engine(str(tmp_path / "m"), EngineOptions(dtype="bfloat16", max_seqs=2, max_seq_len=64))
+        got = decode_some(second, "b")
+        assert second.graphs.captures >= 1 and second.graphs.replays >= 1
+    finally:
+        gc.set_threshold(*old)
+    assert got == want
