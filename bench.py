@@ -140,7 +140,7 @@ def main():
     # prefill of 2,048 tokens: one request, one step, logits at the last place
     prompt = [int(t) for t in torch.randint(0, engine.vocab_size, (PREFILL_TOKENS,), generator=gen)]
     pre_ms = []
-    for i in range(3):
+    for i in range(6):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         engine.step([StepEntry(f"p{i}", prompt, [PREFILL_TOKENS - 1])])
