@@ -77,7 +77,7 @@ def attention(args) -> None:
         splits = args.splits
         per = ((ctx + splits - 1) // splits + 31) // 32 * 32
     if args.kernel == "lds":
-        calls = [lambda c=c: K.attention_lds(qkv, nq * d, out, c[0], c[1], table, meta_d, nq, nkv, d, scale, 0, False)
+        calls = [lambda c=c: K.attention_lds(qkv, nq * d, out, c[0], c[1], table, meta_d, nq, nkv, d, scale, 0, args.pair)
                  for c in caches]
     else:
         tiles = 2 if args.tokens else 1
@@ -140,6 +140,7 @@ def main(argv=None) -> int:
     a.add_argument("--head-dim", type=int, default=64)
     a.add_argument("--reps", type=int, default=20)
     a.add_argument("--no-pair", action="store_true", help="wave kernel: never give a wave two items")
+    a.add_argument("--pair", action="store_true", help="workgroup kernel: a workgroup takes item i and item n-1-i")
     g = sub.add_parser("gemm")
     g.add_argument("--shape", choices=sorted(GEMM_SHAPES), default="gate_up")
     g.add_argument("--rows", type=int, default=8)
