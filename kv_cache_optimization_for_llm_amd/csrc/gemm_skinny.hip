@@ -8,7 +8,7 @@
 //   A = 16 rows of W (an "n-tile") x 32 of K      lane (r, g) loads W[n0 + r][k + 8g .. 8g+7]
 //   B = X^T, 32 of K x 16 tokens                   lane (r, g) loads X[m0 + r][k + 8g .. 8g+7]
 //   D[n0 + 4g + i][m0 + r]                         -> 4 consecutive outputs of token m0 + r
-// W comes pre-tiled ([n-tile][K/32][16][32], made once at load time): a wave's 1 KiB per step is
+// W comes pre-tiled ([n-tile][K/32][g 4][r 16][8], made once at load time): a wave's 1 KiB per step is
 // contiguous.  Both operands are read from memory directly in operand layout (16 bytes per lane).  A wave
 // keeps one accumulator per 16-token tile (MT = ceil(M / 16) <= 4) and per n-tile it owns
 // (NTW = 1, 2 or 4: wide matrices give a wave several n-tiles so that a loaded X fragment is
@@ -125,9 +125,10 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
     const int kper = K / k_waves;
     const int kbeg = kpart * kper, kend = kbeg + kper;
 
-    // W is stored tiled: [n-tile][K / 32][16 rows][32 of K], so the 1 KiB a wave needs per step is
-    // contiguous and a wave walks its n-tile as one sequential stream.  Lane (r, g) takes bytes
-    // (4r + g) * 16 of the chunk.  For EPI_SWIGLU the up tiles follow the gate tiles.
+    // W is stored tiled: [n-tile][K / 32][g][r][8 of K], so the 1 KiB a wave needs per step is
+    // contiguous, in the order of its lanes (lane r + 16 g takes bytes 16 (r + 16 g) ..), and a
+    // wave walks its n-tile as one sequential stream.  For EPI_SWIGLU the up tiles follow the
+    // gate tiles.
     const bf16_t *wp[NTW];
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
@@ -138,7 +139,7 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
         }
         const int last = (EPI == EPI_SWIGLU ? 2 * n_tiles : n_tiles) - 1;
         if (tile > last) tile = last;
-        wp[t] = a.W + (size_t)tile * (size_t)(K / 32) * 512 + (4 * wrow + g) * 8;
+        wp[t] = a.W + (size_t)tile * (size_t)(K / 32) * 512 + (16 * g + wrow) * 8;
     }
     const bf16_t *xr[MT];
 #pragma unroll

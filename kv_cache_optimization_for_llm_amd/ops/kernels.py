@@ -360,9 +360,10 @@ def gemm_skinny_supported(m: int, n: int, k: int) -> bool:
 
 
 class TiledWeight:
-    """A bf16 ``[N, K]`` weight re-laid for the few-rows product: ``[n-tile][K/32][16][32]``, rows
-    padded with zeros to a multiple of 16, so that the 1 KiB a wavefront needs per step is
-    contiguous.  With ``halves=2`` (a joined ``[gate; up]`` matrix) each half is tiled on its own
+    """A bf16 ``[N, K]`` weight re-laid for the few-rows product: ``[n-tile][K/32][4][16][8]``
+    (tile of 16 rows, step of 32 of K, quarter of the step, row, 8 of K), rows padded with zeros
+    to a multiple of 16, so that the 1 KiB a wavefront needs per step is contiguous and in the
+    order of its lanes.  With ``halves=2`` (a joined ``[gate; up]`` matrix) each half is tiled on its own
     and the gate tiles come first."""
 
     def __init__(self, weight: torch.Tensor, halves: int = 1):
@@ -376,7 +377,10 @@ class TiledWeight:
             pad = (-rows) % 16
             if pad:
                 h = torch.cat([h, torch.zeros((pad, k), dtype=h.dtype, device=h.device)])
-            parts.append(h.view((rows + pad) // 16, 16, k // 32, 32).permute(0, 2, 1, 3).contiguous())
+            # [tile][row 16][step][g 4][8] -> [tile][step][g][row][8]: the 16 bytes of lane r + 16 g
+            # of a wavefront lie at byte 16 (r + 16 g) of the step's 1 KiB, so neighbouring lanes
+            # read neighbouring memory (four lanes per 64-byte access instead of one)
+            parts.append(h.view((rows + pad) // 16, 16, k // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous())
         self.data = torch.cat(parts).contiguous()
 
 

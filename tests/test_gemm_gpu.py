@@ -69,7 +69,8 @@ def test_skinny_product_refuses_what_it_cannot_do(gpu):
     with pytest.raises(K.KernelError):
         K.gemm_skinny(x, w, torch.empty((4, 16), dtype=torch.bfloat16, device=gpu))
     tw = K.TiledWeight(rnd(50, 64).to(gpu))                # 50 rows are padded to 64
-    assert tw.data.shape == (4, 2, 16, 32) and tw.data[3, :, 2:].abs().max() == 0
+    # [tile][step of 32][quarter of the step][row][8]: rows 2..15 of the last tile are the padding
+    assert tw.data.shape == (4, 2, 4, 16, 8) and tw.data[3, :, :, 2:].abs().max() == 0
 
 
 def rms(h, w, eps):
