@@ -84,6 +84,11 @@ struct SkinnyArgs {
     int nq, nkv, head_dim, page_size;
     // half tiles: a tile group takes 8 of its tiles' 16 rows (see choose_half_tiles)
     int half;
+    // At most 16 rows: X (x_tiled) or the bf16 result (y_tiled) laid out [columns / 8][16 rows][8],
+    // the order in which the lanes of the consuming product read it (four neighbouring lanes, the
+    // same 8 columns of four neighbouring rows, then take 64 contiguous bytes; row-major they take
+    // four pieces 2 K bytes apart).  A private layout between two products of one part.
+    int x_tiled, y_tiled;
 };
 
 // XL: the waves of a workgroup that work on the same K range (one per tile group) share X through
@@ -145,7 +150,7 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = mt * 16 + r;
-        xr[mt] = a.X + (size_t)(m < a.M ? m : 0) * a.ldx + 8 * g;
+        xr[mt] = a.x_tiled ? a.X + (16 * g + r) * 8 : a.X + (size_t)(m < a.M ? m : 0) * a.ldx + 8 * g;
     }
 
     gf32x4 acc[NTW][MT];
@@ -377,6 +382,7 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
         }
         __syncthreads();                                        // the sums below reuse the buffer
     } else if (group_ok) {
+        const size_t xstep = a.x_tiled ? 16 : 1;               // a step of 32 columns is 4 chunks of 16 rows x 8
 #pragma unroll 8
         for (int k = kbeg; k < kend; k += 32) {
             GFrag8 w[NTW];
@@ -385,7 +391,7 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 GFrag8 x;
-                x.u4 = *reinterpret_cast<const uint4 *>(xr[mt] + k);
+                x.u4 = *reinterpret_cast<const uint4 *>(xr[mt] + (size_t)k * xstep);
 #pragma unroll
                 for (int t = 0; t < NTW; ++t)
                     acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[t].v, x.v, acc[t][mt], 0, 0, 0);
@@ -635,7 +641,8 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
                 }
             } else {
                 bf16_t *dst = reinterpret_cast<bf16_t *>(a.Y) + (size_t)m * a.ldy + n;
-                if (n + 3 < rows && (a.ldy % 4 == 0)) {
+                if (a.y_tiled) dst = reinterpret_cast<bf16_t *>(a.Y) + ((size_t)(n >> 3) * 16 + m) * 8 + (n & 7);
+                if (n + 3 < rows && (a.y_tiled || a.ldy % 4 == 0)) {
                     uint2 w;
                     w.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
                     w.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
@@ -722,7 +729,8 @@ static void launch_mt(const SkinnyArgs &a, dim3 grid, dim3 block, size_t lds, hi
 extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int N, int K, int ldx,
                                int ldy, int mode, const float *sumsq, int sumsq_parts, int norm_width,
                                float eps, void *hidden, const void *next_w, int next_w_f32,
-                               void *scaled_out, float *sumsq_out, hipStream_t stream) {
+                               void *scaled_out, float *sumsq_out, int x_tiled, int y_tiled,
+                               hipStream_t stream) {
     KVA_REQUIRE(kva_gemm_skinny_supported(M, N, K), "gemm_skinny: M=%d N=%d K=%d not supported "
                 "(1 <= M <= 64, K a multiple of 32)", M, N, K);
     KVA_REQUIRE(mode >= 0 && mode <= 3, "gemm_skinny: unknown mode %d", mode);
@@ -740,6 +748,10 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
     a.sumsq = sumsq; a.sumsq_parts = sumsq_parts; a.norm_width = norm_width; a.eps = eps;
     a.hidden = (bf16_t *)hidden; a.next_w = next_w; a.next_w_f32 = next_w_f32;
     a.scaled_out = (bf16_t *)scaled_out; a.sumsq_out = sumsq_out;
+    KVA_REQUIRE(!(x_tiled || y_tiled) || M <= 16, "gemm_skinny: the tiled layouts of X and Y are for at most 16 rows");
+    KVA_REQUIRE(!y_tiled || (mode == 2 && (N / 2) % 8 == 0), "gemm_skinny: a tiled result is for the gated product with a multiple of 8 columns");
+    KVA_REQUIRE(!x_tiled || K % 8 == 0, "gemm_skinny: tiled X");
+    a.x_tiled = x_tiled ? 1 : 0; a.y_tiled = y_tiled ? 1 : 0;
     const int rows = mode == 2 ? a.inter : N;
     KVA_REQUIRE(mode == 3 || ldy >= rows, "gemm_skinny: Y row stride %d is smaller than its %d columns", ldy, rows);
     const int n_tiles = (rows + 15) / 16;

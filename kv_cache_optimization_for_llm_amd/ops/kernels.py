@@ -384,10 +384,42 @@ class TiledWeight:
         self.data = torch.cat(parts).contiguous()
 
 
+class TiledRows:
+    """At most 16 rows of ``width`` bf16 columns laid out ``[width / 8, 16, 8]``: element (m, c)
+    at ``[c // 8, m, c % 8]``, rows past ``rows`` unwritten.  It is the order in which the lanes of
+    a few-rows product read X (four neighbouring lanes take the same 8 columns of four
+    neighbouring rows: 64 contiguous bytes instead of four pieces a row apart), so a product that
+    feeds another can leave its result like this.  ``to_rows()`` gives the plain ``[rows, width]``."""
+
+    MAX_ROWS = 16
+
+    def __init__(self, rows: int, width: int, device):
+        if not (1 <= rows <= self.MAX_ROWS) or width % 8:
+            raise KernelError(f"TiledRows: 1..16 rows and a multiple of 8 columns, not {rows} x {width}")
+        self.rows, self.width = rows, width
+        self.data = torch.empty((width // 8, 16, 8), dtype=torch.bfloat16, device=device)
+
+    @property
+    def shape(self):
+        return (self.rows, self.width)
+
+    @property
+    def dtype(self):
+        return self.data.dtype
+
+    @property
+    def device(self):
+        return self.data.device
+
+    def to_rows(self) -> torch.Tensor:
+        return self.data.permute(1, 0, 2).reshape(16, self.width)[:self.rows].contiguous()
+
+
 def gemm_skinny(x: torch.Tensor, w: TiledWeight, out: Optional[torch.Tensor], swiglu: bool = False, *,
                 sumsq: Optional[torch.Tensor] = None, norm_width: int = 0, eps: float = 0.0,
                 hidden: Optional[torch.Tensor] = None, next_weight: Optional[torch.Tensor] = None,
-                scaled_out: Optional[torch.Tensor] = None, sumsq_out: Optional[torch.Tensor] = None):
+                scaled_out: Optional[torch.Tensor] = None, sumsq_out: Optional[torch.Tensor] = None,
+                x_tiled: bool = False, out_tiled: bool = False):
     """out = x @ W^T for at most 64 rows of x (bf16 operands, fp32 accumulation); ``w`` is the
     :class:`TiledWeight` of W.
 
@@ -397,10 +429,19 @@ def gemm_skinny(x: torch.Tensor, w: TiledWeight, out: Optional[torch.Tensor], sw
       (``round(h * w_norm)``) and the product is scaled per token by
       ``rsqrt(sum(sumsq[m]) / norm_width + eps)``.
     * ``hidden`` (instead of ``out``): ``hidden += x @ W^T`` in place (fp32 add, rounded), plus
-      ``scaled_out = round(hidden * next_weight)`` and ``sumsq_out[M, ceil(N / 16)]``."""
+      ``scaled_out = round(hidden * next_weight)`` and ``sumsq_out[M, ceil(N / 16)]``.
+    * ``out_tiled`` (gated product, at most 16 rows): ``out`` is ``[N / 2 / 8, 16, 8]``, element
+      (m, c) at ``[c // 8, m, c % 8]`` - the order in which the lanes of a following few-rows
+      product read it (a :class:`TiledRows`); such a result is given to that product as ``x``
+      with ``x_tiled``."""
     if not isinstance(w, TiledWeight):
         raise KernelError("gemm_skinny: the weight must be a TiledWeight")
-    m, k = x.shape
+    if x_tiled:
+        if not isinstance(x, TiledRows):
+            raise KernelError("gemm_skinny: x_tiled needs a TiledRows")
+        m, k, x = x.rows, x.width, x.data
+    else:
+        m, k = x.shape
     n = w.n
     if x.dtype != torch.bfloat16 or k != w.k or (swiglu != (w.halves == 2)):
         raise KernelError(f"gemm_skinny: bf16 x {tuple(x.shape)} does not fit weight [{w.n}, {w.k}] "
@@ -423,17 +464,24 @@ def gemm_skinny(x: torch.Tensor, w: TiledWeight, out: Optional[torch.Tensor], sw
             None, _dev(x, "x"), _dev(w.data, "w"), m, n, k, k, n, 3, _opt(sumsq, "sumsq", torch.float32), parts,
             int(norm_width), float(eps), _dev(hidden, "hidden"), _opt(next_weight, "next_weight"),
             1 if next_weight is not None and next_weight.dtype == torch.float32 else 0,
-            _dev(scaled_out, "scaled_out"), _dev(sumsq_out, "sumsq_out", torch.float32), _stream()),
+            _dev(scaled_out, "scaled_out"), _dev(sumsq_out, "sumsq_out", torch.float32),
+            1 if x_tiled else 0, 0, _stream()),
             "gemm_skinny")
         return hidden
     cols = n // 2 if swiglu else n
-    if out.shape != (m, cols) or (swiglu and out.dtype != torch.bfloat16) \
+    out_t = out
+    if out_tiled:
+        if not (isinstance(out, TiledRows) and swiglu and out.rows == m and out.width == cols):
+            raise KernelError("gemm_skinny: out_tiled needs the gated product and a TiledRows of its size")
+        out_t = out.data
+    elif out.shape != (m, cols) or (swiglu and out.dtype != torch.bfloat16) \
             or out.dtype not in (torch.bfloat16, torch.float32):
         raise KernelError(f"gemm_skinny: out {tuple(out.shape)} {out.dtype} does not fit")
-    mode = 2 if swiglu else (1 if out.dtype == torch.float32 else 0)
-    check(lib.kva_gemm_skinny(_dev(out, "out"), _dev(x, "x"), _dev(w.data, "w"), m, n, k, k, cols, mode,
+    mode = 2 if swiglu else (1 if out_t.dtype == torch.float32 else 0)
+    check(lib.kva_gemm_skinny(_dev(out_t, "out"), _dev(x, "x"), _dev(w.data, "w"), m, n, k, k, cols, mode,
                               _opt(sumsq, "sumsq", torch.float32), parts, int(norm_width), float(eps),
-                              None, None, 0, None, None, _stream()), "gemm_skinny")
+                              None, None, 0, None, None, 1 if x_tiled else 0, 1 if out_tiled else 0, _stream()),
+          "gemm_skinny")
     return out
 
 

@@ -40,6 +40,15 @@ class Linear:
         return (self.tiled is not None and x.dtype == torch.bfloat16
                 and use_skinny(x.shape[0], self.out_features, self.in_features, self.halves == 2))
 
+    def will_fuse_residual(self, rows: int, dtype, tail: Optional[BranchTail]) -> bool:
+        """Whether :meth:`into_residual` will fuse for ``rows`` rows of ``dtype`` (then its input may
+        come as ``ops.kernels.TiledRows``)."""
+        from ..ops.gemm_bf16 import use_skinny
+        prep = tail.norm.prepared_by_product() if tail is not None and tail.norm is not None else None
+        return (prep is not None and prep[1] == self.out_features and self.tiled is not None
+                and dtype == torch.bfloat16 and tail.hidden.dtype == torch.bfloat16
+                and use_skinny(rows, self.out_features, self.in_features, self.halves == 2))
+
     def into_residual(self, x, tail: BranchTail) -> Optional[NormedRows]:
         """hidden += x @ W^T in place and the sum prepared for ``tail.norm``; ``None`` when this
         cannot be fused (the caller then takes the plain product)."""
@@ -58,7 +67,7 @@ class Linear:
                           hidden=tail.hidden, next_weight=next_w, scaled_out=scaled, sumsq_out=sumsq)
         else:
             K.gemm_skinny(x, self.tiled, None, hidden=tail.hidden, next_weight=next_w,
-                          scaled_out=scaled, sumsq_out=sumsq)
+                          scaled_out=scaled, sumsq_out=sumsq, x_tiled=isinstance(x, K.TiledRows))
         return NormedRows(scaled, sumsq, width, eps, tail.norm)
 
     def __call__(self, x, out: Optional[torch.Tensor] = None,

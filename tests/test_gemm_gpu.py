@@ -225,3 +225,32 @@ def test_vendor_product_bf16_and_fp32_results(m, n, k, gpu):
                 continue
             err = (out.double().cpu() - want).abs().max() / want.abs().max()
             assert err <= tol, f"{dt}: {err:.3g}"
+
+
+@pytest.mark.parametrize("m", [1, 7, 16])
+@pytest.mark.parametrize("inter, hidden", [(8192, 2048), (256, 96), (96, 64)])
+def test_activations_pass_between_two_products_in_lane_order(m, inter, hidden, gpu):
+    """The gated product can leave its result as TiledRows ([columns / 8][16 rows][8]) and the
+    residual product can read its X in that layout: bit for bit what the row-major route gives."""
+    x = rnd(m, hidden).to(gpu)
+    w_gu = K.TiledWeight(rnd(2 * inter, hidden, scale=0.2, seed=5).to(gpu), halves=2)
+    w_down = K.TiledWeight(rnd(hidden, inter, scale=0.05, seed=6).to(gpu))
+    act_rows = torch.empty((m, inter), dtype=torch.bfloat16, device=gpu)
+    K.gemm_skinny(x, w_gu, act_rows, swiglu=True)
+    act_tiled = K.TiledRows(m, inter, gpu)
+    act_tiled.data.fill_(float("nan"))                       # rows past m stay unwritten and must not matter
+    K.gemm_skinny(x, w_gu, act_tiled, swiglu=True, out_tiled=True)
+    assert torch.equal(act_tiled.to_rows(), act_rows)
+    parts = K.gemm_skinny_sumsq_parts(hidden)
+    results = []
+    for a in (act_rows, act_tiled):
+        h = rnd(m, hidden, seed=7).to(gpu)
+        scaled = torch.empty((m, hidden), dtype=torch.bfloat16, device=gpu)
+        sumsq = torch.empty((m, parts), device=gpu)
+        K.gemm_skinny(a, w_down, None, hidden=h, next_weight=None, scaled_out=scaled, sumsq_out=sumsq,
+                      x_tiled=a is act_tiled)
+        results.append((h, scaled, sumsq))
+    for u, v in zip(*results):
+        assert torch.equal(u, v)
+    with pytest.raises(K.KernelError):
+        K.TiledRows(17, 64, gpu)
