@@ -49,12 +49,32 @@ TINY_D = dict(
                       original_max_position_embeddings=256),
     tie_word_embeddings=True, hidden_act="silu", torch_dtype="bfloat16",
 )
-TINY = {"A": (TINY_A, 11), "B": (TINY_B, 23), "C": (TINY_C, 37), "D": (TINY_D, 41)}
+# Two layers at the head sizes and with widths of the order of the served models (64 as in the 1B
+# shape, 128 as in the 3B and 8B shapes): here the matrix-core attention kernels, the few-rows
+# products with their fused epilogues and the vendor products are the ones that run.
+MID_E = dict(
+    architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=2003, hidden_size=512,
+    intermediate_size=1376, num_hidden_layers=2, num_attention_heads=8, num_key_value_heads=2,
+    head_dim=64, rms_norm_eps=1e-5, rope_theta=500000.0, max_position_embeddings=2048,
+    rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=512),
+    tie_word_embeddings=True, hidden_act="silu", torch_dtype="bfloat16",
+)
+MID_F = dict(
+    architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=1501, hidden_size=640,
+    intermediate_size=1056, num_hidden_layers=2, num_attention_heads=6, num_key_value_heads=2,
+    head_dim=128, rms_norm_eps=1e-6, rope_theta=500000.0, max_position_embeddings=2048,
+    rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=1024),
+    tie_word_embeddings=False, hidden_act="silu", torch_dtype="bfloat16",
+)
+TINY = {"A": (TINY_A, 11), "B": (TINY_B, 23), "C": (TINY_C, 37), "D": (TINY_D, 41),
+        "E": (MID_E, 53), "F": (MID_F, 59)}
 
 
 @pytest.fixture(scope="session")
 def model_dirs(tmp_path_factory):
-    """Model folders of the two tiny configurations, written by the random-weights mode."""
+    """Model folders of the test configurations, written by the random-weights mode."""
     from kv_cache_optimization_for_llm_amd.weights.random_init import write_random_model
     base = tmp_path_factory.mktemp("models")
     out = {}

@@ -48,11 +48,11 @@ def compare(rows, ref, requests, dtype, what):
 
 
 LENGTHS = {"A": [5, 17, 33, 70, 131], "B": [1, 9, 40, 70, 97], "C": [3, 66, 130, 45, 200],
-           "D": [2, 35, 90, 64, 150]}
+           "D": [2, 35, 90, 64, 150], "E": [4, 130, 300, 65, 517], "F": [2, 257, 48, 330, 129]}
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F"])
 def test_every_cut_matches_plain(name, dtype, model_dirs, plain_rows, tmp_path, gpu):
     vocab = TINY[name][0]["vocab_size"]
     requests = make_requests(vocab, LENGTHS[name], seed=5)
