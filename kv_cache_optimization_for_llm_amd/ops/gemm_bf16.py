@@ -41,9 +41,6 @@ def use_skinny(m: int, n: int, k: int, gated: bool = False) -> bool:
         return True
     if m <= SKINNY_MID_ROWS and (n * k <= SKINNY_MID_ELEMENTS or n >= 4 * k):
         return True
-    import os
-    if os.environ.get("KVA_POLICY") == "old":
-        return m <= 48 and n >= SKINNY_WIDE_N
     return m <= SKINNY_WIDE_ROWS and (n >= SKINNY_WIDE_N or (gated and n >= 4 * k))
 
 
