@@ -65,6 +65,8 @@ def main():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=CONTEXT)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the 16 of the configuration")
+    ap.add_argument("--no-gemm-tuning", action="store_true",
+                    help="leave the vendor GEMM library its own choice of algorithm (no timing at start-up)")
     ap.add_argument("--skip-points", action="store_true", help="only the default decode run and the prefill")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -85,8 +87,12 @@ def main():
     cfg["max_position_embeddings"] = max(cfg["max_position_embeddings"], ctx)      # a longer --context
     # room for max_batch requests at the context, one more page each for the tokens decoded
     pool = max_batch * (ctx + 2 * PAGE)
+    # the vendor library's algorithms are timed once, at start-up, for the row counts whose
+    # products go to it here: the prefill's 2,048 tokens and decode batches above 32
+    tune_rows = [] if args.no_gemm_tuning else [PREFILL_TOKENS] + [b for b in {args.batch, max_batch} if b > 32]
     engine = Engine(None, EngineOptions(dtype="bfloat16", page_size=PAGE, cache_tokens=pool,
-                                        max_seqs=max_batch, max_seq_len=cfg["max_position_embeddings"]),
+                                        max_seqs=max_batch, max_seq_len=cfg["max_position_embeddings"],
+                                        gemm_tune_rows=tune_rows),
                     config_dict=cfg, random_seed=0)
     dev = engine.device
     gen = torch.Generator().manual_seed(0)

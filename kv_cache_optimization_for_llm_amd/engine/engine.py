@@ -44,6 +44,10 @@ class EngineOptions:
     max_seqs: int = 8                   # seats (reference: MAX_SEQUENCES)
     max_seq_len: Optional[int] = None   # longest request (default: max_position_embeddings)
     use_graphs: bool = True             # replay decode-only steps as HIP graphs (bfloat16 engine)
+    # Row counts (tokens per step) for which the vendor GEMM library's algorithms are timed at
+    # start-up and the fastest kept, e.g. the prompt portion size and large decode batches
+    # (bfloat16 engine; a few seconds per row count and matrix shape).  Empty: the library's own choice.
+    gemm_tune_rows: Sequence[int] = ()
     device: str = "cuda:0"
 
 
@@ -86,6 +90,11 @@ class Engine:
                                                self.device)
         self.model.load(tensors)
         del tensors
+        self.gemm_tuning: List[dict] = []
+        if options.gemm_tune_rows and self.dtype == torch.bfloat16:
+            import sys
+            self.gemm_tuning = self.model.tune_products(
+                options.gemm_tune_rows, say=lambda line: print(f"[kva tune] {line}", file=sys.stderr, flush=True))
         self.vocab_size = self.spec.vocab_size
         max_seq_len = options.max_seq_len or self.spec.max_positions
         max_seq_len = min(max_seq_len, self.spec.max_positions)

@@ -132,6 +132,34 @@ class Model:
         head = tensors[self.spec.head_name] if self.spec.head_name is not None else self.embedding
         self.head = Linear(head)
 
+    def linears(self) -> List[Linear]:
+        """Every Linear a block's parts hold as an attribute, in layer order."""
+        return [v for b in self.blocks for part in b.parts() for v in vars(part).values()
+                if isinstance(v, Linear)]
+
+    def tune_products(self, row_counts, say=None) -> List[dict]:
+        """For every row count, has the vendor GEMM library's algorithms timed for each shape of
+        bf16 Linear that goes to the library at that many rows (``ops.kernels.gemm_vendor_tune``;
+        the same projection of all layers shares a shape and the layers' weights are used in
+        turn).  Seconds per shape: start-up work.  Returns one record per (rows, shape)."""
+        from ..ops.gemm_bf16 import use_skinny
+        shapes: Dict[tuple, List[Linear]] = {}
+        for lin in self.linears():
+            if lin.weight.is_cuda and lin.weight.dtype == torch.bfloat16:
+                shapes.setdefault((lin.out_features, lin.in_features, lin.halves), []).append(lin)
+        report = []
+        for rows in sorted(set(int(r) for r in row_counts)):
+            for (n, k, halves), lins in shapes.items():
+                if lins[0].tiled is not None and (use_skinny(rows, n, k, halves == 2) or use_skinny(rows, n, k)):
+                    continue                                    # the few-rows kernel takes these
+                first, best, tried = K.gemm_vendor_tune(rows, [lin.weight for lin in lins[:16]])
+                report.append(dict(rows=rows, n=n, k=k, heuristic_us=round(first, 2), kept_us=round(best, 2),
+                                   algorithms_run=tried))
+                if say is not None:
+                    say(f"vendor product {rows} x {k} -> {n}: {first:.1f} us by the library's choice, "
+                        f"{best:.1f} us by the fastest of {tried}")
+        return report
+
     # ---- forward
     def forward(self, batch, cache) -> torch.Tensor:
         """Runs the batch's tokens through every layer call and returns fp32 logits

@@ -355,6 +355,43 @@ def gemm_vendor(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
     return True
 
 
+def gemm_vendor_tune(rows: int, weights, out_dtype: torch.dtype = torch.bfloat16) -> tuple:
+    """Finds the vendor library's fastest algorithm for products of ``rows`` rows with weights of
+    the shape of ``weights`` (bf16 matrices of one shape, e.g. the same projection of every
+    layer; they are used in turn so that each comes from memory) and keeps it for later
+    :func:`gemm_vendor` calls of that shape.  Runs every algorithm the library has for the shape:
+    seconds, at start-up, never inside a graph capture.  A winner whose product differs from the
+    heuristic's choice by more than rounding is dropped again.  Returns (microseconds of the
+    heuristic's choice, microseconds of the one kept, algorithms run)."""
+    import ctypes
+    weights = list(weights)
+    if not weights or rows < 1:
+        raise KernelError("gemm_vendor_tune: needs at least one weight and one row")
+    n, k = weights[0].shape
+    for w in weights:
+        if w.shape != (n, k) or w.dtype != torch.bfloat16 or not w.is_cuda or not w.is_contiguous():
+            raise KernelError("gemm_vendor_tune: weights must be contiguous bf16 matrices of one shape on the GPU")
+    dev = weights[0].device
+    x = (torch.randn((rows, k), device=dev, dtype=torch.float32) * 0.5).to(torch.bfloat16)
+    out = torch.empty((rows, n), dtype=out_dtype, device=dev)
+    if not gemm_vendor(x, weights[0], out):
+        return (-1.0, -1.0, 0)
+    before = out.float()
+    ptrs = (ctypes.c_void_p * len(weights))(*[w.data_ptr() for w in weights])
+    first, best, tried = ctypes.c_float(), ctypes.c_float(), ctypes.c_int()
+    check(hip_lib().kva_gemm_vendor_tune(_dev(out, "out"), _dev(x, "x"), ptrs, len(weights), rows, n, k, k, n,
+                                         1 if out_dtype == torch.float32 else 0, _stream(),
+                                         ctypes.byref(first), ctypes.byref(best), ctypes.byref(tried)),
+          "gemm_vendor_tune")
+    gemm_vendor(x, weights[0], out)
+    scale = float(before.abs().max())
+    if not float((out.float() - before).abs().max()) <= 0.02 * scale:
+        check(hip_lib().kva_gemm_vendor_forget(rows, n, k, k, n, 1 if out_dtype == torch.float32 else 0),
+              "gemm_vendor_forget")
+        return (first.value, first.value, tried.value)
+    return (first.value, best.value, tried.value)
+
+
 def gemm_skinny_supported(m: int, n: int, k: int) -> bool:
     return bool(hip_lib().kva_gemm_skinny_supported(int(m), int(n), int(k)))
 

@@ -53,6 +53,8 @@ _HIP_SIGNATURES = {
     "kva_gemm_nt_f32": [P, P, P, I, I, I, I, I, I, P],
     "kva_gemm_vendor": [P, P, P, I, I, I, I, I, I, P],
     "kva_gemm_vendor_init": [],
+    "kva_gemm_vendor_tune": [P, P, P, I, I, I, I, I, I, I, P, P, P, P],
+    "kva_gemm_vendor_forget": [I, I, I, I, I, I],
     "kva_sample": [P, P, I, I, I, P, P, F, P, U, P, P, I, P, P],
     "kva_mark_tokens": [P, P, P, I, I, P],
 }

@@ -254,3 +254,22 @@ def test_activations_pass_between_two_products_in_lane_order(m, inter, hidden, g
         assert torch.equal(u, v)
     with pytest.raises(K.KernelError):
         K.TiledRows(17, 64, gpu)
+
+
+def test_vendor_product_keeps_the_fastest_algorithm_and_the_same_result(gpu):
+    """Timing every algorithm of the vendor library for a shape keeps one that is no slower than
+    the library's own choice and computes the same product."""
+    m, n, k = 64, 512, 1024
+    ws = [rnd(n, k, scale=0.05, seed=s).to(gpu) for s in range(3)]
+    x = rnd(m, k, seed=9).to(gpu)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=gpu)
+    assert K.gemm_vendor(x, ws[1], out)
+    before = out.clone()
+    first, best, tried = K.gemm_vendor_tune(m, ws)
+    assert tried >= 1 and 0 < best <= first
+    assert K.gemm_vendor(x, ws[1], out)
+    want = x.double().cpu() @ ws[1].double().cpu().t()
+    for got in (before, out):
+        assert (got.double().cpu() - want).abs().max() / want.abs().max() <= 2 ** -8
+    with pytest.raises(K.KernelError):
+        K.gemm_vendor_tune(m, [ws[0], rnd(n, k + 32, seed=1).to(gpu)])
