@@ -37,7 +37,7 @@ def test_embed_gather(dtype, table_dtype, gpu):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("width", [50, 64, 2050, 4096])
+@pytest.mark.parametrize("width", [50, 64, 520, 1000, 2048, 2050, 4096, 4104])
 def test_rmsnorm_plain_fused_and_gathered(dtype, width, gpu):
     dt = DT[dtype]
     x, d, w = rnd(9, width, dtype=dt), rnd(9, width, dtype=dt, seed=1), (1 + 0.1 * rnd(width, seed=2)).to(dt)
