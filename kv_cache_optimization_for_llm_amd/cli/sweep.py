@@ -76,6 +76,7 @@ def run_one(args, shape: str, batch: int, mode: str) -> dict:
     pool = args.cache_tokens or seats * (longest + 2 * args.page_size) * (2 if mode == "contiguous" else 1)
     engine = Engine(None, EngineOptions(dtype="bfloat16", cache_mode=mode, page_size=args.page_size,
                                         cache_tokens=pool, max_seqs=seats, max_seq_len=longest,
+                                        use_graphs=not args.no_graphs,
                                         gemm_tune_rows=[seats] if args.tune_gemm and seats > 16 else []),
                     config_dict=cfg, random_seed=args.seed)
     runner = Runner(engine, ServeOptions(ignore_eos=True, max_batch_tokens=args.max_batch_tokens,
@@ -177,6 +178,7 @@ def main(argv=None) -> int:
     ap.add_argument("--chunk-size", type=int, default=None)
     ap.add_argument("--tune-gemm", action="store_true",
                     help="time the vendor GEMM library's algorithms at start-up for decode batches above 16")
+    ap.add_argument("--no-graphs", action="store_true", help="launch every step's kernels one by one")
     ap.add_argument("--no-run-ahead", action="store_true")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--out", default=None, help="also append the lines to this file")

@@ -55,6 +55,7 @@ class StepBatch:
     logits_for_all_rows: bool = False    # logit_rows is exactly 0, 1, ..., T-1
     feedback: torch.Tensor = None        # device int32: tokens that negative token_ids stand for
     meta_provider: object = None         # callable(group, row_tiles) -> attention items, or None
+    static_items: bool = False           # a captured step: every set of attention items is prepared ahead
     _items: Dict[tuple, tuple] = field(default_factory=dict, repr=False)
 
     def attention_items(self, group: int, row_tiles: int = 1, which: str = "all"):
@@ -73,36 +74,14 @@ class StepBatch:
                 if made is not None:
                     self._items[key] = made
                     return made
-            lens = np.diff(self.h_entry_q_start)
-            ent, row0 = [np.zeros(0, np.int32)], [np.zeros(0, np.int32)]
-            for e, n in enumerate(lens):
-                if which != "all" and (int(n) * group > 16) != (which == "long"):
-                    continue
-                starts = np.arange(0, int(n) * group, 16 * row_tiles, dtype=np.int32)
-                ent.append(np.full(starts.shape[0], e, dtype=np.int32))
-                row0.append(starts)
-            ent, row0 = np.concatenate(ent), np.concatenate(row0)
+            if self.static_items:
+                raise RuntimeError(f"attention items {key} were not prepared for this captured step")
+            ent, row0, meta = attention_work_items(self.h_entry_q_start, self.h_entry_start_pos,
+                                                   self.h_entry_seat, group, row_tiles, which)
             n = ent.shape[0]
-            parts = [ent, row0]
-            known = self.h_entry_start_pos is not None and self.h_entry_seat is not None
-            if known:
-                if n > 1:
-                    # most keys first: the kernel hands out items in list order (and may give a
-                    # wavefront the i-th and the i-th last), so the long ones should start early
-                    last_row = np.minimum(row0 + 16 * row_tiles, lens[ent] * group) - 1
-                    keys = self.h_entry_start_pos[ent] + last_row // group + 1
-                    order = np.argsort(-keys, kind="stable")
-                    ent, row0 = ent[order], row0[order]
-                    parts = [ent, row0]
-                meta = np.zeros((n, 8), dtype=np.int32)
-                meta[:, 0] = self.h_entry_q_start[:-1][ent]
-                meta[:, 1] = lens[ent]
-                meta[:, 2] = self.h_entry_start_pos[ent]
-                meta[:, 3] = self.h_entry_seat[ent]
-                meta[:, 4] = row0
-                parts.append(meta.reshape(-1))
+            parts = [ent, row0] + ([meta.reshape(-1)] if meta is not None else [])
             dev = torch.from_numpy(np.concatenate(parts)).to(self.token_ids.device, non_blocking=True)
-            self._items[key] = (dev[:n], dev[n:2 * n], dev[2 * n:].view(n, 8) if known else None)
+            self._items[key] = (dev[:n], dev[n:2 * n], dev[2 * n:].view(n, 8) if meta is not None else None)
         return self._items[key]
 
     def mean_keys_of_long_entries(self) -> float:
@@ -114,6 +93,39 @@ class StepBatch:
         if not long.any():
             return 0.0
         return float(((self.h_entry_start_pos[long] + (lens[long] + 1) / 2) * lens[long]).sum() / lens[long].sum())
+
+
+def attention_work_items(entry_q_start: np.ndarray, entry_start_pos, entry_seat, group: int,
+                         row_tiles: int, which: str):
+    """Host arrays ``(entry, row0, meta)`` of :meth:`StepBatch.attention_items`; ``meta`` is
+    ``None`` when start positions or seats are not known on the host.  The number of items depends
+    on the entries' lengths, ``group``, ``row_tiles`` and ``which`` alone."""
+    lens = np.diff(entry_q_start)
+    ent, row0 = [np.zeros(0, np.int32)], [np.zeros(0, np.int32)]
+    for e, n in enumerate(lens):
+        if which != "all" and (int(n) * group > 16) != (which == "long"):
+            continue
+        starts = np.arange(0, int(n) * group, 16 * row_tiles, dtype=np.int32)
+        ent.append(np.full(starts.shape[0], e, dtype=np.int32))
+        row0.append(starts)
+    ent, row0 = np.concatenate(ent), np.concatenate(row0)
+    n = ent.shape[0]
+    if entry_start_pos is None or entry_seat is None:
+        return ent, row0, None
+    if n > 1:
+        # most keys first: the kernel hands out items in list order (and may give a
+        # wavefront the i-th and the i-th last), so the long ones should start early
+        last_row = np.minimum(row0 + 16 * row_tiles, lens[ent] * group) - 1
+        keys = entry_start_pos[ent] + last_row // group + 1
+        order = np.argsort(-keys, kind="stable")
+        ent, row0 = ent[order], row0[order]
+    meta = np.zeros((n, 8), dtype=np.int32)
+    meta[:, 0] = entry_q_start[:-1][ent]
+    meta[:, 1] = lens[ent]
+    meta[:, 2] = entry_start_pos[ent]
+    meta[:, 3] = entry_seat[ent]
+    meta[:, 4] = row0
+    return ent, row0, meta
 
 
 def _align(n: int, a: int = 4) -> int:

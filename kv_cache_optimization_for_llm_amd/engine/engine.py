@@ -43,7 +43,8 @@ class EngineOptions:
     cache_tokens: Optional[int] = None  # pool size in tokens (default: max_seqs * max_seq_len)
     max_seqs: int = 8                   # seats (reference: MAX_SEQUENCES)
     max_seq_len: Optional[int] = None   # longest request (default: max_position_embeddings)
-    use_graphs: bool = True             # replay decode-only steps as HIP graphs (bfloat16 engine)
+    use_graphs: bool = True             # replay decode-only steps, and steps with prompt portions whose
+                                        # shape comes back, as HIP graphs (bfloat16 engine)
     # Row counts (tokens per step) for which the vendor GEMM library's algorithms are timed at
     # start-up and the fastest kept, e.g. the prompt portion size and large decode batches
     # (bfloat16 engine; a few seconds per row count and matrix shape).  Empty: the library's own choice.
@@ -111,9 +112,11 @@ class Engine:
         # next step's single-token entries may name a row of it instead of a token id
         self.feedback = torch.zeros(max(1, options.max_seqs), dtype=torch.int32, device=self.device)
         self.graphs = None
+        self.portion_graphs = None
         if options.use_graphs and self.dtype == torch.bfloat16 and self.model.graph_safe():
-            from .graphs import DecodeGraphs
+            from .graphs import DecodeGraphs, PortionGraphs
             self.graphs = DecodeGraphs(self.model, self.cache, self.device, self.feedback)
+            self.portion_graphs = PortionGraphs(self.model, self.cache, self.device, self.feedback)
 
     # ------------------------------------------------------------------ requests
     def has_request(self, request_id) -> bool:
@@ -156,7 +159,9 @@ class Engine:
     # ------------------------------------------------------------------ the step
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Runs one batch; returns fp32 logits ``[wanted places, vocab]`` on the device, in the
-        order of the entries and of each entry's ``want``."""
+        order of the entries and of each entry's ``want``.  A step replayed from a graph returns
+        the graph's own buffer: it holds until the next step of the same shape, so copy what has
+        to outlive that."""
         logits = self._run(entries)
         self.finish(entries)
         return logits
@@ -192,6 +197,23 @@ class Engine:
             slot_maps = [[self.cache.slot_mapping(seat, start, len(arr), g.index)
                           for seat, start, arr in zip(seats, starts, toks)] for g in groups]
             self.cache.flush_tables()
+            if self.portion_graphs is not None:
+                # a step shape that has been seen before runs from its graph
+                lens = [len(t) for t in toks]
+                first = np.cumsum([0] + lens[:-1])
+                key = self.portion_graphs.shape_key(lens, starts, [int(f) + int(i) for f, w in zip(first, wants) for i in w])
+                if key is not None:
+                    logits = self.portion_graphs.run(
+                        key, np.concatenate([np.asarray(t, dtype=np.int32) for t in toks]),
+                        np.asarray(seats, dtype=np.int32), np.asarray(starts, dtype=np.int32),
+                        [np.concatenate(m).astype(np.int32) for m in slot_maps])
+                    if logits is not None:
+                        return logits
+                    batch = build_batch(seats, starts, toks, wants, slot_maps, self.device)
+                    batch.feedback = self.feedback
+                    logits = self.model.forward(batch, self.cache)
+                    self.portion_graphs.note(key, batch)
+                    return logits
         batch = build_batch(seats, starts, toks, wants, slot_maps, self.device)
         batch.feedback = self.feedback
         return self.model.forward(batch, self.cache)

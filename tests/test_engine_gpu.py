@@ -252,6 +252,61 @@ def test_graph_replays_equal_eager_steps_with_work_in_between(model_dirs, gpu):
     assert a.graphs.replays >= 30
 
 
+def test_portion_graph_replays_equal_eager_steps(gpu, monkeypatch):
+    """Steps with prompt portions whose shape comes back run from a graph of that shape: every
+    replay is checked against the same step run eagerly by a second engine (whose steps are the
+    eager work between the replays), at layer sizes where the vendor library's large-product
+    kernels take part; portions alone, portions beside decoded tokens, pages used again.  A
+    graph cuts the keys into splits by its context bucket, an eager step by the context it sees:
+    here the eager steps are given the bucket too, and then every replay must be bit for bit
+    what the eager step gives."""
+    import kv_cache_optimization_for_llm_amd.engine.engine as engine_module
+    from kv_cache_optimization_for_llm_amd.engine.graphs import context_bucket
+    plain_build = engine_module.build_batch
+
+    def build_with_bucket(*args, **kwargs):
+        batch = plain_build(*args, **kwargs)
+        batch.max_context = context_bucket(batch.max_context)
+        return batch
+    monkeypatch.setattr(engine_module, "build_batch", build_with_bucket)
+    cfg = dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=1531, hidden_size=2048,
+               intermediate_size=8192, num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8,
+               head_dim=64, rms_norm_eps=1e-5, rope_theta=500000.0, max_position_embeddings=8192,
+               tie_word_embeddings=True, hidden_act="silu", torch_dtype="bfloat16")
+    opts = dict(dtype="bfloat16", max_seqs=4, max_seq_len=4608, cache_tokens=3 * 4608)
+    a = Engine(None, EngineOptions(use_graphs=True, **opts), config_dict=cfg, random_seed=3)
+    b = Engine(None, EngineOptions(use_graphs=False, **opts), config_dict=cfg, random_seed=3)
+    rng = np.random.default_rng(1)
+    toks = lambda n: [int(t) for t in rng.integers(0, 1531, n)]
+    n_steps = 0
+
+    def both(step):
+        nonlocal n_steps
+        la, lb = a.step(step), b.step(step)
+        torch.cuda.synchronize()
+        assert torch.equal(la, lb), f"step {n_steps} from its graph is not what the eager step gives"
+        n_steps += 1
+
+    for round_ in range(2):            # the second round reuses the pages the first gave back
+        # three prompts in portions of 512, each alone in its step
+        for chunk in range(8):
+            for r in ("x", "y", "z"):
+                both([StepEntry(r, toks(512), [511] if chunk >= 5 else [])])
+        # two of them decode beside portions of a fourth request; then portions of 200 beside three decoding
+        for r in ("x",):
+            a.release(r), b.release(r)
+        for i in range(6):
+            both([StepEntry("y", toks(1), [0]), StepEntry("z", toks(1), [0]), StepEntry("w", toks(256), [255])])
+        for i in range(5):
+            both([StepEntry("y", toks(1), [0]), StepEntry("z", toks(1), [0]), StepEntry("w", toks(1), [0]),
+                  StepEntry("x", toks(200), [])])
+        for r in ("x", "y", "z", "w"):
+            a.release(r), b.release(r)
+    a.cache.check(), b.cache.check()
+    assert a.portion_graphs.captures >= 4 and a.portion_graphs.replays >= 40, \
+        (a.portion_graphs.captures, a.portion_graphs.replays, n_steps)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_contiguous_mode_gives_the_same_logits(dtype, model_dirs, gpu):
     name = "A"
