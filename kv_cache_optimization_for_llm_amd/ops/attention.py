@@ -17,9 +17,10 @@ _MIN_KEYS_PER_SPLIT = 128
 _WIDE_MIN_WAVES = 1024
 _PAIR_MIN_WAVES = 2048      # two items per wavefront once that still leaves a wavefront per SIMD
 # The workgroup kernel (128 query rows share each key block through LDS) pays one barrier per key
-# block: it wins once there are three workgroups per compute unit, or one per unit when the rows
-# visit thousands of keys each (measured: 2,048-token prompt from position 0 a tie, 4,096 1.5x).
-_LDS_MIN_GROUPS = 256
+# block: it wins once there are three workgroups per compute unit, or one per two units when the
+# rows visit thousands of keys each (measured: 2,048-token prompt from position 0 a tie, 4,096 1.5x;
+# portions of 512 tokens of an 8,192-token prompt, 128 workgroups, 5 % faster; of 256 tokens slower).
+_LDS_MIN_GROUPS = 128
 _LDS_MANY_GROUPS = 768
 _LDS_MIN_MEAN_KEYS = 2048
 
