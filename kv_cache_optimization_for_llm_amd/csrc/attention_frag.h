@@ -28,3 +28,9 @@ union Frag4 {
 __device__ inline b16x2 pack_bf16(float a, float b) {
     return __builtin_convertvector(f32x2{a, b}, b16x2);
 }
+
+// attention_mfma.hip: merge of key-split partials (see there)
+int kva_attention_merge_launch(void *out, const float *part_o, const float *part_ml, int head_dim, int splits,
+                               const int *item_meta, const int *item_entry, const int *item_row0,
+                               const int *entry_q_start, int num_items, int rows_per_item, int total_rows,
+                               int num_q_heads, int num_kv_heads, int all_rows, hipStream_t stream);

@@ -13,7 +13,10 @@
 //
 // The arithmetic per block is the other kernel's: S^T = K Q^T, online softmax in fp32 per query
 // row with a lazily re-based reference, O^T += V^T P^T with P taken from the registers S^T came
-// out in.  Every row's keys lie in one workgroup, so there are no splits and no merge.
+// out in.  Usually every row's keys lie in one workgroup.  When a step has too few workgroups to
+// fill the chip but each walks thousands of keys (a portion late in a long prompt), the keys are
+// cut into `splits` ranges of `keys_per_split`, one workgroup each; a split writes un-normalised
+// partials (o, m, l) as the one-wavefront kernel does and the same merge kernel combines them.
 //
 // Reference: the same recurrence as the tiled prefill kernel base/src/kernels.cu:361-466, which
 // shares K/V tiles of 32 keys among the 8 query rows of a 256-thread block and cannot read keys
@@ -38,11 +41,12 @@ struct LdsGeom {
 
 template <int D>
 __device__ __forceinline__ void
-attention_lds_item(char *lds, bf16_t *__restrict__ out, const bf16_t *__restrict__ q, int q_row_stride,
+attention_lds_item(char *lds, bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
+                   const bf16_t *__restrict__ q, int q_row_stride,
                    const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
                    const int *__restrict__ block_table, int max_blocks,
                    const int *__restrict__ item_meta, int num_q_heads, int num_kv_heads, float scale,
-                   int window, const int item, const int kvh) {
+                   int window, int splits, int keys_per_split, const int item, const int kvh, const int split) {
     using Geo = LdsGeom<D>;
     constexpr int RT = 2, NKS = D / 32, NDT = D / 16;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -83,8 +87,13 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, const bf16_t *__restrict
     const int g_hi = start_pos + g_last / G;
     const int g_first_pos = start_pos + row0 / G;
     const int g_lo = (window > 0 && g_first_pos - window + 1 > 0) ? g_first_pos - window + 1 : 0;
-    const int k_begin = g_lo & ~31;
-    const int k_end = g_hi + 1;
+    int k_begin = g_lo & ~31;
+    int k_end = g_hi + 1;
+    if (splits > 1) {               // uniform over the workgroup; an empty range leaves m = -inf, l = 0
+        const int s_lo = split * keys_per_split, s_hi = s_lo + keys_per_split;
+        if (s_lo > k_begin) k_begin = s_lo;
+        if (s_hi < k_end) k_end = s_hi;
+    }
     const int lo_tile = g_lo & ~15, hi_tile = g_hi & ~15;
 
     // ---- Q^T operand: lane (r, g) holds Q[row r][ks * 32 + g * 8 ...]
@@ -288,6 +297,18 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, const bf16_t *__restrict
     for (int rt = 0; rt < RT; ++rt) {
         if (!row_valid[rt]) continue;
         const size_t orow = (size_t)(q_start + tq[rt]) * num_q_heads + head[rt];
+        if (splits > 1) {
+            float *dst = part_o + (orow * splits + split) * D;
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt)
+                *reinterpret_cast<float4 *>(dst + dt * 16 + 4 * g) =
+                    make_float4(o[rt][dt][0], o[rt][dt][1], o[rt][dt][2], o[rt][dt][3]);
+            if (g == 0) {
+                part_ml[(orow * splits + split) * 2] = m[rt] * scale2;   // the merge works in the base-2 domain
+                part_ml[(orow * splits + split) * 2 + 1] = ol[rt][0];
+            }
+            continue;
+        }
         const float inv = 1.f / ol[rt][0];
         bf16_t *dst = out + orow * D;
 #pragma unroll
@@ -305,31 +326,35 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, const bf16_t *__restrict
 // takes item w and then item n-1-w of the list, which the caller orders by keys visited.
 template <int D>
 __device__ __forceinline__ void
-attention_lds_body(bf16_t *__restrict__ out, const bf16_t *__restrict__ q, int q_row_stride,
+attention_lds_body(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
+                   const bf16_t *__restrict__ q, int q_row_stride,
                    const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
                    const int *__restrict__ block_table, int max_blocks,
                    const int *__restrict__ item_meta, int num_items, int pair, int num_q_heads,
-                   int num_kv_heads, float scale, int window) {
+                   int num_kv_heads, float scale, int window, int splits, int keys_per_split) {
     using Geo = LdsGeom<D>;
     __shared__ __align__(16) char lds[2 * Geo::STAGE_BYTES];
     const int kvh = blockIdx.x % num_kv_heads;
-    const int w = blockIdx.x / num_kv_heads;
-    attention_lds_item<D>(lds, out, q, q_row_stride, k_cache, v_cache, block_table, max_blocks, item_meta,
-                          num_q_heads, num_kv_heads, scale, window, w, kvh);
+    const int w = blockIdx.x / num_kv_heads, split = blockIdx.z;
+    attention_lds_item<D>(lds, out, part_o, part_ml, q, q_row_stride, k_cache, v_cache, block_table, max_blocks,
+                          item_meta, num_q_heads, num_kv_heads, scale, window, splits, keys_per_split, w, kvh, split);
     const int other = num_items - 1 - w;
     if (pair && other > w)      // the last barrier of the first item has passed: LDS is free again
-        attention_lds_item<D>(lds, out, q, q_row_stride, k_cache, v_cache, block_table, max_blocks, item_meta,
-                              num_q_heads, num_kv_heads, scale, window, other, kvh);
+        attention_lds_item<D>(lds, out, part_o, part_ml, q, q_row_stride, k_cache, v_cache, block_table, max_blocks,
+                              item_meta, num_q_heads, num_kv_heads, scale, window, splits, keys_per_split, other, kvh,
+                              split);
 }
 
 #define LDS_KERNEL_PARAMS                                                                          \
-    bf16_t *__restrict__ out, const bf16_t *__restrict__ q, int q_row_stride,                      \
+    bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,             \
+    const bf16_t *__restrict__ q, int q_row_stride,                                                \
     const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,                        \
     const int *__restrict__ block_table, int max_blocks, const int *__restrict__ item_meta,        \
-    int num_items, int pair, int num_q_heads, int num_kv_heads, float scale, int window
+    int num_items, int pair, int num_q_heads, int num_kv_heads, float scale, int window,           \
+    int splits, int keys_per_split
 #define LDS_KERNEL_ARGS                                                                            \
-    out, q, q_row_stride, k_cache, v_cache, block_table, max_blocks, item_meta, num_items, pair,   \
-    num_q_heads, num_kv_heads, scale, window
+    out, part_o, part_ml, q, q_row_stride, k_cache, v_cache, block_table, max_blocks, item_meta,   \
+    num_items, pair, num_q_heads, num_kv_heads, scale, window, splits, keys_per_split
 
 template <int D>
 __global__ void __launch_bounds__(256) attention_lds_kernel(LDS_KERNEL_PARAMS) {
@@ -352,11 +377,18 @@ extern "C" int kva_attention_lds_supported(int head_dim, int page_size) {
 // item_meta: [num_items, 8] int32 = (q_start, q_len, start_pos, seat, row0, 0, 0, 0) per item of
 // 128 query rows (row0 a multiple of 128).  q: bf16 rows `q_row_stride` elements apart; out
 // [tokens, num_q_heads * head_dim] bf16.
-extern "C" int kva_attention_lds(void *out, const void *q, int q_row_stride, const void *k_cache,
-                                 const void *v_cache, const int *block_table, int max_blocks,
+// With splits > 1: part_o [tokens * num_q_heads, splits, head_dim] and part_ml [.., splits, 2] fp32
+// take the partials, keys_per_split is a multiple of 32, and the merge runs after the kernel: over
+// every row of out (`all_rows`: the items cover them all) or over the items' rows alone.
+extern "C" int kva_attention_lds(void *out, float *part_o, float *part_ml, const void *q, int q_row_stride,
+                                 const void *k_cache, const void *v_cache, const int *block_table, int max_blocks,
                                  const int *item_meta, int num_items, int pair, int num_q_heads,
                                  int num_kv_heads, int head_dim, int page_size, float scale, int window,
+                                 int splits, int keys_per_split, int total_rows, int all_rows,
                                  hipStream_t stream) {
+    KVA_REQUIRE(splits >= 1 && splits <= 256 && num_kv_heads <= 65535, "attention_lds: 1..256 splits");
+    KVA_REQUIRE(splits == 1 || (keys_per_split > 0 && keys_per_split % 32 == 0 && part_o && part_ml),
+                "attention_lds: splits need a key count that is a multiple of 32 and a workspace");
     KVA_REQUIRE(num_items >= 0 && num_q_heads > 0 && num_kv_heads > 0 && max_blocks > 0, "attention_lds: bad sizes");
     KVA_REQUIRE(num_q_heads % num_kv_heads == 0, "attention_lds: %d query heads is not a multiple of %d kv heads",
                 num_q_heads, num_kv_heads);
@@ -368,11 +400,12 @@ extern "C" int kva_attention_lds(void *out, const void *q, int q_row_stride, con
     if (num_items == 0) return KVA_OK;
     const int groups = pair ? (num_items + 1) / 2 : num_items;
     KVA_REQUIRE((long)groups * num_kv_heads < (1L << 31), "attention_lds: too many work items");
-    dim3 grid(groups * num_kv_heads), block(256);
+    dim3 grid(groups * num_kv_heads, 1, splits), block(256);
 #define LAUNCH(KERNEL, DD)                                                                          \
-    hipLaunchKernelGGL((KERNEL<DD>), grid, block, 0, stream, (bf16_t *)out, (const bf16_t *)q,      \
-                       q_row_stride, (const bf16_t *)k_cache, (const bf16_t *)v_cache, block_table, \
-                       max_blocks, item_meta, num_items, pair, num_q_heads, num_kv_heads, scale, window)
+    hipLaunchKernelGGL((KERNEL<DD>), grid, block, 0, stream, (bf16_t *)out, part_o, part_ml,        \
+                       (const bf16_t *)q, q_row_stride, (const bf16_t *)k_cache,                    \
+                       (const bf16_t *)v_cache, block_table, max_blocks, item_meta, num_items, pair, \
+                       num_q_heads, num_kv_heads, scale, window, splits, keys_per_split)
     switch (head_dim) {
     case 32: LAUNCH(attention_lds_kernel_3, 32); break;
     case 64: LAUNCH(attention_lds_kernel_3, 64); break;
@@ -381,5 +414,8 @@ extern "C" int kva_attention_lds(void *out, const void *q, int q_row_stride, con
     }
 #undef LAUNCH
     KVA_CHECK_LAUNCH("attention_lds");
+    if (splits > 1)
+        return kva_attention_merge_launch(out, part_o, part_ml, head_dim, splits, item_meta, nullptr, nullptr, nullptr,
+                                          num_items, 128, total_rows, num_q_heads, num_kv_heads, all_rows, stream);
     return KVA_OK;
 }

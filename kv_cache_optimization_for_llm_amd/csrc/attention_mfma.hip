@@ -401,7 +401,7 @@ attention_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_
     // Either one workgroup per row of `out` (the launch covered every row: item arrays null), or
     // one per (item, kv head, row of the item): then only the rows the items name are touched.
     size_t row = blockIdx.x;
-    if (item_entry != nullptr) {
+    if (item_entry != nullptr || item_meta != nullptr) {
         const int kvh = blockIdx.x % num_kv_heads, item = blockIdx.x / num_kv_heads;
         int row0, q_start, q_len;
         if (item_meta != nullptr) {
@@ -458,6 +458,27 @@ attention_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_
         for (int s = s0; s < splits; ++s) acc += po[(size_t)s * head_dim + j] * w_s[s];
         out[row * head_dim + j].bits = float_to_bf16_bits(acc * inv);
     }
+}
+
+// Merges the partials of `splits` key splits into `out`: over every row of `out` (`all_rows`), or
+// over the rows of the items alone, `rows_per_item` rows each, named by item_meta or by
+// (item_entry, item_row0, entry_q_start).  Shared by the two matrix-core attention kernels.
+int kva_attention_merge_launch(void *out, const float *part_o, const float *part_ml, int head_dim, int splits,
+                               const int *item_meta, const int *item_entry, const int *item_row0,
+                               const int *entry_q_start, int num_items, int rows_per_item, int total_rows,
+                               int num_q_heads, int num_kv_heads, int all_rows, hipStream_t stream) {
+    KVA_REQUIRE(splits >= 2 && splits <= MERGE_MAX_SPLITS && part_o && part_ml,
+                "attention_merge: 2..%d splits and their partial results are needed", MERGE_MAX_SPLITS);
+    if (all_rows)
+        hipLaunchKernelGGL(attention_merge_kernel, dim3(total_rows), dim3(64), 0, stream, (bf16_t *)out,
+                           part_o, part_ml, head_dim, splits, nullptr, nullptr, nullptr, nullptr,
+                           num_q_heads, num_kv_heads);
+    else
+        hipLaunchKernelGGL(attention_merge_kernel, dim3(num_items * num_kv_heads, rows_per_item), dim3(64),
+                           0, stream, (bf16_t *)out, part_o, part_ml, head_dim, splits, item_meta,
+                           item_entry, item_row0, entry_q_start, num_q_heads, num_kv_heads);
+    KVA_CHECK_LAUNCH("attention_merge");
+    return KVA_OK;
 }
 
 extern "C" int kva_attention_mfma_supported(int head_dim, int page_size) {
@@ -531,16 +552,9 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
 #undef CASE
 #undef LAUNCH
     KVA_CHECK_LAUNCH("attention_mfma");
-    if (splits > 1) {
-        if (all_rows)
-            hipLaunchKernelGGL(attention_merge_kernel, dim3(total_rows), dim3(64), 0, stream, (bf16_t *)out,
-                               part_o, part_ml, head_dim, splits, nullptr, nullptr, nullptr, nullptr,
-                               num_q_heads, num_kv_heads);
-        else
-            hipLaunchKernelGGL(attention_merge_kernel, dim3(num_items * num_kv_heads, 16 * row_tiles), dim3(64),
-                               0, stream, (bf16_t *)out, part_o, part_ml, head_dim, splits, item_meta,
-                               item_entry, item_row0, entry_q_start, num_q_heads, num_kv_heads);
-        KVA_CHECK_LAUNCH("attention_merge");
-    }
+    if (splits > 1)
+        return kva_attention_merge_launch(out, part_o, part_ml, head_dim, splits, item_meta, item_entry, item_row0,
+                                          entry_q_start, num_items, 16 * row_tiles, total_rows, num_q_heads,
+                                          num_kv_heads, all_rows, stream);
     return KVA_OK;
 }

@@ -19,10 +19,14 @@ _PAIR_MIN_WAVES = 2048      # two items per wavefront once that still leaves a w
 # The workgroup kernel (128 query rows share each key block through LDS) pays one barrier per key
 # block: it wins once there are three workgroups per compute unit, or one per two units when the
 # rows visit thousands of keys each (measured: 2,048-token prompt from position 0 a tie, 4,096 1.5x;
-# portions of 512 tokens of an 8,192-token prompt, 128 workgroups, 5 % faster; of 256 tokens slower).
+# portions of 512 tokens of an 8,192-token prompt, 128 workgroups, 5 % faster, and 25 % faster with
+# their keys cut into ranges so that about a thousand workgroups run; portions of 256 tokens no faster).
 _LDS_MIN_GROUPS = 128
 _LDS_MANY_GROUPS = 768
 _LDS_MIN_MEAN_KEYS = 2048
+# few workgroups that each walk thousands of keys: the keys are cut into ranges, one workgroup each
+_LDS_TARGET_GROUPS = 1024
+_LDS_MIN_KEYS_PER_SPLIT = 1024
 
 
 def choose_splits(num_items: int, num_kv_heads: int, max_context: int) -> tuple:
@@ -35,6 +39,17 @@ def choose_splits(num_items: int, num_kv_heads: int, max_context: int) -> tuple:
         return 1, 0
     per = (max_context + splits - 1) // splits
     per = (per + 31) // 32 * 32
+    splits = (max_context + per - 1) // per
+    return (splits, per) if splits > 1 else (1, 0)
+
+
+def choose_lds_splits(groups: int, max_context: int) -> tuple:
+    """(splits, keys_per_split) for the workgroup kernel."""
+    want = max(1, _LDS_TARGET_GROUPS // max(1, groups))
+    splits = min(want, max(1, max_context // _LDS_MIN_KEYS_PER_SPLIT))
+    if splits <= 1:
+        return 1, 0
+    per = ((max_context + splits - 1) // splits + 31) // 32 * 32
     splits = (max_context + per - 1) // per
     return (splits, per) if splits > 1 else (1, 0)
 
@@ -83,8 +98,10 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
         groups = items[0].shape[0] * num_kv_heads
         if items[2] is not None and groups >= _LDS_MIN_GROUPS and (
                 groups >= _LDS_MANY_GROUPS or batch.mean_keys_of_long_entries() >= _LDS_MIN_MEAN_KEYS):
+            splits, per = choose_lds_splits(groups, batch.max_context)
             K.attention_lds(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table, items[2], num_q_heads,
-                            num_kv_heads, head_dim, scale, window, False)
+                            num_kv_heads, head_dim, scale, window, False, splits, per,
+                            covers_all_rows=which == "all")
             done = True
     if not done:
         # two row tiles per wave, so each key and value loaded serves 32 query rows; whole key

@@ -308,12 +308,15 @@ def attention_lds_supported(head_dim: int, page_size: int) -> bool:
 def attention_lds(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cache: torch.Tensor,
                   v_cache: torch.Tensor, block_table: torch.Tensor, item_meta: torch.Tensor,
                   num_q_heads: int, num_kv_heads: int, head_dim: int, scale: float, window: int = 0,
-                  pair: bool = False) -> torch.Tensor:
+                  pair: bool = False, splits: int = 1, keys_per_split: int = 0,
+                  covers_all_rows: bool = True) -> torch.Tensor:
     """bf16 matrix-core attention for prompt portions: a workgroup of four wavefronts per 128
     query rows (row = token_in_step * (nq / nkv) + head_in_group) shares every key and value
     block through LDS.  ``item_meta`` ``[items, 8]`` int32: (q_start, q_len, start_pos, seat,
     row0, 0, 0, 0) with ``row0`` a multiple of 128.  With ``pair`` a workgroup takes item i and
-    item n-1-i of the list."""
+    item n-1-i of the list.  With ``splits`` > 1 the keys are cut into ranges of
+    ``keys_per_split`` (a multiple of 32), one workgroup each, and merged afterwards
+    (``covers_all_rows=False``: only over the items' rows, the others belong to another launch)."""
     tokens = out.shape[0]
     if out.dtype != torch.bfloat16 or q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16:
         raise KernelError("attention_lds: bfloat16 only")
@@ -324,11 +327,17 @@ def attention_lds(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cache
         raise KernelError("attention_lds: item_meta must be [items, 8] and the block table [seats, blocks]")
     if q.data_ptr() % 16 or q_row_stride < num_q_heads * head_dim:
         raise KernelError("attention_lds: q view is misaligned or its stride is too small")
+    part_o = part_ml = None
+    if splits > 1:
+        part_o = torch.empty((tokens * num_q_heads, splits, head_dim), dtype=torch.float32, device=out.device)
+        part_ml = torch.empty((tokens * num_q_heads, splits, 2), dtype=torch.float32, device=out.device)
     check(hip_lib().kva_attention_lds(
-        _dev(out, "out"), _dev(q, "q", contiguous=False), q_row_stride, _dev(k_cache, "k_cache"),
+        _dev(out, "out"), _opt(part_o, "part_o"), _opt(part_ml, "part_ml"),
+        _dev(q, "q", contiguous=False), q_row_stride, _dev(k_cache, "k_cache"),
         _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32), block_table.shape[1],
         _dev(item_meta, "item_meta", torch.int32), item_meta.shape[0], 1 if pair else 0, num_q_heads,
-        num_kv_heads, head_dim, k_cache.shape[2], float(scale), int(window), _stream()), "attention_lds")
+        num_kv_heads, head_dim, k_cache.shape[2], float(scale), int(window), int(splits), int(keys_per_split),
+        tokens * num_q_heads, 1 if covers_all_rows else 0, _stream()), "attention_lds")
     return out
 
 

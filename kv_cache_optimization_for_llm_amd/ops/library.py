@@ -43,7 +43,7 @@ _HIP_SIGNATURES = {
     "kva_attention_mfma_row_tiles": [I, I],
     "kva_attention_mfma_supported": [I, I],
     "kva_attention_lds_supported": [I, I],
-    "kva_attention_lds": [P, P, I, P, P, P, I, P, I, I, I, I, I, I, F, I, P],
+    "kva_attention_lds": [P, P, P, P, I, P, P, P, I, P, I, I, I, I, I, I, F, I, I, I, I, I, P],
     "kva_gemm_skinny": [P, P, P, I, I, I, I, I, I, P, I, I, F, P, P, I, P, P, I, I, P],
     "kva_gemm_skinny_sumsq_parts": [I],
     "kva_normed_rows_finish": [P, P, P, I, I, P, I, F, P],

@@ -353,21 +353,25 @@ def test_preempted_requests_finish_with_the_tokens_of_an_unpreempted_run(model_d
     assert got_t == want_t
 
 
-def test_prompt_portions_through_the_workgroup_attention_kernel(model_dirs, gpu, monkeypatch):
+@pytest.mark.parametrize("split_keys", [False, True])
+def test_prompt_portions_through_the_workgroup_attention_kernel(split_keys, model_dirs, gpu, monkeypatch):
     """The attention kernel that shares key blocks through LDS is chosen for steps with many long
     rows; with its thresholds lowered it runs on a tiny model: whole prompts, portions that start
     deep in a request, and portions beside decoded tokens (two launches) all match the plain
-    implementation."""
+    implementation - also with the keys cut into ranges of 64, one workgroup each, and merged."""
     from kv_cache_optimization_for_llm_amd.ops import attention as policy
     from kv_cache_optimization_for_llm_amd.ops import kernels as K
-    calls = {"lds": 0}
+    calls = {"lds": 0, "split": 0}
     real = K.attention_lds
 
     def counted(*a, **kw):
         calls["lds"] += 1
+        calls["split"] += 1 if a[13] > 1 else 0
         return real(*a, **kw)
     monkeypatch.setattr(policy, "_LDS_MIN_GROUPS", 1)
     monkeypatch.setattr(policy, "_LDS_MANY_GROUPS", 1)
+    if split_keys:
+        monkeypatch.setattr(policy, "_LDS_MIN_KEYS_PER_SPLIT", 64)
     monkeypatch.setattr(K, "attention_lds", counted)
     cfg, W = plain.load_model_dir(model_dirs["D"])
     eng = Engine(model_dirs["D"], EngineOptions(dtype="bfloat16", max_seqs=3, max_seq_len=512))
@@ -387,6 +391,7 @@ def test_prompt_portions_through_the_workgroup_attention_kernel(model_dirs, gpu,
     assert calls["lds"] == 2 * cfg["num_hidden_layers"]
     out = eng.step([StepEntry("a", pa[201:], list(range(99)))])          # a portion that starts at 201
     assert worst(out, ref["a"][201:]) <= TOL["bfloat16"]
+    assert calls["split"] == (calls["lds"] if split_keys else 0)
     eng.cache.check()
 
 

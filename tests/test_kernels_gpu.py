@@ -266,8 +266,8 @@ LONG_ENTRIES = [(0, 300), (40, 1), (200, 131), (5, 64), (0, 33)]
 
 @pytest.mark.parametrize("nq, nkv, d, window", [(4, 2, 32, 0), (32, 8, 64, 0), (8, 2, 64, 70), (6, 2, 96, 0),
                                                 (24, 8, 128, 0), (5, 1, 64, 0), (3, 3, 128, 150)])
-@pytest.mark.parametrize("pair", [False, True])
-def test_attention_with_keys_shared_through_lds(nq, nkv, d, window, pair, gpu):
+@pytest.mark.parametrize("pair, splits", [(False, 1), (True, 1), (False, 3), (True, 2), (False, 11)])
+def test_attention_with_keys_shared_through_lds(nq, nkv, d, window, pair, splits, gpu):
     """The workgroup kernel for prompt portions (128 query rows share each key block): long and
     short entries, entries that start deep in their request, groups that do not divide 128,
     windows, and work items taken in pairs."""
@@ -283,8 +283,21 @@ def test_attention_with_keys_shared_through_lds(nq, nkv, d, window, pair, gpu):
     rows.sort(key=lambda m: -(m[2] + (min(m[4] + 128, m[1] * group) - 1) // group))     # most keys first
     meta = torch.tensor(rows, dtype=torch.int32, device=gpu)
     out = torch.full((T, nq * d), float("nan"), dtype=torch.bfloat16, device=gpu)
-    K.attention_lds(dev["qkv"], stride, out, dev["kc"], dev["vc"], dev["table"], meta, nq, nkv, d, scale, window, pair)
-    close(out, want, torch.bfloat16, f"attention_lds pair={pair}", tol16=8e-3)
+    per = 0
+    if splits > 1:      # key ranges cut anywhere in blocks of 32: some are empty for the short entries
+        per = ((max(s + n for s, n in LONG_ENTRIES) + splits - 1) // splits + 31) // 32 * 32
+    K.attention_lds(dev["qkv"], stride, out, dev["kc"], dev["vc"], dev["table"], meta, nq, nkv, d, scale, window, pair,
+                    splits, per)
+    close(out, want, torch.bfloat16, f"attention_lds pair={pair} splits={splits}", tol16=8e-3)
+    if splits > 1:
+        # merged over the items' rows alone: rows of other launches are left as they are
+        some = meta[meta[:, 0] == int(qs[2])]
+        out2 = torch.full((T, nq * d), 7.0, dtype=torch.bfloat16, device=gpu)
+        K.attention_lds(dev["qkv"], stride, out2, dev["kc"], dev["vc"], dev["table"], some, nq, nkv, d, scale,
+                        window, False, splits, per, covers_all_rows=False)
+        lo, hi = int(qs[2]), int(qs[3])
+        assert torch.equal(out2[lo:hi], out[lo:hi]) or (out2[lo:hi].float() - out[lo:hi].float()).abs().max() < 1e-2
+        assert bool((out2[:lo] == 7.0).all()) and bool((out2[hi:] == 7.0).all())
 
 
 @pytest.mark.parametrize("slope", [0.0, 0.35, -0.35, 3.0])
