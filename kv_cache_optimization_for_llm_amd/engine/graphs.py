@@ -216,9 +216,10 @@ class PortionGraphs:
     for; its second step is captured over static buffers; later ones upload their indices and
     replay.  Logits come back in the shape's static buffer: they hold until its next step."""
 
-    MAX_TOKENS = 1024          # longer steps keep the device busy for longer than their launches take
+    MAX_TOKENS = 4096          # tokens of one captured step
     MAX_LOGIT_ROWS = 64        # a graph keeps its logits: [rows, vocabulary] fp32
-    MAX_SHAPES = 32            # captured shapes kept (least recently used goes first)
+    MAX_SHAPES = 32            # captured shapes kept (least recently used goes first) ...
+    MAX_KEPT_TOKENS = 16384    # ... and the tokens of all of them: a graph keeps its step's activations
     MAX_SEEN = 4096
 
     def __init__(self, model, cache, device, feedback=None):
@@ -256,9 +257,10 @@ class PortionGraphs:
             return None
         slot = self.slots.get(key)
         if slot is None:
-            while len(self.slots) >= self.MAX_SHAPES:
-                self.slots.popitem(last=False)
             lens, rows, bucket, _ = key
+            while self.slots and (len(self.slots) >= self.MAX_SHAPES or
+                                  sum(s.T for s in self.slots.values()) + sum(lens) > self.MAX_KEPT_TOKENS):
+                self.slots.popitem(last=False)
             slot = self.slots[key] = _PortionSlot(lens, rows, bucket, variants, len(self.cache.groups),
                                                   self.device, self.feedback)
         else:
