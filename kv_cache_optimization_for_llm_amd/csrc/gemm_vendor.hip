@@ -99,14 +99,17 @@ bool make_plan(int dev, const Key &key, Plan &p) {
              HIPBLAS_STATUS_SUCCESS;
     }
     if (ok) {
-        hipblasLtMatmulHeuristicResult_t result[1];
+        // the first of the heuristic's choices that is usable with this workspace
+        constexpr int kAsk = 8;
+        hipblasLtMatmulHeuristicResult_t result[kAsk];
         int returned = 0;
-        const hipblasStatus_t st = hipblasLtMatmulAlgoGetHeuristic(g_handle[dev], p.desc, p.a, p.b, p.c, p.c, pref, 1,
+        const hipblasStatus_t st = hipblasLtMatmulAlgoGetHeuristic(g_handle[dev], p.desc, p.a, p.b, p.c, p.c, pref, kAsk,
                                                                    result, &returned);
-        if (st == HIPBLAS_STATUS_SUCCESS && returned > 0 && result[0].state == HIPBLAS_STATUS_SUCCESS &&
-            result[0].workspaceSize <= kWorkspaceBytes) {
-            p.algo = result[0].algo;
-            p.found = true;
+        for (int i = 0; st == HIPBLAS_STATUS_SUCCESS && i < returned && i < kAsk && !p.found; ++i) {
+            if (result[i].state == HIPBLAS_STATUS_SUCCESS && result[i].workspaceSize <= kWorkspaceBytes) {
+                p.algo = result[i].algo;
+                p.found = true;
+            }
         }
     }
     if (pref) hipblasLtMatmulPreferenceDestroy(pref);
