@@ -307,6 +307,25 @@ def test_portion_graph_replays_equal_eager_steps(gpu, monkeypatch):
         (a.portion_graphs.captures, a.portion_graphs.replays, n_steps)
 
 
+@pytest.mark.parametrize("run_ahead", [False, True])
+def test_serving_with_small_portions_replays_portion_graphs(run_ahead, model_dirs, gpu):
+    """A small token budget and portions of 24 tokens: the same step shapes (a portion alone,
+    decoded tokens beside a portion) come back again and again and are replayed from graphs, with
+    the serving loop one step ahead of the device or not; every token is the plain model's choice."""
+    name = "D"
+    cfg, W = plain.load_model_dir(model_dirs[name])
+    prompts = prompts_for(name, [96, 120, 96, 72, 120, 96, 48, 96], seed=4)
+    llm = LLM(model_dirs[name], EngineOptions(dtype="bfloat16", max_seqs=3, max_seq_len=256, cache_tokens=512),
+              ServeOptions(chunk_size=24, max_batch_tokens=40, run_ahead=run_ahead))
+    got = llm.generate(prompts, max_new_tokens=12, ignore_eos=True)
+    for p, g in zip(prompts, got):
+        assert len(g) == 12
+        check_choices(cfg, W, p, g, "bfloat16")
+    pg = llm.engine.portion_graphs
+    assert pg.captures >= 2 and pg.replays >= 10, (pg.captures, pg.replays)
+    llm.engine.cache.check()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_contiguous_mode_gives_the_same_logits(dtype, model_dirs, gpu):
     name = "A"
