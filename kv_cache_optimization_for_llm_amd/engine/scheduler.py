@@ -263,6 +263,17 @@ class Scheduler:
                 committed[i] += n
             entries.append(PlanEntry(seq, [seq.next_token], seq.computed, sample=True))
         budget = self.max_batch_tokens - len(entries)
+        decode_pages = list(committed)          # pages the decoding requests take in this step
+
+        def prompt_pages_outstanding() -> List[int]:
+            """Pages the admitted requests still need to finish their prompts: a prompt is mapped
+            portion by portion, so what is free now is not all free for a newcomer."""
+            need = [0] * len(cache.groups)
+            for s in self.running:
+                if s.prefilling:
+                    for i, n in enumerate(cache.pages_needed(s.seat, len(s.prompt))):
+                        need[i] += n
+            return need
 
         def fit_tokens(seq: Sequence_, want: int) -> int:
             """Largest portion <= want whose pages are still free."""
@@ -314,7 +325,7 @@ class Scheduler:
             reserve = None
             if paged:
                 pages = (plen + cache.page_size - 1) // cache.page_size
-                free = [f - c for f, c in zip(self._free_pages(), committed)]
+                free = [f - d - o for f, d, o in zip(self._free_pages(), decode_pages, prompt_pages_outstanding())]
                 if any(pages > f for f in free):
                     if not self.running and not entries and any(pages > g.num_pages for g in cache.groups):
                         self.waiting.popleft()
@@ -344,6 +355,19 @@ class Scheduler:
             if self.on_admit:
                 self.on_admit(seq)
             add_portion(seq)
+
+        # Nothing to run although requests hold seats: every one of them is part-way through its
+        # prompt and no page is free (decoding neighbours that have since left took the pages their
+        # prompts were admitted against; requests that wait for their last token's value, which
+        # will free theirs, are excluded).  The newest gives its pages back and re-enters at the
+        # front of the queue; one alone that cannot go on does not fit the cache at all.
+        if paged and not entries and self.running and not self.closing \
+                and all(s.prefilling for s in self.running):
+            victims = sorted(self.running, key=lambda s: s.request.arrival)
+            if len(victims) > 1:
+                self._preempt(victims[-1], events)
+            else:
+                self._finish(victims[0], "kv_cache_exhausted", events)
         return StepPlan(entries, events)
 
     # ------------------------------------------------------------------ after the forward

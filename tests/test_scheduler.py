@@ -312,3 +312,46 @@ def test_planning_refuses_to_preempt_while_tokens_are_unseen_and_changes_nothing
     p3 = s.plan()
     assert [e.kind for e in p3.events] == ["preempted"] and p3.events[0].request_id == 1
     assert s.waiting[0].tokens[-2:] == [fake_token(1, 31), fake_token(1, 32)]
+
+
+def test_prompts_admitted_together_are_counted_with_the_pages_they_still_need():
+    """Two seats, 32 pages of 4 tokens, portions of 8: a prompt is mapped portion by portion, so
+    the pages free at admission are not all free for a second newcomer.  Prompts of 84 and 58
+    tokens (36 pages) must not both be admitted - they would stop half-way with no page left and
+    nothing to give one back."""
+    s = Scheduler(cache(pages=32, seqs=2, page=4, max_len=101), max_batch_tokens=64, chunk_size=8, ignore_eos=True)
+    lens = [63, 57, 12, 28, 84, 58, 16, 53]
+    for i, n in enumerate(lens):
+        s.add(Request(i, [8 + (j % 30) for j in range(n)], 16))
+    out, reasons, events, plans = run(s, max_steps=2000)
+    for i, n in enumerate(lens):
+        assert reasons[(i, 0)] == "length" and out[(i, 0)] == [fake_token(i, n + k) for k in range(16)]
+    for p in plans:
+        assert p.entries or p.events, "a plan with nothing to run and nothing to report"
+
+
+@pytest.mark.parametrize("ahead", [False, True])
+@pytest.mark.parametrize("seed", range(40))
+def test_random_tight_pools_always_finish(seed, ahead):
+    """Random prompts, budgets, portion sizes, page sizes and pools barely larger than the longest
+    request: every request ends, with its full budget of the right tokens unless the cache
+    could not hold it, and no page is lost."""
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    page = int(rng.choice([16, 8, 4]))
+    lens = [int(x) for x in rng.integers(1, 90, int(rng.integers(3, 9)))]
+    new = int(rng.integers(4, 20))
+    seats = int(rng.integers(2, 5))
+    longest = max(lens) + new + 1
+    pool = int(rng.integers(longest + page, seats * longest + 2 * page))
+    chunk = int(rng.choice([0, 8, 24, 64])) or None
+    s = Scheduler(cache(pages=(pool + page - 1) // page, seqs=seats, page=page, max_len=longest),
+                  max_batch_tokens=int(rng.choice([32, 64, 256])), chunk_size=chunk, ignore_eos=True)
+    for i, n in enumerate(lens):
+        s.add(Request(i, [8 + (j % 30) for j in range(n)], new))
+    out, reasons, events, plans = (run_ahead if ahead else run)(s, max_steps=4000)
+    for i, n in enumerate(lens):
+        assert reasons[(i, 0)] == "length", (i, reasons)
+        assert out[(i, 0)] == [fake_token(i, n + k) for k in range(new)]
+    s.cache.check()
+    assert s.cache.free_seats == seats
