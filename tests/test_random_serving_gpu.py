@@ -1,0 +1,64 @@
+"""The serving loop on seeded random workloads: small models, pools barely larger than the longest
+request (so requests are preempted and recomputed), small token budgets and portion sizes.
+Greedy tokens equal the plain model's; sampled tokens, end-of-sequence stops and the repetition
+penalty give the same output in a roomy cache and in a tight one, with the loop one step ahead of
+the device or not."""
+import numpy as np
+import pytest
+
+import plain_llama as plain
+from test_random_configs_gpu import random_config
+from kv_cache_optimization_for_llm_amd.engine.engine import EngineOptions
+from kv_cache_optimization_for_llm_amd.engine.runner import LLM, ServeOptions
+from kv_cache_optimization_for_llm_amd.weights.random_init import write_random_model
+
+pytestmark = pytest.mark.gpu
+
+
+def workload(case):
+    rng = np.random.default_rng(8800 + case)
+    cfg = random_config(rng)
+    cfg["vocab_size"] = vocab = int(rng.integers(20, 200))
+    cfg["eos_token_id"] = [int(x) for x in rng.choice(vocab, 2, replace=False)]
+    page = int(rng.choice([16, 8, 4]))
+    lengths = [int(x) for x in rng.integers(1, 80, int(rng.integers(3, 8)))]
+    new = int(rng.integers(5, 20))
+    seats = int(rng.integers(2, 5))
+    longest = max(lengths) + new + 1
+    tight = int(rng.integers(longest + page, 2 * longest + page))
+    prompts = [[int(t) for t in rng.integers(0, vocab, n)] for n in lengths]
+    return rng, cfg, page, prompts, new, seats, longest, tight
+
+
+@pytest.mark.parametrize("case", range(8))
+def test_greedy_tokens_in_a_tight_cache_are_the_plain_model_s(case, tmp_path, gpu):
+    rng, cfg, page, prompts, new, seats, longest, tight = workload(case)
+    model_dir = write_random_model(str(tmp_path / "m"), cfg, case)
+    pcfg, W = plain.load_model_dir(model_dir)
+    want = [plain.generate(pcfg, W, p, new) for p in prompts]
+    llm = LLM(model_dir, EngineOptions(dtype="float32", page_size=page, max_seqs=seats, max_seq_len=longest,
+                                       cache_tokens=tight),
+              ServeOptions(chunk_size=int(rng.choice([8, 24])), max_batch_tokens=int(rng.choice([32, 64])),
+                           ignore_eos=True))
+    got, reasons = llm.generate(prompts, max_new_tokens=new, return_reasons=True)
+    assert reasons == ["length"] * len(prompts)
+    assert got == want
+    llm.engine.cache.check()
+    assert llm.engine.cache.free_seats == seats
+
+
+@pytest.mark.parametrize("case", range(8, 16))
+def test_sampled_output_does_not_depend_on_room_portions_or_running_ahead(case, tmp_path, gpu):
+    rng, cfg, page, prompts, new, seats, longest, tight = workload(case)
+    model_dir = write_random_model(str(tmp_path / "m"), cfg, case)
+    temperature, penalty = float(rng.choice([0.7, 1.3])), float(rng.choice([1.0, 1.15]))
+    runs = []
+    for pool, chunk, budget, ahead, n_seats in ((seats * longest + 64, None, 256, True, seats),
+                                                (tight, 8, 32, True, seats), (tight, 24, 64, False, 2)):
+        llm = LLM(model_dir, EngineOptions(dtype="float32", page_size=page, max_seqs=n_seats, max_seq_len=longest,
+                                           cache_tokens=pool),
+                  ServeOptions(chunk_size=chunk, max_batch_tokens=budget, temperature=temperature,
+                               sampling_seed=case, repetition_penalty=penalty, run_ahead=ahead))
+        runs.append(llm.generate(prompts, max_new_tokens=new, return_reasons=True))
+        llm.engine.cache.check()
+    assert runs[1] == runs[0] and runs[2] == runs[0]
