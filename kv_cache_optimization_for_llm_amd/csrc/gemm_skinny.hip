@@ -390,12 +390,8 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
             for (int t = 0; t < NTW; ++t) w[t].u4 = load_streamed_u4(wp[t] + (size_t)k * 16);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-                // lanes whose row of X does not exist load nothing (their columns of the product
-                // are never stored): with 8 rows that halves what the loads of X bring into the
-                // compute unit, with one row it leaves a sixteenth
                 GFrag8 x;
-                x.u4 = make_uint4(0, 0, 0, 0);
-                if (mt * 16 + r < a.M) x.u4 = *reinterpret_cast<const uint4 *>(xr[mt] + (size_t)k * xstep);
+                x.u4 = *reinterpret_cast<const uint4 *>(xr[mt] + (size_t)k * xstep);
 #pragma unroll
                 for (int t = 0; t < NTW; ++t)
                     acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[t].v, x.v, acc[t][mt], 0, 0, 0);
