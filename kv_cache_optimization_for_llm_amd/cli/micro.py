@@ -3,6 +3,7 @@
     python -m kv_cache_optimization_for_llm_amd.cli.micro attention --tokens 8192 --kernel lds
     python -m kv_cache_optimization_for_llm_amd.cli.micro attention --batch 8 --context 8192 --splits 32
     python -m kv_cache_optimization_for_llm_amd.cli.micro gemm --rows 8 --shape gate_up
+    python -m kv_cache_optimization_for_llm_amd.cli.micro prompt --tokens 8192 --portion 512
 
 The reference keeps a harness that runs its attention kernels alone over made-up caches
 (``micro/harness.cuh``); this is the same idea for the kernels here.  Sizes default to the
@@ -125,6 +126,38 @@ def gemm(args) -> None:
     print(line, flush=True)
 
 
+def prompt(args) -> None:
+    """One prompt through the whole engine (Llama-3.2-1B sizes, random weights) in portions of
+    ``--portion`` tokens, one portion per step: the time of the fastest of ``--reps`` passes."""
+    import torch
+    from ..engine.batch import StepEntry
+    from ..engine.engine import Engine, EngineOptions
+    from .sweep import SHAPES
+
+    cfg = dict(SHAPES["1b"])
+    cfg["max_position_embeddings"] = max(8192, args.tokens)
+    if args.layers:
+        cfg["num_hidden_layers"] = args.layers
+    eng = Engine(None, EngineOptions(dtype="bfloat16", cache_tokens=args.tokens + 64, max_seqs=2,
+                                     max_seq_len=cfg["max_position_embeddings"], use_graphs=not args.no_graphs),
+                 config_dict=cfg, random_seed=0)
+    gen = torch.Generator().manual_seed(0)
+    tokens = [int(t) for t in torch.randint(0, eng.vocab_size, (args.tokens,), generator=gen)]
+    best = float("inf")
+    for _ in range(args.reps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(0, args.tokens, args.portion):
+            part = tokens[i:i + args.portion]
+            eng.step([StepEntry("p", part, [len(part) - 1] if i + args.portion >= args.tokens else [])])
+        torch.cuda.synchronize()
+        best = min(best, time.perf_counter() - t0)
+        eng.release("p")
+    steps = (args.tokens + args.portion - 1) // args.portion
+    print(f"prompt of {args.tokens} in portions of {args.portion} ({steps} steps): {best * 1e3:8.2f} ms  "
+          f"{args.tokens / best:9.0f} tok/s", flush=True)
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description="one kernel in a loop")
     sub = ap.add_subparsers(dest="what", required=True)
@@ -146,7 +179,16 @@ def main(argv=None) -> int:
     g.add_argument("--rows", type=int, default=8)
     g.add_argument("--vendor", action="store_true", help="also time the vendor GEMM on the plain weight")
     g.add_argument("--reps", type=int, default=48)
+    pr = sub.add_parser("prompt")
+    pr.add_argument("--tokens", type=int, default=8192)
+    pr.add_argument("--portion", type=int, default=512)
+    pr.add_argument("--layers", type=int, default=0, help="fewer layers than the 16 of the shape")
+    pr.add_argument("--reps", type=int, default=4)
+    pr.add_argument("--no-graphs", action="store_true")
     args = ap.parse_args(argv)
+    if args.what == "prompt":
+        prompt(args)
+        return 0
     if args.what == "attention":
         if args.kernel == "lds" and not args.tokens:
             ap.error("the workgroup kernel is for prompts: give --tokens")
