@@ -92,9 +92,12 @@ class _DecodeSlot:
 
 
 class DecodeGraphs:
+    MAX_SHAPES = 256           # captured (entries, context bucket) shapes kept (least recently used goes first) ...
+    MAX_KEPT_ROWS = 8192       # ... and the rows of all of them: a graph keeps its logits [entries, vocabulary]
+
     def __init__(self, model, cache, device, feedback=None):
         self.model, self.cache, self.device, self.feedback = model, cache, device, feedback
-        self.slots: Dict[Tuple[int, int], _DecodeSlot] = {}
+        self.slots: "OrderedDict[Tuple[int, int], _DecodeSlot]" = OrderedDict()
         self.replays = 0
         self.captures = 0
 
@@ -106,7 +109,12 @@ class DecodeGraphs:
         key = (n, bucket)
         slot = self.slots.get(key)
         if slot is None:
+            while self.slots and (len(self.slots) >= self.MAX_SHAPES or
+                                  sum(s.n for s in self.slots.values()) + n > self.MAX_KEPT_ROWS):
+                self.slots.popitem(last=False)
             slot = self.slots[key] = _DecodeSlot(n, bucket, len(self.cache.groups), self.device, self.feedback)
+        else:
+            self.slots.move_to_end(key)
         slot.fill(tokens, positions, seats, slot_maps)
         if not slot.warm:
             # first step of this shape runs eagerly: it warms up lazy initialisation (GEMM

@@ -307,6 +307,37 @@ def test_portion_graph_replays_equal_eager_steps(gpu, monkeypatch):
         (a.portion_graphs.captures, a.portion_graphs.replays, n_steps)
 
 
+def test_graphs_kept_are_bounded_and_a_dropped_shape_is_captured_again(model_dirs, gpu):
+    """Only so many captured shapes are kept (the least recently used goes first); a shape that
+    was dropped and comes back is captured again, and every step still equals the eager step."""
+    name = "D"
+    opts = dict(dtype="bfloat16", max_seqs=6, max_seq_len=256, cache_tokens=1536)
+    a = Engine(model_dirs[name], EngineOptions(use_graphs=True, **opts))
+    b = Engine(model_dirs[name], EngineOptions(use_graphs=False, **opts))
+    a.graphs.MAX_SHAPES, a.portion_graphs.MAX_SHAPES = 2, 1
+    rng = np.random.default_rng(2)
+    v = TINY[name][0]["vocab_size"]
+    toks = lambda n: [int(t) for t in rng.integers(0, v, n)]
+    for eng_step in (lambda st: (a.step(st), b.step(st)),):
+        for r in "pqrs":
+            eng_step([StepEntry(r, toks(20), [])])
+        for i in range(48):
+            live = "pqrs"[:1 + (i // 4) % 4]            # batch sizes 1, 2, 3, 4, four steps each, then again
+            la, lb = eng_step([StepEntry(r, toks(1), [0]) for r in live])
+            torch.cuda.synchronize()
+            assert (la - lb).abs().max() <= 4e-3 * lb.abs().max(), f"decode step {i}"
+            if i % 3 == 0:                              # two portion shapes, a few steps each, then again
+                n = 24 if (i // 6) % 2 == 0 else 40
+                for r in ("x", "y"):
+                    la, lb = eng_step([StepEntry(r + str(i), toks(n), [n - 1])])
+                    torch.cuda.synchronize()
+                    assert (la - lb).abs().max() <= 4e-3 * lb.abs().max(), f"portion step {i}"
+                    a.release(r + str(i)), b.release(r + str(i))
+    assert len(a.graphs.slots) <= 2 and len(a.portion_graphs.slots) <= 1
+    assert a.graphs.captures > 4 and a.portion_graphs.captures > 2        # shapes came back after being dropped
+    a.cache.check(), b.cache.check()
+
+
 @pytest.mark.parametrize("run_ahead", [False, True])
 def test_serving_with_small_portions_replays_portion_graphs(run_ahead, model_dirs, gpu):
     """A small token budget and portions of 24 tokens: the same step shapes (a portion alone,
