@@ -307,6 +307,48 @@ def test_portion_graph_replays_equal_eager_steps(gpu, monkeypatch):
         (a.portion_graphs.captures, a.portion_graphs.replays, n_steps)
 
 
+def test_a_long_prompt_in_portions_takes_the_split_kernels_and_matches_plain(tmp_path, gpu, monkeypatch):
+    """A 4,352-token prompt in portions of 1,024, then 256: late portions are few workgroups that
+    each walk thousands of keys, so the workgroup attention kernel cuts their keys into ranges
+    (and the 256-token portion takes the one-wavefront kernel with two row tiles and key splits);
+    with the policy's own thresholds, against the plain model."""
+    from kv_cache_optimization_for_llm_amd.ops import kernels as K
+    from kv_cache_optimization_for_llm_amd.weights.random_init import write_random_model
+    cfg = dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=997, hidden_size=1024,
+               intermediate_size=1408, num_hidden_layers=2, num_attention_heads=16, num_key_value_heads=4,
+               head_dim=64, rms_norm_eps=1e-5, rope_theta=500000.0, max_position_embeddings=8192,
+               rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                 original_max_position_embeddings=2048),
+               tie_word_embeddings=True, hidden_act="silu", torch_dtype="bfloat16")
+    model_dir = write_random_model(str(tmp_path / "m"), cfg, 77)
+    pcfg, W = plain.load_model_dir(model_dir)
+    rng = np.random.default_rng(12)
+    prompt = [int(t) for t in rng.integers(0, 997, 4352)]
+    ref = plain.logits_all(pcfg, W, prompt).numpy()
+    seen = {"lds_splits": 0, "wave_splits": 0}
+    real_lds, real_mfma = K.attention_lds, K.attention_mfma
+
+    def lds(*a, **kw):
+        seen["lds_splits"] += 1 if a[13] > 1 else 0
+        return real_lds(*a, **kw)
+
+    def mfma(*a, **kw):
+        seen["wave_splits"] += 1 if (a[16] > 1 and a[18] == 2) else 0
+        return real_mfma(*a, **kw)
+    monkeypatch.setattr(K, "attention_lds", lds)
+    monkeypatch.setattr(K, "attention_mfma", mfma)
+    eng = Engine(model_dir, EngineOptions(dtype="bfloat16", max_seqs=2, max_seq_len=4608, cache_tokens=4608))
+    at, scale = 0, float(np.abs(ref).max())
+    for n in (1024, 1024, 1024, 1024, 256):
+        want = list(range(0, n, 97)) + [n - 1]
+        out = eng.step([StepEntry("p", prompt[at:at + n], want)]).float().cpu().numpy()
+        err = float(np.abs(out - ref[[at + i for i in want]]).max()) / scale
+        assert err <= TOL["bfloat16"], f"portion at {at}: {err:.3g}"
+        at += n
+    assert seen["lds_splits"] >= 2 * cfg["num_hidden_layers"] and seen["wave_splits"] >= cfg["num_hidden_layers"], seen
+    eng.cache.check()
+
+
 def test_graphs_kept_are_bounded_and_a_dropped_shape_is_captured_again(model_dirs, gpu):
     """Only so many captured shapes are kept (the least recently used goes first); a shape that
     was dropped and comes back is captured again, and every step still equals the eager step."""
