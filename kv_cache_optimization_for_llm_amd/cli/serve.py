@@ -101,9 +101,10 @@ def main(argv=None) -> int:
     ap.add_argument("--cache-tokens", type=int, default=None)
     ap.add_argument("--max-batch-tokens", type=int, default=3072)
     ap.add_argument("--chunk-size", type=int, default=None)
-    ap.add_argument("--gemm-tune-rows", default="",
+    ap.add_argument("--gemm-tune-rows", default="auto",
                     help="comma list of row counts (tokens per step) for which the vendor GEMM library's "
-                         "algorithms are timed at start-up, e.g. the portion size and large decode batches")
+                         "algorithms are timed at start-up (a few seconds); smaller row counts down to half "
+                         "share what is found.  'auto': the number of seats when above 16; '' for none")
     args = ap.parse_args(argv)
     if not args.model_dir:
         print("no model folder: pass it as the first argument or set MODEL_DIR", file=sys.stderr)
@@ -133,7 +134,8 @@ def main(argv=None) -> int:
     engine = Engine(args.model_dir, EngineOptions(
         dtype=args.dtype, cache_mode=args.cache_mode, page_size=args.page_size, max_seqs=args.max_seqs,
         max_seq_len=args.max_seq_len, cache_tokens=args.cache_tokens,
-        gemm_tune_rows=[int(r) for r in args.gemm_tune_rows.split(",") if r.strip()]))
+        gemm_tune_rows=([args.max_seqs] if args.max_seqs > 16 else []) if args.gemm_tune_rows == "auto"
+        else [int(r) for r in args.gemm_tune_rows.split(",") if r.strip()]))
     runner = Runner(engine, ServeOptions(
         temperature=temperature, sampling_seed=seed, ignore_eos=ignore_eos, repetition_penalty=penalty,
         max_batch_tokens=args.max_batch_tokens, chunk_size=args.chunk_size, reserve_policy=policy))

@@ -61,6 +61,23 @@ std::mutex g_mutex;
 hipblasLtHandle_t g_handle[kMaxDevices];
 void *g_workspace[kMaxDevices];
 std::unordered_map<Key, Plan, KeyHash> g_plans;
+// Algorithms that timing has kept, per (device, N, K, result type) with the row count they were
+// timed at.  A row count that has not been timed itself takes the algorithm of the nearest timed
+// one above it (at most twice as many rows) when the library says it supports the exact shape:
+// decode batches of 33..64 requests then share what was found for 64.
+struct TunedKey {
+    int dev, n, k, f32;
+    bool operator==(const TunedKey &o) const { return dev == o.dev && n == o.n && k == o.k && f32 == o.f32; }
+};
+struct TunedHash {
+    size_t operator()(const TunedKey &x) const {
+        size_t h = 1469598103934665603ull;
+        for (int v : {x.dev, x.n, x.k, x.f32}) h = (h ^ (size_t)(unsigned)v) * 1099511628211ull;
+        return h;
+    }
+};
+std::unordered_map<TunedKey, std::vector<std::pair<int, hipblasLtMatmulAlgo_t>>, TunedHash> g_tuned;
+
 // every algorithm of the library for bf16 x bf16 -> bf16 [0] / fp32 [1], asked for once per device
 std::vector<hipblasLtMatmulHeuristicResult_t> g_all_algos[kMaxDevices][2];
 
@@ -91,6 +108,29 @@ bool make_plan(int dev, const Key &key, Plan &p) {
     ok = ok && hipblasLtMatrixLayoutCreate(&p.a, HIP_R_16BF, key.k, key.n, key.k) == HIPBLAS_STATUS_SUCCESS;
     ok = ok && hipblasLtMatrixLayoutCreate(&p.b, HIP_R_16BF, key.k, key.m, key.ldx) == HIPBLAS_STATUS_SUCCESS;
     ok = ok && hipblasLtMatrixLayoutCreate(&p.c, out_type, key.n, key.m, key.ldy) == HIPBLAS_STATUS_SUCCESS;
+    if (ok) {
+        auto it = g_tuned.find(TunedKey{dev, key.n, key.k, key.f32});
+        if (it != g_tuned.end()) {
+            int best_rows = 0;
+            const hipblasLtMatmulAlgo_t *best = nullptr;
+            for (const auto &entry : it->second)
+                if (entry.first >= key.m && entry.first <= 2 * key.m && (best == nullptr || entry.first < best_rows)) {
+                    best_rows = entry.first;
+                    best = &entry.second;
+                }
+            if (best != nullptr) {
+                const float alpha = 1.f, beta = 0.f;
+                size_t need = 0;
+                hipblasLtMatmulAlgo_t algo = *best;
+                if (hipblaslt_ext::matmulIsAlgoSupported(g_handle[dev], p.desc, &alpha, p.a, p.b, &beta, p.c, p.c, algo,
+                                                         need) == HIPBLAS_STATUS_SUCCESS && need <= kWorkspaceBytes) {
+                    p.algo = algo;
+                    p.found = true;
+                    return true;
+                }
+            }
+        }
+    }
     hipblasLtMatmulPreference_t pref = nullptr;
     ok = ok && hipblasLtMatmulPreferenceCreate(&pref) == HIPBLAS_STATUS_SUCCESS;
     if (ok) {
@@ -211,6 +251,16 @@ extern "C" int kva_gemm_vendor_tune(void *Y, const void *X, const void *const *W
     }
     (void)hipEventDestroy(t0);
     (void)hipEventDestroy(t1);
+    if (p.found) {
+        auto &list = g_tuned[TunedKey{dev, N, K, key.f32}];
+        bool replaced = false;
+        for (auto &entry : list)
+            if (entry.first == M) {
+                entry.second = p.algo;
+                replaced = true;
+            }
+        if (!replaced) list.emplace_back(M, p.algo);
+    }
     if (first_us) *first_us = first;
     if (best_us) *best_us = best;
     if (tried) *tried = (int)timed.size();
@@ -222,6 +272,13 @@ extern "C" int kva_gemm_vendor_forget(int M, int N, int K, int ldx, int ldy, int
     int dev = 0;
     KVA_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDevices, "gemm_vendor_forget: no current device");
     std::lock_guard<std::mutex> lock(g_mutex);
+    auto tuned = g_tuned.find(TunedKey{dev, N, K, out_f32 ? 1 : 0});
+    if (tuned != g_tuned.end()) {
+        auto &list = tuned->second;
+        list.erase(std::remove_if(list.begin(), list.end(),
+                                  [M](const std::pair<int, hipblasLtMatmulAlgo_t> &e) { return e.first == M; }),
+                   list.end());
+    }
     auto it = g_plans.find(Key{dev, M, N, K, ldx, ldy, out_f32 ? 1 : 0});
     if (it != g_plans.end()) {
         Plan &p = it->second;

@@ -47,7 +47,8 @@ class EngineOptions:
                                         # shape comes back, as HIP graphs (bfloat16 engine)
     # Row counts (tokens per step) for which the vendor GEMM library's algorithms are timed at
     # start-up and the fastest kept, e.g. the prompt portion size and large decode batches
-    # (bfloat16 engine; a few seconds per row count and matrix shape).  Empty: the library's own choice.
+    # (bfloat16 engine; a few seconds per row count and matrix shape; row counts down to half of a
+    # timed one share what was found for it).  Empty: the library's own choice.
     gemm_tune_rows: Sequence[int] = ()
     device: str = "cuda:0"
 

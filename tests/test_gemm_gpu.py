@@ -271,5 +271,11 @@ def test_vendor_product_keeps_the_fastest_algorithm_and_the_same_result(gpu):
     want = x.double().cpu() @ ws[1].double().cpu().t()
     for got in (before, out):
         assert (got.double().cpu() - want).abs().max() / want.abs().max() <= 2 ** -8
+    # a row count that was not timed itself takes the algorithm of the timed one above it
+    x40 = rnd(40, k, seed=10).to(gpu)
+    out40 = torch.empty((40, n), dtype=torch.bfloat16, device=gpu)
+    assert K.gemm_vendor(x40, ws[2], out40)
+    want40 = x40.double().cpu() @ ws[2].double().cpu().t()
+    assert (out40.double().cpu() - want40).abs().max() / want40.abs().max() <= 2 ** -8
     with pytest.raises(K.KernelError):
         K.gemm_vendor_tune(m, [ws[0], rnd(n, k + 32, seed=1).to(gpu)])
