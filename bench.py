@@ -88,8 +88,8 @@ def main():
     # room for max_batch requests at the context, one more page each for the tokens decoded
     pool = max_batch * (ctx + 2 * PAGE)
     # the vendor library's algorithms are timed once, at start-up, for the row counts whose
-    # products go to it here: the prefill's 2,048 tokens and decode batches above 32
-    tune_rows = [] if args.no_gemm_tuning else [PREFILL_TOKENS] + [b for b in {args.batch, max_batch} if b > 32]
+    # products go to it here: the prefill's 2,048 tokens and decode batches above 16
+    tune_rows = [] if args.no_gemm_tuning else [PREFILL_TOKENS] + [b for b in {args.batch, max_batch} if b > 16]
     engine = Engine(None, EngineOptions(dtype="bfloat16", page_size=PAGE, cache_tokens=pool,
                                         max_seqs=max_batch, max_seq_len=cfg["max_position_embeddings"],
                                         gemm_tune_rows=tune_rows),
