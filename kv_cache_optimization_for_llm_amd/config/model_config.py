@@ -113,6 +113,9 @@ class LlamaConfig:
                 f"num_key_value_heads {kv_heads}")
         if not isinstance(head_dim, int) or head_dim <= 0 or head_dim % 2 != 0:
             raise ConfigError(f"config.json: head_dim {head_dim} must be a positive even integer")
+        if head_dim % 4 != 0:
+            raise ConfigError(f"config.json: head_dim {head_dim} is not supported: the attention kernels "
+                              f"take head sizes that are multiples of 4 (multiples of 16 run on the matrix cores)")
         act = d.get("hidden_act", "silu")
         if act != "silu":
             raise ConfigError(f"config.json: hidden_act {act!r} is not supported (only 'silu')")

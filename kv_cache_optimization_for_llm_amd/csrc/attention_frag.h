@@ -29,6 +29,10 @@ __device__ inline b16x2 pack_bf16(float a, float b) {
     return __builtin_convertvector(f32x2{a, b}, b16x2);
 }
 
+// Most key splits the attention kernels and their merge take (the merge keeps one weight per
+// split in LDS).  The host's split policy asks kva_attention_max_splits() for it.
+#define MERGE_MAX_SPLITS 256
+
 // attention_mfma.hip: merge of key-split partials (see there)
 int kva_attention_merge_launch(void *out, const float *part_o, const float *part_ml, int head_dim, int splits,
                                const int *item_meta, const int *item_entry, const int *item_row0,

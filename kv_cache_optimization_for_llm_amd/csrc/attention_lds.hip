@@ -386,7 +386,8 @@ extern "C" int kva_attention_lds(void *out, float *part_o, float *part_ml, const
                                  int num_kv_heads, int head_dim, int page_size, float scale, int window,
                                  int splits, int keys_per_split, int total_rows, int all_rows,
                                  hipStream_t stream) {
-    KVA_REQUIRE(splits >= 1 && splits <= 256 && num_kv_heads <= 65535, "attention_lds: 1..256 splits");
+    KVA_REQUIRE(splits >= 1 && splits <= MERGE_MAX_SPLITS && num_kv_heads <= 65535,
+                "attention_lds: 1..%d splits and at most 65535 kv heads", MERGE_MAX_SPLITS);
     KVA_REQUIRE(splits == 1 || (keys_per_split > 0 && keys_per_split % 32 == 0 && part_o && part_ml),
                 "attention_lds: splits need a key count that is a multiple of 32 and a workspace");
     KVA_REQUIRE(num_items >= 0 && num_q_heads > 0 && num_kv_heads > 0 && max_blocks > 0, "attention_lds: bad sizes");

@@ -389,7 +389,6 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
 // weights go to LDS), then own value dimensions and add the weighted partials.  The partials of
 // the first MERGE_EARLY splits are loaded before the weights are known, so that the kernel makes
 // one trip to memory, not two.
-#define MERGE_MAX_SPLITS 256
 #define MERGE_EARLY 32
 __global__ void __launch_bounds__(KVA_WAVE)
 attention_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o,
@@ -480,6 +479,8 @@ int kva_attention_merge_launch(void *out, const float *part_o, const float *part
     KVA_CHECK_LAUNCH("attention_merge");
     return KVA_OK;
 }
+
+extern "C" int kva_attention_max_splits() { return MERGE_MAX_SPLITS; }
 
 extern "C" int kva_attention_mfma_supported(int head_dim, int page_size) {
     switch (head_dim) {

@@ -1,18 +1,24 @@
 // Host-side allocators of the cache manager, behind a C ABI (loaded with ctypes).
 //
 //  * PagePool  - fixed-size pages with a LIFO free stack and per-page reference counts: the
-//    paged mode.  Mirrors what the reference keeps in its KVCacheState
+//    paged mode.  Keeps what the reference keeps in its KVCacheState
 //    (paged_attention/src/engine.cuh:135-178; take/share/drop paged_attention/src/engine.cu:376-404;
 //    the accounting invariant :456-475): a page is on the free stack xor has refcount > 0.
-//  * Buddy     - binary buddy allocator over a pool of units: the contiguous (Orca-style) mode.
-//    Same scheme as base/src/engine.cu:169-254: the pool is viewed as a tree over the next power
-//    of two; parts past the real end are never free; frees merge buddies upward.  It also counts
-//    the failures where enough units were free in total but no aligned run existed
-//    (base/src/engine.cu:336-346).
+//  * Buddy     - binary buddy allocation of power-of-two, self-aligned runs of units: the
+//    contiguous (Orca-style) mode, with the behaviour of base/src/engine.cu:169-254 (a pool that
+//    is no power of two never hands out its missing end; freed buddies merge; failures where
+//    enough units were free in total but no aligned run existed are counted, :336-346).  The
+//    structure is another one: not lists of free runs per order that are searched, but one array
+//    over the implicit binary tree of all possible runs, holding for every node the largest
+//    order of a wholly free run inside it.  Allocation walks down from the root (always into
+//    the tighter fit, so large runs stay whole), freeing finds its node by arithmetic, both fix
+//    the path to the root: O(log pool) each, and a run that is not allocated (a double free) is
+//    seen from one flag, not by comparing against every free run.
 //
 // No GPU code here: this library builds with a plain C++ compiler.
 #include <algorithm>
 #include <cstdint>
+#include <utility>
 #include <vector>
 
 namespace {
@@ -25,32 +31,44 @@ struct PagePool {
     std::vector<uint8_t> ever_used;
 };
 
+// Ceiling of log2(n) for n >= 1.
+int order_for(int n) { return n <= 1 ? 0 : 32 - __builtin_clz((unsigned)(n - 1)); }
+
 struct Buddy {
+    static constexpr int8_t NONE = -1;
     int pool_units = 0;
-    int max_order = 0;
-    std::vector<std::vector<int>> free_lists;
+    int max_order = 0;      // the tree spans 1 << max_order units; those past pool_units never exist
+    // Heap numbering: node 1 is the whole span; node i has children 2i and 2i + 1; the node of the
+    // run (start, order) is (1 << (max_order - order)) + (start >> order).
+    std::vector<int8_t> best;    // largest order of a wholly free run inside the node, or NONE
+    std::vector<uint8_t> taken;  // 1: the node is handed out as one run
     int free_units = 0;
     int reserved_units = 0;
     long long fragmentation_failures = 0;
-};
 
-int ceil_log2(int n) {
-    int order = 0;
-    while ((1LL << order) < n) ++order;
-    return order;
-}
+    int node_of(int start, int order) const { return (1 << (max_order - order)) + (start >> order); }
 
-void buddy_init_range(Buddy &b, int start, int order) {
-    if (start >= b.pool_units) return;
-    const int size = 1 << order;
-    if (start + size <= b.pool_units) {
-        b.free_lists[order].push_back(start);
-        return;
+    // What a node of `order` holds, given its children: the whole run if both halves are whole.
+    int8_t joined(int node, int order) const {
+        const int8_t l = best[2 * node], r = best[2 * node + 1];
+        return (l == order - 1 && r == order - 1) ? (int8_t)order : std::max(l, r);
     }
-    if (order == 0) return;
-    buddy_init_range(b, start, order - 1);
-    buddy_init_range(b, start + size / 2, order - 1);
-}
+
+    void fix_upwards(int node, int order) {
+        for (node >>= 1, ++order; node >= 1; node >>= 1, ++order) best[node] = joined(node, order);
+    }
+
+    void build() {
+        const int span = 1 << max_order;
+        best.assign(2 * (size_t)span, NONE);
+        taken.assign(2 * (size_t)span, 0);
+        for (int u = 0; u < pool_units; ++u) best[span + u] = 0;
+        for (int order = 1; order <= max_order; ++order) {
+            const int first = 1 << (max_order - order);
+            for (int node = first; node < 2 * first; ++node) best[node] = joined(node, order);
+        }
+    }
+};
 
 } // namespace
 
@@ -140,12 +158,11 @@ int kva_pool_accounting_holds(void *h) {
 
 // ------------------------------------------------------------------ buddy allocator
 void *kva_buddy_create(int pool_units) {
-    if (pool_units <= 0) return nullptr;
+    if (pool_units <= 0 || pool_units > (1 << 29)) return nullptr;
     Buddy *b = new Buddy();
     b->pool_units = pool_units;
-    b->max_order = ceil_log2(pool_units);
-    b->free_lists.assign(b->max_order + 1, {});
-    buddy_init_range(*b, 0, b->max_order);
+    b->max_order = order_for(pool_units);
+    b->build();
     b->free_units = pool_units;
     return b;
 }
@@ -153,54 +170,48 @@ void *kva_buddy_create(int pool_units) {
 void kva_buddy_destroy(void *h) { delete static_cast<Buddy *>(h); }
 
 // Size a request of `units` really takes: the next power of two.
-int kva_buddy_round(int units) { return units <= 0 ? 0 : 1 << ceil_log2(units); }
+int kva_buddy_round(int units) { return units <= 0 ? 0 : 1 << order_for(units); }
 
 // Start of a self-aligned run of round(units) units, or -1.
 int kva_buddy_alloc(void *h, int units) {
     Buddy *b = static_cast<Buddy *>(h);
     if (units <= 0) return -1;
-    const int want = ceil_log2(units);
-    const int size = 1 << want;
-    int k = want;
-    while (k <= b->max_order && b->free_lists[k].empty()) ++k;
-    if (k > b->max_order) {
-        if (b->free_units >= size) ++b->fragmentation_failures;
+    const int want = order_for(units);
+    if (want > b->max_order || b->best[1] < want) {
+        if (want <= 30 && b->free_units >= (1 << want)) ++b->fragmentation_failures;
         return -1;
     }
-    const int start = b->free_lists[k].back();
-    b->free_lists[k].pop_back();
-    while (k > want) {
-        --k;
-        b->free_lists[k].push_back(start + (1 << k));
+    int node = 1;
+    for (int order = b->max_order; order > want; --order) {
+        const int8_t l = b->best[2 * node], r = b->best[2 * node + 1];
+        // into the half that fits more tightly; the lower addresses on a tie
+        const bool left = l >= want && (r < want || l <= r);
+        node = 2 * node + (left ? 0 : 1);
     }
-    b->free_units -= size;
-    b->reserved_units += size;
-    return start;
+    b->taken[node] = 1;
+    b->best[node] = Buddy::NONE;
+    b->fix_upwards(node, want);
+    b->free_units -= 1 << want;
+    b->reserved_units += 1 << want;
+    return (node - (1 << (b->max_order - want))) << want;
 }
 
-// Gives back the run that kva_buddy_alloc(units) returned at `start`.  0 ok, -1 on a bad run.
+// Gives back the run that kva_buddy_alloc(units) returned at `start`.  0 ok, -1 if that is not an
+// allocated run (never handed out, or given back already).
 int kva_buddy_free(void *h, int start, int units) {
     Buddy *b = static_cast<Buddy *>(h);
     if (units <= 0 || start < 0) return -1;
-    int order = ceil_log2(units);
+    const int order = order_for(units);
+    if (order > b->max_order) return -1;
     const int size = 1 << order;
     if (start % size != 0 || start + size > b->pool_units) return -1;
-    // refuse a run that overlaps anything free (a double free)
-    for (int o = 0; o <= b->max_order; ++o)
-        for (int s : b->free_lists[o])
-            if (s < start + size && start < s + (1 << o)) return -1;
+    const int node = b->node_of(start, order);
+    if (!b->taken[node]) return -1;
+    b->taken[node] = 0;
+    b->best[node] = (int8_t)order;     // everything below it has stayed as it was: wholly free
+    b->fix_upwards(node, order);
     b->free_units += size;
     b->reserved_units -= size;
-    while (order < b->max_order) {
-        const int buddy = start ^ (1 << order);
-        std::vector<int> &list = b->free_lists[order];
-        auto it = std::find(list.begin(), list.end(), buddy);
-        if (it == list.end()) break;
-        list.erase(it);
-        start = std::min(start, buddy);
-        ++order;
-    }
-    b->free_lists[order].push_back(start);
     return 0;
 }
 
@@ -211,19 +222,28 @@ long long kva_buddy_fragmentation_failures(void *h) {
     return static_cast<Buddy *>(h)->fragmentation_failures;
 }
 
-// Writes the free runs as (start, order) pairs, sorted; returns how many there are (even if
-// that is more than `cap`).
+// Writes the free runs as (start, order) pairs in address order, each as large as it can be
+// (two free buddies are one run); returns how many there are (even if more than `cap`).
 int kva_buddy_free_runs(void *h, int *out, int cap) {
     Buddy *b = static_cast<Buddy *>(h);
-    std::vector<std::pair<int, int>> runs;
-    for (int o = 0; o <= b->max_order; ++o)
-        for (int s : b->free_lists[o]) runs.push_back({s, o});
-    std::sort(runs.begin(), runs.end());
-    for (int i = 0; i < (int)runs.size() && i < cap; ++i) {
-        out[2 * i] = runs[i].first;
-        out[2 * i + 1] = runs[i].second;
+    int count = 0;
+    std::vector<std::pair<int, int>> todo{{1, b->max_order}};     // (node, order), a stack: left halves first
+    while (!todo.empty()) {
+        const auto [node, order] = todo.back();
+        todo.pop_back();
+        if (b->best[node] == Buddy::NONE) continue;
+        if (b->best[node] == order) {
+            if (count < cap) {
+                out[2 * count] = (node - (1 << (b->max_order - order))) << order;
+                out[2 * count + 1] = order;
+            }
+            ++count;
+            continue;
+        }
+        todo.push_back({2 * node + 1, order - 1});
+        todo.push_back({2 * node, order - 1});
     }
-    return (int)runs.size();
+    return count;
 }
 
 } // extern "C"

@@ -40,9 +40,15 @@ class EngineOptions:
     dtype: str = "bfloat16"             # "bfloat16": serving kernels; "float32": true 32-bit everywhere
     cache_mode: str = "paged"           # "paged" | "contiguous"
     page_size: int = 16                 # tokens per page (reference: BLOCK_SIZE, paged config.h:181)
-    cache_tokens: Optional[int] = None  # pool size in tokens (default: max_seqs * max_seq_len)
+    # Pool size in tokens.  None: what is free on the device after weights, tables and the GEMM
+    # workspace, less ``memory_margin_bytes`` and a step's activations, but never more than every
+    # seat at its longest (reference: the pool is sized last, from leftover memory,
+    # base/src/engine.cu:257-299, paged_attention/src/engine.cu:186-215).
+    cache_tokens: Optional[int] = None
+    memory_margin_bytes: int = 2 << 30  # left free when the pool is sized from leftover memory
     max_seqs: int = 8                   # seats (reference: MAX_SEQUENCES)
     max_seq_len: Optional[int] = None   # longest request (default: max_position_embeddings)
+    max_batch_tokens: int = 8192        # most tokens one step may bring (reference: MAX_BATCH_TOKENS)
     use_graphs: bool = True             # replay decode-only steps, and steps with prompt portions whose
                                         # shape comes back, as HIP graphs (bfloat16 engine)
     # Row counts (tokens per step) for which the vendor GEMM library's algorithms are timed at
@@ -51,6 +57,24 @@ class EngineOptions:
     # timed one share what was found for it).  Empty: the library's own choice.
     gemm_tune_rows: Sequence[int] = ()
     device: str = "cuda:0"
+
+
+def pool_pages_from_memory(free_bytes: int, page_bytes: int, *, page_size: int, max_seqs: int,
+                           max_seq_len: int, margin_bytes: int, step_bytes: int = 0) -> int:
+    """Pages of a cache pool that is sized from leftover device memory: ``free_bytes`` less a
+    margin and a step's activations, in whole pages of ``page_bytes`` (all cache slots of all
+    groups together), but no more than every seat needs at its longest.  The reference sizes
+    its pool this way after everything else is allocated
+    (``paged_attention/src/engine.cu:186-215``: free memory - 128 MiB, in pages)."""
+    if page_bytes <= 0 or page_size <= 0:
+        raise EngineError("page_bytes and page_size must be positive")
+    most = max_seqs * ((max_seq_len + page_size - 1) // page_size)
+    room = (int(free_bytes) - int(margin_bytes) - int(step_bytes)) // page_bytes
+    if room < 1:
+        raise EngineError(
+            f"no room for a cache pool: {free_bytes / 2**30:.2f} GiB free, {margin_bytes / 2**30:.2f} GiB "
+            f"margin, {step_bytes / 2**30:.2f} GiB for a step's activations, {page_bytes} bytes a page")
+    return int(min(most, room))
 
 
 def require_gpu(device: str = "cuda:0") -> torch.device:
@@ -100,9 +124,27 @@ class Engine:
         self.vocab_size = self.spec.vocab_size
         max_seq_len = options.max_seq_len or self.spec.max_positions
         max_seq_len = min(max_seq_len, self.spec.max_positions)
-        cache_tokens = options.cache_tokens or options.max_seqs * max_seq_len
-        num_pages = (cache_tokens + options.page_size - 1) // options.page_size
+        if options.max_batch_tokens < 1:
+            raise EngineError("max_batch_tokens must be at least 1")
+        self.max_batch_tokens = int(options.max_batch_tokens)
         groups, states = self.model.cache_requirements()
+        if options.cache_tokens:
+            num_pages = (options.cache_tokens + options.page_size - 1) // options.page_size
+        else:
+            elem = torch.empty((), dtype=self.dtype).element_size()
+            page_bytes = sum(2 * len(slots) * kv.num_kv_heads * kv.head_dim * options.page_size * elem
+                             for kv, slots in groups)
+            if page_bytes == 0:
+                num_pages = 1           # no mixer keeps keys and values
+            else:
+                torch.cuda.empty_cache()        # what loading left cached is free for the pool as well
+                free_bytes, _ = torch.cuda.mem_get_info(self.device)
+                tables = sum(4 * options.max_seqs * ((max_seq_len + options.page_size - 1) // options.page_size)
+                             for _ in groups)
+                num_pages = pool_pages_from_memory(
+                    free_bytes - tables, page_bytes, page_size=options.page_size, max_seqs=options.max_seqs,
+                    max_seq_len=max_seq_len, margin_bytes=options.memory_margin_bytes,
+                    step_bytes=self.model.step_activation_bytes(self.max_batch_tokens))
         self.cache = CacheManager(groups, states, page_size=options.page_size, num_pages=num_pages,
                                   max_seqs=options.max_seqs, max_seq_len=max_seq_len,
                                   mode=options.cache_mode, device=self.device, dtype=self.dtype)
@@ -145,17 +187,6 @@ class Engine:
 
     def length(self, request_id) -> int:
         return self.cache.length(self._seat_of[request_id])
-
-    def preload_context(self, request_id, num_tokens: int) -> None:
-        """For measurements: the request is taken to hold ``num_tokens`` tokens already; pages are
-        mapped for them and whatever the cache arrays contain there stands for their keys and
-        values.  Nothing is computed."""
-        if request_id not in self._seat_of and self.add_request(request_id) is None:
-            raise CacheExhausted(f"no seat for request {request_id!r}")
-        seat = self._seat_of[request_id]
-        if not self.cache.grow(seat, num_tokens):
-            raise CacheExhausted(f"no pages for {num_tokens} tokens of request {request_id!r}")
-        self.cache.commit(seat, num_tokens)
 
     # ------------------------------------------------------------------ the step
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
@@ -248,6 +279,10 @@ class Engine:
                                       f"{n} tokens")
             toks.append(arr)
             wants.append(e.want if isinstance(e.want, list) else list(e.want))
+        total = sum(len(t) for t in toks)
+        if total > self.max_batch_tokens:
+            raise EngineError(f"a step of {total} tokens is larger than max_batch_tokens "
+                              f"({self.max_batch_tokens}); cut the prompts into smaller portions")
         seat_of, cache = self._seat_of, self.cache
         for e in entries:
             seat = seat_of.get(e.request_id)

@@ -31,8 +31,10 @@ class Runner:
     def __init__(self, engine: Engine, options: Optional[ServeOptions] = None):
         self.engine = engine
         self.options = options = options or ServeOptions()
+        # the engine refuses a step above its own bound, so the scheduler never plans one
         self.scheduler = Scheduler(
-            engine.cache, max_batch_tokens=options.max_batch_tokens, chunk_size=options.chunk_size,
+            engine.cache, max_batch_tokens=min(options.max_batch_tokens, engine.max_batch_tokens),
+            chunk_size=options.chunk_size,
             eos_token_ids=engine.spec.eos_token_ids, ignore_eos=options.ignore_eos,
             reserve_policy=options.reserve_policy)
         self.sampler = Sampler(engine.vocab_size, engine.cache.max_seqs, engine.device,

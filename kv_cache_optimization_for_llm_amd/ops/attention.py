@@ -29,29 +29,33 @@ _LDS_TARGET_GROUPS = 1024
 _LDS_MIN_KEYS_PER_SPLIT = 1024
 
 
-def choose_splits(num_items: int, num_kv_heads: int, max_context: int) -> tuple:
-    """(splits, keys_per_split) for the matrix-core kernel."""
-    waves = max(1, num_items * num_kv_heads)
-    want = max(1, _TARGET_WAVES // waves)
-    most = max(1, (max_context + _MIN_KEYS_PER_SPLIT - 1) // _MIN_KEYS_PER_SPLIT)
-    splits = min(want, most)
-    if splits <= 1:
-        return 1, 0
-    per = (max_context + splits - 1) // splits
-    per = (per + 31) // 32 * 32
-    splits = (max_context + per - 1) // per
-    return (splits, per) if splits > 1 else (1, 0)
-
-
-def choose_lds_splits(groups: int, max_context: int) -> tuple:
-    """(splits, keys_per_split) for the workgroup kernel."""
-    want = max(1, _LDS_TARGET_GROUPS // max(1, groups))
-    splits = min(want, max(1, max_context // _LDS_MIN_KEYS_PER_SPLIT))
+def _cut_keys(want: int, max_context: int, max_splits: int) -> tuple:
+    """``max_context`` keys in at most ``min(want, max_splits)`` ranges of a multiple of 32 keys."""
+    splits = min(want, max_splits)
     if splits <= 1:
         return 1, 0
     per = ((max_context + splits - 1) // splits + 31) // 32 * 32
-    splits = (max_context + per - 1) // per
+    splits = (max_context + per - 1) // per      # rounding up the range never adds a range
     return (splits, per) if splits > 1 else (1, 0)
+
+
+def choose_splits(num_items: int, num_kv_heads: int, max_context: int, max_splits: int = None) -> tuple:
+    """(splits, keys_per_split) for the matrix-core kernel; never more splits than the kernels
+    and their merge take (``max_splits``, by default what the library says)."""
+    if max_splits is None:
+        max_splits = K.attention_max_splits()
+    waves = max(1, num_items * num_kv_heads)
+    want = max(1, _TARGET_WAVES // waves)
+    most = max(1, (max_context + _MIN_KEYS_PER_SPLIT - 1) // _MIN_KEYS_PER_SPLIT)
+    return _cut_keys(min(want, most), max_context, max_splits)
+
+
+def choose_lds_splits(groups: int, max_context: int, max_splits: int = None) -> tuple:
+    """(splits, keys_per_split) for the workgroup kernel, under the same limit."""
+    if max_splits is None:
+        max_splits = K.attention_max_splits()
+    want = max(1, _LDS_TARGET_GROUPS // max(1, groups))
+    return _cut_keys(min(want, max(1, max_context // _LDS_MIN_KEYS_PER_SPLIT)), max_context, max_splits)
 
 
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads: int,

@@ -245,6 +245,17 @@ def mark_tokens(mask: torch.Tensor, seats: torch.Tensor, tokens: torch.Tensor) -
           "mark_tokens")
 
 
+_MAX_SPLITS = None
+
+
+def attention_max_splits() -> int:
+    """Most key splits the matrix-core attention kernels and their merge take."""
+    global _MAX_SPLITS
+    if _MAX_SPLITS is None:
+        _MAX_SPLITS = int(hip_lib().kva_attention_max_splits())
+    return _MAX_SPLITS
+
+
 def attention_mfma_supported(head_dim: int, page_size: int) -> bool:
     return bool(hip_lib().kva_attention_mfma_supported(int(head_dim), int(page_size)))
 

@@ -60,6 +60,10 @@ class GQAAttention(Mixer):
 
     fuses_tail = True
 
+    def activation_elements(self) -> int:
+        # the joined projection, the attention output and the output projection
+        return (2 * self.num_heads + 2 * self.num_kv_heads) * self.head_dim + self.hidden_size
+
     def _project_encode_cache(self, x, batch, kv):
         """Q (position-encoded) for the attention kernel, with K and V of the step's tokens put
         into the cache.  Few rows: one product does all of it in its epilogue; otherwise the

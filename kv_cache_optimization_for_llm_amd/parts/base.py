@@ -139,6 +139,11 @@ class Part:
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         """Takes the tensors named by ``tensor_specs`` (already on the device)."""
 
+    def activation_elements(self) -> int:
+        """Elements of intermediate results this part makes per token of a step (an estimate for
+        sizing memory; 0 when negligible)."""
+        return 0
+
 
 class Norm(Part):
     def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None,

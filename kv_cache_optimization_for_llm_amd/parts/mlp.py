@@ -44,6 +44,10 @@ class SwiGLU(FeedForward):
 
     fuses_tail = True
 
+    def activation_elements(self) -> int:
+        # gate and up, their gated product, the down projection
+        return 3 * self.intermediate_size + self.hidden_size
+
     def forward(self, x, ctx: MixerContext, tail: Optional[BranchTail] = None):
         """``x`` may be NormedRows; with a ``tail`` the down projection adds into the residual
         stream and prepares the next norm when the shapes allow (NormedRows are returned)."""

@@ -34,6 +34,9 @@ class RMSNorm(Norm):
     def prepared_by_product(self):
         return (self.weight, self.width, self.eps)
 
+    def activation_elements(self) -> int:
+        return self.width
+
     def forward(self, x, out=None, delta=None, row_idx=None):
         if out is None:
             rows = x.shape[0] if row_idx is None else row_idx.shape[0]

@@ -49,6 +49,26 @@ def rotary_inv_freq(rot_dim: int, theta: float, scaling: Optional[dict]) -> np.n
     return out.astype(f32)
 
 
+# cos/sin tables shared by every encoding with the same frequencies, length and device: the
+# layers of a model all rotate alike, and a table for 131,072 positions is tens of megabytes
+_TABLES: "dict" = {}
+_TABLES_KEPT = 8
+
+
+def shared_tables(inv_freq: np.ndarray, max_positions: int, device) -> tuple:
+    key = (inv_freq.tobytes(), int(max_positions), str(torch.device(device)))
+    hit = _TABLES.pop(key, None)
+    if hit is None:
+        pos = np.arange(max_positions, dtype=np.float32)[:, None]
+        angle = (pos * inv_freq[None, :]).astype(np.float32)
+        hit = (torch.from_numpy(np.cos(angle).astype(np.float32)).to(device),
+               torch.from_numpy(np.sin(angle).astype(np.float32)).to(device))
+    _TABLES[key] = hit                      # most recently used last
+    while len(_TABLES) > _TABLES_KEPT:
+        _TABLES.pop(next(iter(_TABLES)))
+    return hit
+
+
 @POSITION_ENCODINGS.register("rotary")
 class RotaryEncoding(PositionEncoding):
     graph_safe = True
@@ -67,10 +87,7 @@ class RotaryEncoding(PositionEncoding):
 
     def tables(self, device) -> tuple:
         if self._cos is None or self._cos.device != torch.device(device):
-            pos = np.arange(self.max_positions, dtype=np.float32)[:, None]
-            angle = (pos * self.inv_freq[None, :]).astype(np.float32)
-            self._cos = torch.from_numpy(np.cos(angle).astype(np.float32)).to(device)
-            self._sin = torch.from_numpy(np.sin(angle).astype(np.float32)).to(device)
+            self._cos, self._sin = shared_tables(self.inv_freq, self.max_positions, device)
         return self._cos, self._sin
 
     def rotate_half_tables(self, device, head_dim: int):

@@ -8,7 +8,8 @@ missing tensors, unexpected tensors, wrong shapes, unusable dtypes - is collecte
 
 Dtypes.  A tensor stored in bfloat16 stays bfloat16 on a bfloat16 engine and is widened
 (exactly) on a float32 engine.  A tensor stored in 32-bit float stays 32-bit on either engine.
-Integer tables become int32.
+A tensor stored in float16 is widened to 32-bit (exactly: bfloat16 would drop three of its
+mantissa bits) and from then on is a tensor in 32-bit.  Integer tables become int32.
 """
 from __future__ import annotations
 
@@ -111,9 +112,9 @@ def validate(index: Mapping[str, Tuple[str, dict]], specs: Mapping[str, TensorSp
 def target_dtype(stored: torch.dtype, role: str, engine_dtype: torch.dtype) -> torch.dtype:
     if role == "table":
         return torch.int32
-    if stored == torch.float32:
-        return torch.float32            # a tensor stored in 32-bit stays so
-    return engine_dtype                 # bf16 (or fp16) storage: engine dtype; widening is exact
+    if stored in (torch.float32, torch.float16):
+        return torch.float32            # a tensor stored in 32-bit stays so; float16 only fits into 32-bit exactly
+    return engine_dtype                 # bf16 storage: the engine's dtype (widening to 32-bit is exact)
 
 
 def load_tensors(model_dir: str, specs: Mapping[str, TensorSpec], engine_dtype: torch.dtype,

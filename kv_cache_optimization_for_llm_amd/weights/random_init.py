@@ -1,7 +1,10 @@
 """Random-weights mode: writes a model folder (``config.json`` + ``model.safetensors``) from a
 configuration and a seed.
 
-Matrices are N(0, 0.02), norm weights 1 + U(-0.1, 0.1).  Each tensor's generator is seeded from
+Matrices are N(0, 0.02), norm weights 1 + U(-0.1, 0.1).  With a ``gain`` a matrix ``[out, in]``
+is N(0, gain / sqrt(in)) instead: its products of unit-size inputs are of size ``gain`` at any
+width, so attention scores spread and a tied model's best next token is not its input token -
+what tests of generation need from random weights.  Each tensor's generator is seeded from
 (seed, tensor name), so a tensor's values do not depend on which other tensors exist or on the
 order they are made in.  Values are drawn in fp32 and stored in the configuration's
 ``torch_dtype`` (or the dtype asked for).
@@ -27,12 +30,14 @@ def _generator(seed: int, name: str) -> torch.Generator:
     return g
 
 
-def random_tensor(name: str, spec: TensorSpec, seed: int, dtype: torch.dtype) -> torch.Tensor:
+def random_tensor(name: str, spec: TensorSpec, seed: int, dtype: torch.dtype,
+                  gain: Optional[float] = None) -> torch.Tensor:
     g = _generator(seed, name)
     if spec.role == "table":
         return torch.zeros(spec.shape, dtype=torch.int32)
     if spec.init == "normal":
-        t = torch.randn(spec.shape, generator=g, dtype=torch.float32) * 0.02
+        std = 0.02 if gain is None or len(spec.shape) != 2 else float(gain) / float(spec.shape[1]) ** 0.5
+        t = torch.randn(spec.shape, generator=g, dtype=torch.float32) * std
     elif spec.init == "norm":
         t = 1.0 + (torch.rand(spec.shape, generator=g, dtype=torch.float32) * 0.2 - 0.1)
     elif spec.init == "zeros":
@@ -42,8 +47,9 @@ def random_tensor(name: str, spec: TensorSpec, seed: int, dtype: torch.dtype) ->
     return t.to(dtype)
 
 
-def random_state_dict(specs: Mapping[str, TensorSpec], seed: int, dtype: torch.dtype) -> Dict[str, torch.Tensor]:
-    return {name: random_tensor(name, spec, seed, dtype) for name, spec in specs.items()}
+def random_state_dict(specs: Mapping[str, TensorSpec], seed: int, dtype: torch.dtype,
+                      gain: Optional[float] = None) -> Dict[str, torch.Tensor]:
+    return {name: random_tensor(name, spec, seed, dtype, gain) for name, spec in specs.items()}
 
 
 def random_tensors_on_device(specs: Mapping[str, TensorSpec], seed: int, dtype: torch.dtype,
@@ -68,7 +74,7 @@ def random_tensors_on_device(specs: Mapping[str, TensorSpec], seed: int, dtype: 
 
 
 def write_random_model(model_dir: str, config_dict: Mapping[str, Any], seed: int,
-                       dtype: Optional[str] = None) -> str:
+                       dtype: Optional[str] = None, gain: Optional[float] = None) -> str:
     """Creates ``model_dir`` with ``config.json`` and a seeded ``model.safetensors``."""
     from safetensors.torch import save_file
     from ..models.builder import tensor_specs_for_config
@@ -81,7 +87,7 @@ def write_random_model(model_dir: str, config_dict: Mapping[str, Any], seed: int
     specs = tensor_specs_for_config(cfg)
     os.makedirs(model_dir, exist_ok=True)
     write_config_json(model_dir, cfg)
-    state = random_state_dict(specs, seed, _DTYPES[dtype_name])
+    state = random_state_dict(specs, seed, _DTYPES[dtype_name], gain)
     save_file(state, os.path.join(model_dir, "model.safetensors"), metadata={"format": "pt"})
     return model_dir
 
@@ -99,10 +105,12 @@ def main(argv=None) -> int:
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--dtype", choices=sorted(_DTYPES), default=None,
                     help="storage type of the tensors (default: the configuration's torch_dtype)")
+    ap.add_argument("--gain", type=float, default=None,
+                    help="matrices [out, in] are N(0, gain / sqrt(in)) instead of N(0, 0.02)")
     args = ap.parse_args(argv)
     with open(args.config) as f:
         cfg = json.load(f)
-    print(write_random_model(args.out, cfg, args.seed, args.dtype))
+    print(write_random_model(args.out, cfg, args.seed, args.dtype, args.gain))
     return 0
 
 

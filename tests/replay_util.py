@@ -45,6 +45,12 @@ def run_trace(model_dir: str, dtype: str, steps: List[dict], max_tokens: int, ou
     return rows
 
 
+def cache_stats(out_dir: str) -> dict:
+    """What trace_run's cache manager counted during the replay that wrote ``out_dir``."""
+    with open(os.path.join(out_dir, "cache_stats.json")) as f:
+        return json.load(f)
+
+
 def whole(requests: Dict[str, List[int]]) -> List[dict]:
     """Each request alone and whole, one step each, logits everywhere."""
     return [{"step": i, "entries": [{"id": rid, "tokens": toks, "want": list(range(len(toks)))}],

@@ -29,7 +29,7 @@ def test_checksum_is_order_sensitive():
 
 
 @pytest.mark.gpu
-def test_served_tokens_are_the_same_in_both_cache_modes(model_dirs, tmp_path, gpu):
+def test_served_tokens_are_the_same_in_both_cache_modes(sharp_model_dirs, tmp_path, gpu):
     """The reference's cross-build gate (bench.py:226-237): the paged and the contiguous engine
     emit the same ids, and every sequence emits exactly its budget."""
     results = {}
@@ -37,7 +37,7 @@ def test_served_tokens_are_the_same_in_both_cache_modes(model_dirs, tmp_path, gp
         out = tmp_path / f"{mode}.json"
         env = dict(os.environ, IGNORE_EOS="1", ORCA_POLICY="oracle", REPETITION_PENALTY="1.15",
                    PYTHONPATH=ROOT)
-        cmd = [sys.executable, "-m", "kv_cache_optimization_for_llm_amd.cli.client", model_dirs["C"], "5",
+        cmd = [sys.executable, "-m", "kv_cache_optimization_for_llm_amd.cli.client", sharp_model_dirs["C"], "5",
                "--prompt-len", "21", "--max-new-tokens", "12", "--num-seqs", "2", "--out", str(out), "--",
                "--dtype", "float32", "--cache-mode", mode, "--max-seqs", "6", "--max-seq-len", "64",
                "--cache-tokens", "512", "--chunk-size", "8", "--max-batch-tokens", "24"]
@@ -53,12 +53,12 @@ def test_served_tokens_are_the_same_in_both_cache_modes(model_dirs, tmp_path, gp
 
 
 @pytest.mark.gpu
-def test_sweep_reports_both_cache_modes_on_a_small_shape(model_dirs, tmp_path, gpu, capsys):
+def test_sweep_reports_both_cache_modes_on_a_small_shape(sharp_model_dirs, tmp_path, gpu, capsys):
     """The sweep command on a tiny configuration: every request finishes with its budget, the
     contiguous cache reserves more than it holds (whole reservations), the paged cache about what
     it holds, and with a small pool pages are used again."""
     from kv_cache_optimization_for_llm_amd.cli import sweep
-    cfg = os.path.join(model_dirs["A"], "config.json")
+    cfg = os.path.join(sharp_model_dirs["A"], "config.json")
     out = tmp_path / "sweep.jsonl"
     assert sweep.main(["--shapes", cfg, "--batches", "3,6", "--cache-modes", "paged,contiguous", "--prompt-len", "40",
                        "--prompt-min", "5", "--workload", "mixed", "--new-tokens", "12", "--max-seqs", "3",
@@ -72,3 +72,30 @@ def test_sweep_reports_both_cache_modes_on_a_small_shape(model_dirs, tmp_path, g
     paged, contiguous = lines[1], lines[3]
     assert paged["reserved_over_live"] < contiguous["reserved_over_live"]
     assert paged["pages_reused"] > 0                  # six requests through three seats
+
+
+@pytest.mark.gpu
+def test_plain_serve_command_starts_on_a_config_with_131072_positions(tmp_path, gpu):
+    """``serve MODEL_DIR`` with nothing else given: 64 seats and a config.json that allows 131,072
+    positions.  Every seat at its longest is far more cache than a served model leaves room
+    for; the pool is made from what is free instead (the reference sizes its pool last, from
+    leftover memory, paged_attention/src/engine.cu:186-215) and says how large it is."""
+    from conftest import MID_E
+    from kv_cache_optimization_for_llm_amd.weights.random_init import write_random_model
+    cfg = dict(MID_E, max_position_embeddings=131072, num_hidden_layers=4)
+    model_dir = write_random_model(str(tmp_path / "m"), cfg, 3, gain=1.0)
+    env = dict(os.environ, IGNORE_EOS="1", PYTHONPATH=ROOT)
+    proc = subprocess.run([sys.executable, "-m", "kv_cache_optimization_for_llm_amd.cli.serve", model_dir,
+                           "--gemm-tune-rows", ""],
+                          input="1 6 1 5 6 7 8 9\n2 4 2 11 12 13\n", env=env, cwd=ROOT, capture_output=True,
+                          text=True, timeout=280)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    lines = [json.loads(l) for l in proc.stdout.splitlines()]
+    conf = lines[0]
+    assert conf["type"] == "engine_config" and conf["batch_size"] == 64 and conf["max_seq_len"] == 131072
+    page_bytes = 4 * 2 * 2 * 64 * 16 * 2                       # layers x (K, V) x kv heads x head size x tokens x bf16
+    assert 0 < conf["kv_pool_tokens"] <= 64 * 131072
+    assert conf["kv_pool_tokens"] // 16 * page_bytes < 280 * 2 ** 30
+    done = {(l["id"], l["seq"]): l for l in lines if l.get("done")}
+    assert {k: v["tokens"] for k, v in done.items()} == {(1, 0): 6, (2, 0): 4, (2, 1): 4}
+    assert not any("error" in v for v in done.values())

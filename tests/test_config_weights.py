@@ -36,6 +36,7 @@ def test_config_defaults_follow_the_keys():
 @pytest.mark.parametrize("patch, word", [
     ({"num_key_value_heads": 3}, "multiple"),
     ({"head_dim": 15}, "even"),
+    ({"head_dim": 18}, "multiples of 4"),
     ({"hidden_act": "gelu"}, "hidden_act"),
     ({"attention_bias": True}, "attention_bias"),
     ({"mlp_bias": True}, "mlp_bias"),
@@ -160,6 +161,8 @@ def test_dtype_rule():
     assert target_dtype(bf, "matrix", bf) == bf          # kept in bfloat16
     assert target_dtype(bf, "matrix", f32) == f32        # widened exactly for the 32-bit path
     assert target_dtype(f32, "vector", bf) == f32        # stored in 32-bit stays so
+    # float16 does not fit into bfloat16: it is widened to 32-bit on either engine
+    assert target_dtype(torch.float16, "matrix", bf) == f32 and target_dtype(torch.float16, "matrix", f32) == f32
     assert target_dtype(torch.int64, "table", bf) == torch.int32
 
 

@@ -380,6 +380,52 @@ def test_attention_finds_one_far_key_among_hundreds(gpu):
                     close(out2, want, dt, f"mfma far={far} splits={splits}", tol16=8e-3)
 
 
+@pytest.mark.parametrize("nkv, ctx", [(1, 65536), (2, 65536), (4, 131072), (1, 131072)])
+def test_attention_of_one_decoded_token_over_a_very_long_context(nkv, ctx, gpu):
+    """Few kv heads, one request, a context of 65,536 or 131,072 keys: the split policy wants more
+    key ranges than the kernels take and must stop at their limit.  One key at a range's edge is
+    made to dominate, so a range that is dropped or counted twice shows."""
+    nq, d, page = 2 * nkv, 64, 16
+    splits, per = choose_splits(1, nkv, ctx)
+    assert splits == K.attention_max_splits() == 256 and splits * per >= ctx
+    far = per * 101 - 1                                   # the last key of range 100
+    g = torch.Generator().manual_seed(ctx + nkv)
+    k = torch.randn(ctx, nkv, d, generator=g) * 0.1
+    v = torch.randn(ctx, nkv, d, generator=g)
+    q = torch.randn(nq, d, generator=g) * 0.1
+    k[far] = 0
+    k[far, :, 3] = 12.0
+    q[:, 3] = 12.0
+    k, v, q = (t.to(torch.bfloat16) for t in (k, v, q))
+    pages = ctx // page
+    perm = torch.randperm(pages, generator=g)
+    kc = torch.empty(pages, nkv, page, d, dtype=torch.bfloat16)
+    vc = torch.empty(pages, nkv, d, page, dtype=torch.bfloat16)
+    kc[perm] = k.view(pages, page, nkv, d).permute(0, 2, 1, 3)
+    vc[perm] = v.view(pages, page, nkv, d).permute(0, 2, 3, 1)
+    # the last row of plain causal attention, written out for one query (the plain function
+    # computes every row: 131,072 squared is too much)
+    want = torch.empty(nq, d)
+    for h in range(nq):
+        kh = h // (nq // nkv)
+        scores = (k[:, kh].float() @ q[h].float()) / 8.0
+        p = torch.softmax(scores.double(), 0).float()
+        want[h] = p @ v[:, kh].float()
+    assert (want[0] - v[far, 0].float()).abs().max() < 0.3          # that key really dominates
+    qkv = torch.zeros(1, (nq + 2 * nkv) * d, dtype=torch.bfloat16)
+    qkv[0, :nq * d] = q.reshape(-1)
+    out = torch.empty(1, nq * d, dtype=torch.bfloat16, device=gpu)
+    zero = torch.zeros(1, dtype=torch.int32, device=gpu)
+    K.attention_mfma(qkv.to(gpu), qkv.shape[1], out, kc.to(gpu), vc.to(gpu), perm.to(torch.int32)[None].to(gpu),
+                     zero, zero, zero, torch.tensor([0, 1], dtype=torch.int32, device=gpu),
+                     torch.tensor([ctx - 1], dtype=torch.int32, device=gpu), nq, nkv, d, 1 / 8.0, 0, splits, per)
+    close(out, want.reshape(1, -1), torch.bfloat16, f"{nkv} kv heads, {ctx} keys, {splits} splits", tol16=8e-3)
+    with pytest.raises(K.KernelError):                    # and the kernel itself refuses more
+        K.attention_mfma(qkv.to(gpu), qkv.shape[1], out, kc.to(gpu), vc.to(gpu), perm.to(torch.int32)[None].to(gpu),
+                         zero, zero, zero, torch.tensor([0, 1], dtype=torch.int32, device=gpu),
+                         torch.tensor([ctx - 1], dtype=torch.int32, device=gpu), nq, nkv, d, 1 / 8.0, 0, 512, 256)
+
+
 def test_choose_splits():
     assert choose_splits(4096, 8, 2048) == (1, 0)                 # a big prompt fills the GPU by itself
     s, per = choose_splits(1, 8, 8192)

@@ -71,10 +71,42 @@ def test_llama3_scaling_has_three_bands_and_is_continuous():
     assert ((got[mid] < base[mid]) & (got[mid] > base[mid] / 8.0)).all()    # between the two
     # factor 1 changes nothing
     assert np.allclose(plain.rope_inv_freq(64, 500000.0, dict(sc, factor=1.0)), base, rtol=1e-6)
-    # continuity at both edges: smooth is 0 at wavelen = low_wl and 1 at wavelen = high_wl
-    for wavelen, want in ((64.0, 1 / 8.0), (16.0, 1.0)):
-        smooth = (64.0 / wavelen - 1.0) / (4.0 - 1.0)
-        assert abs((1 - smooth) / 8.0 + smooth - want) < 1e-12
+
+
+def theta_for_wavelength(wavelen, head_dim, i):
+    """The theta that gives frequency index ``i`` (of ``head_dim / 2``) the wavelength
+    ``wavelen``: 2 pi theta^(2i/d) = wavelen."""
+    return (wavelen / (2 * math.pi)) ** (head_dim / (2.0 * i))
+
+
+def test_llama3_mid_band_meets_the_outer_bands_at_both_edges():
+    """``rope_inv_freq`` itself is evaluated at frequencies put on and just inside both edges of
+    the middle band: at wavelength orig / low_freq_factor it must give inv / factor (where the
+    long-wave band begins), at orig / high_freq_factor the unscaled inv, and just inside each
+    edge a value next to those.  A swapped pair of factors, a smooth that runs the wrong way or
+    an interpolation of wavelengths instead of frequencies fails here."""
+    d, i, orig, factor, low, high = 64, 8, 256.0, 8.0, 1.0, 4.0
+    sc = dict(rope_type="llama3", factor=factor, low_freq_factor=low, high_freq_factor=high,
+              original_max_position_embeddings=int(orig))
+    low_wl, high_wl = orig / low, orig / high
+
+    def at(wavelen):
+        theta = theta_for_wavelength(wavelen, d, i)
+        base = plain.rope_inv_freq(d, theta, None)[i]
+        assert abs(2 * math.pi / base - wavelen) < 1e-3 * wavelen      # the frequency sits where it was put
+        return plain.rope_inv_freq(d, theta, sc)[i] / base              # what scaling made of it
+
+    assert abs(at(low_wl * 1.01) - 1 / factor) < 1e-6          # beyond the long edge: / factor
+    assert abs(at(low_wl * 0.999) - 1 / factor) < 2e-3         # just inside: next to it ...
+    assert at(low_wl * 0.999) > 1 / factor                     # ... and already above it
+    assert abs(at(high_wl * 1.001) - 1.0) < 2e-3               # just inside the short edge: next to unscaled
+    assert at(high_wl * 1.001) < 1.0
+    assert at(high_wl * 0.99) == 1.0                           # beyond the short edge: unchanged
+    # half-way in frequency (wavelength orig / 2.5: smooth = 0.5) the value is the mean of the two ends
+    assert abs(at(orig / 2.5) - 0.5 * (1 / factor + 1.0)) < 1e-4
+    # the ratio falls as the wavelength grows, all the way through the band
+    ratios = [at(w) for w in np.linspace(high_wl * 1.001, low_wl * 0.999, 9)]
+    assert all(a > b for a, b in zip(ratios, ratios[1:]))
 
 
 @pytest.mark.parametrize("nq, nkv, d", [(4, 2, 16), (6, 1, 24), (3, 3, 8)])
@@ -149,8 +181,14 @@ def test_model_is_causal_and_a_shift_of_all_positions_changes_nothing(cfg):
     a = plain.hidden_states(cfg, W, toks, first_position=0)
     b = plain.hidden_states(cfg, W, toks, first_position=37)
     assert torch.allclose(a, b, atol=2e-4)                        # only distances count
-    head = W["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings") else W["lm_head.weight"]
-    assert torch.allclose(full, plain.hidden_states(cfg, W, toks) @ head.t(), atol=1e-6)
+    # tied: the table is the output matrix; untied: lm_head is, and the table is not
+    x = plain.hidden_states(cfg, W, toks)
+    table = W["model.embed_tokens.weight"]
+    if cfg.get("tie_word_embeddings"):
+        assert torch.allclose(full, F.linear(x, table), atol=1e-6)
+    else:
+        assert torch.allclose(full, F.linear(x, W["lm_head.weight"]), atol=1e-6)
+        assert not torch.allclose(full, F.linear(x, table), atol=1e-2)
 
 
 def test_bf16_emulation_rounds_every_output():
@@ -167,6 +205,17 @@ def peaked_logits(vocab=128256, seed=0):
     logits = rng.normal(0.0, 2.0, vocab)
     logits[rng.choice(vocab, 20, replace=False)] += 12.0
     return logits
+
+
+def test_counter_uniform_is_splitmix64_of_the_counter():
+    """With seed, key and step all 0 the mixed word is splitmix64's first output for state 0,
+    0xE220A8397B1DCDAF (the public test vector of that generator); its top 24 bits make u."""
+    assert plain.counter_uniform(0, 0, 0) == 0xE220A8 / 2 ** 24
+    # key sits in the upper half of the counter, step in the lower half, and the seed is folded in
+    # by a multiplication: each of them alone moves the draw
+    assert len({plain.counter_uniform(0, 0, 0), plain.counter_uniform(1, 0, 0),
+                plain.counter_uniform(0, 1, 0), plain.counter_uniform(0, 0, 1)}) == 4
+    assert plain.counter_uniform(0, 1, 0) != plain.counter_uniform(0, 0, 1)
 
 
 def test_counter_uniform_is_in_range_and_a_pure_function():

@@ -1,0 +1,49 @@
+"""Host-side decisions that need no GPU: how attention keys are cut into splits, and how large a
+cache pool is made from leftover device memory."""
+import pytest
+
+from kv_cache_optimization_for_llm_amd.engine.engine import EngineError, pool_pages_from_memory
+from kv_cache_optimization_for_llm_amd.ops.attention import choose_lds_splits, choose_splits
+
+KERNEL_MAX_SPLITS = 256         # what the kernels and their merge take (kva_attention_max_splits)
+
+
+@pytest.mark.parametrize("nkv", [1, 2, 4, 8])
+@pytest.mark.parametrize("items", [1, 2, 3])
+@pytest.mark.parametrize("context", [4096, 32768, 65536, 100000, 131072])
+def test_key_splits_never_exceed_what_the_kernels_take(nkv, items, context):
+    """Few kv heads, one or two decoding requests and a long context ask for many splits; the
+    policy must stop at the kernels' limit, and its ranges must still cover every key."""
+    for splits, per in (choose_splits(items, nkv, context, KERNEL_MAX_SPLITS),
+                        choose_lds_splits(items * nkv, context, KERNEL_MAX_SPLITS)):
+        assert 1 <= splits <= KERNEL_MAX_SPLITS
+        if splits > 1:
+            assert per % 32 == 0 and splits * per >= context and (splits - 1) * per < context
+
+
+def test_the_clamp_is_what_bites_for_few_kv_heads():
+    # one request on one kv head at 131,072 keys would ask for 1,024 ranges of 128 keys
+    assert choose_splits(1, 1, 131072, 4096)[0] == 1024
+    assert choose_splits(1, 1, 131072, KERNEL_MAX_SPLITS) == (256, 512)
+    assert choose_splits(1, 4, 65536, KERNEL_MAX_SPLITS) == (256, 256)
+    assert choose_splits(4096, 8, 2048, KERNEL_MAX_SPLITS) == (1, 0)      # a big prompt fills the GPU by itself
+    assert choose_splits(1, 8, 100, KERNEL_MAX_SPLITS) == (1, 0)          # too short to split
+
+
+def test_pool_from_leftover_memory():
+    GiB = 1 << 30
+    # Llama-3.2-1B: 16 layers x 2 x 8 heads x 64 x 16 tokens x 2 bytes = 512 KiB a page
+    page_bytes = 16 * 2 * 8 * 64 * 16 * 2
+    # config.json says 131,072 positions and the server has 64 seats: every seat at its longest
+    # would be 256 GiB; the pool takes what is free instead
+    pages = pool_pages_from_memory(200 * GiB, page_bytes, page_size=16, max_seqs=64, max_seq_len=131072,
+                                   margin_bytes=2 * GiB, step_bytes=4 * GiB)
+    assert pages == (200 - 2 - 4) * GiB // page_bytes
+    assert pages * page_bytes <= 194 * GiB < 64 * 131072 // 16 * page_bytes
+    # a small model on a big device: never more than every seat at its longest
+    assert pool_pages_from_memory(200 * GiB, 4096, page_size=16, max_seqs=8, max_seq_len=100,
+                                  margin_bytes=GiB) == 8 * 7
+    with pytest.raises(EngineError) as e:
+        pool_pages_from_memory(3 * GiB, page_bytes, page_size=16, max_seqs=8, max_seq_len=8192,
+                               margin_bytes=2 * GiB, step_bytes=2 * GiB)
+    assert "no room for a cache pool" in str(e.value)

@@ -54,10 +54,24 @@ def replay(model_dir, dtype, steps, page):
     return rows
 
 
-@pytest.mark.parametrize("case", range(12))
+def wide_group_config(nq, nkv, d):
+    """More than 16 query heads on one kv head: a decoded token is then more than one tile of 16
+    query rows for the matrix-core attention kernel."""
+    return dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=211, hidden_size=nq * d // 4,
+                intermediate_size=320, num_hidden_layers=2, num_attention_heads=nq, num_key_value_heads=nkv,
+                head_dim=d, rms_norm_eps=1e-5, rope_theta=10000.0, max_position_embeddings=1024,
+                tie_word_embeddings=False, hidden_act="silu", torch_dtype="bfloat16")
+
+
+@pytest.mark.parametrize("case", list(range(12)) + ["32 heads on 1", "40 heads on 2", "17 heads on 1"])
 def test_random_configuration_under_two_cuts(case, tmp_path, gpu):
-    rng = np.random.default_rng(4000 + case)
-    cfg = random_config(rng)
+    if isinstance(case, str):
+        nq, nkv, d = {"32 heads on 1": (32, 1, 64), "40 heads on 2": (40, 2, 32), "17 heads on 1": (17, 1, 16)}[case]
+        rng = np.random.default_rng(nq * 100 + d)
+        cfg, case = wide_group_config(nq, nkv, d), nq
+    else:
+        rng = np.random.default_rng(4000 + case)
+        cfg = random_config(rng)
     page = int(rng.choice([16, 16, 8, 32, 4]))
     lengths = [int(x) for x in rng.integers(1, 200, 5)]
     model_dir = write_random_model(str(tmp_path / "m"), cfg, case)

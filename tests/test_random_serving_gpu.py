@@ -33,7 +33,7 @@ def workload(case):
 @pytest.mark.parametrize("case", range(8))
 def test_greedy_tokens_in_a_tight_cache_are_the_plain_model_s(case, tmp_path, gpu):
     rng, cfg, page, prompts, new, seats, longest, tight = workload(case)
-    model_dir = write_random_model(str(tmp_path / "m"), cfg, case)
+    model_dir = write_random_model(str(tmp_path / "m"), cfg, case, gain=1.0)
     pcfg, W = plain.load_model_dir(model_dir)
     want = [plain.generate(pcfg, W, p, new) for p in prompts]
     llm = LLM(model_dir, EngineOptions(dtype="float32", page_size=page, max_seqs=seats, max_seq_len=longest,
@@ -50,7 +50,7 @@ def test_greedy_tokens_in_a_tight_cache_are_the_plain_model_s(case, tmp_path, gp
 @pytest.mark.parametrize("case", range(8, 16))
 def test_sampled_output_does_not_depend_on_room_portions_or_running_ahead(case, tmp_path, gpu):
     rng, cfg, page, prompts, new, seats, longest, tight = workload(case)
-    model_dir = write_random_model(str(tmp_path / "m"), cfg, case)
+    model_dir = write_random_model(str(tmp_path / "m"), cfg, case, gain=1.0)
     temperature, penalty = float(rng.choice([0.7, 1.3])), float(rng.choice([1.0, 1.15]))
     runs = []
     for pool, chunk, budget, ahead, n_seats in ((seats * longest + 64, None, 256, True, seats),

@@ -51,14 +51,57 @@ LENGTHS = {"A": [5, 17, 33, 70, 131], "B": [1, 9, 40, 70, 97], "C": [3, 66, 130,
            "D": [2, 35, 90, 64, 150], "E": [4, 130, 300, 65, 517], "F": [2, 257, 48, 330, 129]}
 
 
+# the page size each configuration is replayed at (B: the 8 its baseline configuration names)
+PAGE = {"A": 16, "B": 8, "C": 16, "D": 16, "E": 16, "F": 16}
+
+
+def same_rows(a, b, dtype, what):
+    """float32: every reduction has a fixed order that does not depend on the batch, so two cuts
+    give the same bits.  bfloat16: the split counts of attention and of the few-rows products
+    depend on the batch, which changes rounding only."""
+    assert a.keys() == b.keys()
+    if dtype == "float32":
+        bad = [k for k in a if not np.array_equal(a[k], b[k])]
+        assert not bad, f"{what}: float32 logits are not bit-identical at {bad[:5]} ({len(bad)} rows)"
+    else:
+        for k in a:
+            scale = float(np.abs(a[k]).max())
+            assert float(np.abs(a[k] - b[k]).max()) <= 2 * TOL[dtype] * scale, f"{what}: rows differ at {k}"
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F"])
 def test_every_cut_matches_plain(name, dtype, model_dirs, plain_rows, tmp_path, gpu):
     vocab = TINY[name][0]["vocab_size"]
     requests = make_requests(vocab, LENGTHS[name], seed=5)
     ref = plain_rows(name, requests)
+    page = ["--page-size", str(PAGE[name])]
+    got = {}
     for what, steps in (("whole", ru.whole(requests)), ("tail decoded", ru.tail_decoded(requests)),
                         ("portions", ru.chunked(requests)), ("mixed", ru.mixed(requests, seed=3))):
         budget = ru.max_live_tokens(steps)
-        rows = ru.run_trace(model_dirs[name], dtype, steps, budget, str(tmp_path / what.replace(" ", "_")), vocab)
+        out = str(tmp_path / what.replace(" ", "_"))
+        rows = ru.run_trace(model_dirs[name], dtype, steps, budget, out, vocab, page)
         compare(rows, ref, requests, dtype, what)
+        got[what] = rows
+        if what == "mixed":
+            # the pool holds the most that is live at a time, less than all requests together:
+            # later requests can only have run on pages that earlier ones gave back
+            stats = ru.cache_stats(out)
+            assert stats["pages_reused"] > 0 and stats["kv_tokens_total"] < sum(
+                (len(t) + 63) // 64 * 64 for t in requests.values()), f"mixed: no page was used again: {stats}"
+    # the same mixed trace over the contiguous (buddy) cache: every request reserves one run that
+    # holds the longest of them, four runs fill the pool, and runs are handed out again
+    longest = max(len(t) for t in requests.values())
+    run = PAGE[name]
+    while run < longest:
+        run *= 2
+    out = str(tmp_path / "mixed_contiguous")
+    rows = ru.run_trace(model_dirs[name], dtype, ru.mixed(requests, seed=3), 4 * run, out, vocab,
+                        page + ["--cache-mode", "contiguous", "--reserve-tokens", str(run)])
+    compare(rows, ref, requests, dtype, "mixed, contiguous")
+    got["mixed, contiguous"] = rows
+    assert ru.cache_stats(out)["kv_tokens_total"] == 4 * run
+    # and the cuts agree with each other, not only with the plain implementation
+    for what in ("tail decoded", "portions", "mixed", "mixed, contiguous"):
+        same_rows(got["whole"], got[what], dtype, f"whole against {what}")
