@@ -65,6 +65,19 @@ class CacheGroup:
     def free_pages(self) -> int:
         return self.pool.free_count if self.pool is not None else self.buddy.free_units
 
+    def pages_for(self, tokens: int, portion: Optional[int] = None) -> int:
+        """Most pages one request holds in this group at any time while a prompt of ``tokens``
+        tokens is brought in by steps of at most ``portion`` tokens.  All keys stay: one page per
+        ``page_size`` tokens.  A window group keeps only what the newest position can still see
+        plus the step being written, whatever the prompt's length: ``window - 1 + portion``
+        positions, which touch one page more than they fill when they straddle page edges."""
+        whole = (tokens + self.page_size - 1) // self.page_size
+        if self.spec.kind != "window" or self.spec.window <= 0:
+            return whole
+        step = min(tokens, portion) if portion else tokens
+        span = self.spec.window - 1 + step
+        return min(whole, (span + self.page_size - 1) // self.page_size + 1)
+
     def mark_dirty(self, seat: int, lo: int, hi: int) -> None:
         d = self.dirty.get(seat)
         if d is None:
@@ -244,6 +257,16 @@ class CacheManager:
         blocks = (new_len + self.page_size - 1) // self.page_size
         return [max(0, blocks - s.next_block[g.index]) for g in self.groups]
 
+    def pages_outstanding(self, seat: int, final_len: int, portion: Optional[int] = None) -> List[int]:
+        """Pages each group may still have to find for this seat until ``final_len`` tokens are in
+        the cache (a prompt is mapped portion by portion): what the group needs at most at one
+        time, less what the seat holds now."""
+        s = self.seat(seat)
+        if self.mode == "contiguous":
+            return self._no_pages
+        return [max(0, g.pages_for(final_len, portion) - (s.next_block[g.index] - s.first_block[g.index]))
+                for g in self.groups]
+
     def can_grow(self, seat: int, new_len: int) -> bool:
         if new_len > self.capacity_tokens(seat):
             return False
@@ -278,7 +301,9 @@ class CacheManager:
             g.table_host[seat, lo:lo + n] = np.asarray(pages, dtype=np.int32)
             g.mark_dirty(seat, lo, lo + n)
             s.next_block[g.index] = lo + n
-        s.mapped_tokens = min(min(s.next_block) * self.page_size, self.capacity_tokens(seat))   # never past the longest sequence
+        # never past the longest sequence; a model without any paged group has a place for all of them
+        mapped = min(s.next_block) * self.page_size if s.next_block else new_len
+        s.mapped_tokens = min(mapped, self.capacity_tokens(seat))
         self._note_peak()
         return True
 

@@ -237,6 +237,37 @@ extern "C" int kva_residual_add(void *hidden, const void *delta, long long n, in
 }
 
 // ---------------------------------------------------------------------------------------
+// x <- x * scale, and then, with cap > 0, x <- cap * tanh(x / cap): the constants a model may put
+// on its embeddings and on its logits.  fp32 arithmetic, rounded to the storage type.
+template <typename T>
+__global__ void scale_softcap_kernel(T *__restrict__ x, size_t n, float scale, float cap) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const float inv_cap = cap > 0.f ? 1.f / cap : 0.f;
+    for (; i < n; i += stride) {
+        float v = to_float(x[i]) * scale;
+        if (cap > 0.f) v = cap * tanhf(v * inv_cap);
+        x[i] = from_float<T>(v);
+    }
+}
+
+extern "C" int kva_scale_softcap(void *x, long long n, float scale, float cap, int dtype, hipStream_t stream) {
+    KVA_REQUIRE(n >= 0 && cap >= 0.f, "scale_softcap: bad size or a negative cap");
+    if (n == 0) return KVA_OK;
+    int blocks = (int)((n + 255) / 256);
+    if (blocks > 8192) blocks = 8192;
+    if (dtype == KVA_F32)
+        hipLaunchKernelGGL(scale_softcap_kernel<float>, dim3(blocks), dim3(256), 0, stream, (float *)x, (size_t)n,
+                           scale, cap);
+    else if (dtype == KVA_BF16)
+        hipLaunchKernelGGL(scale_softcap_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, (bf16_t *)x,
+                           (size_t)n, scale, cap);
+    else KVA_REQUIRE(false, "scale_softcap: unsupported dtype %d", dtype);
+    KVA_CHECK_LAUNCH("scale_softcap");
+    return KVA_OK;
+}
+
+// ---------------------------------------------------------------------------------------
 // out[t, i] = silu(gu[t, i]) * gu[t, inter + i]; silu(g) = g / (1 + exp(-g)) in fp32.
 template <typename T>
 __global__ void silu_mul_kernel(T *__restrict__ out, const T *__restrict__ gate_up, int inter) {

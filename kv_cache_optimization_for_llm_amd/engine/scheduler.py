@@ -271,7 +271,7 @@ class Scheduler:
             need = [0] * len(cache.groups)
             for s in self.running:
                 if s.prefilling:
-                    for i, n in enumerate(cache.pages_needed(s.seat, len(s.prompt))):
+                    for i, n in enumerate(cache.pages_outstanding(s.seat, len(s.prompt), self.chunk_size)):
                         need[i] += n
             return need
 
@@ -324,10 +324,13 @@ class Scheduler:
                 continue
             reserve = None
             if paged:
-                pages = (plen + cache.page_size - 1) // cache.page_size
+                # every group says what a prompt of this length needs of it (all its pages where
+                # all keys stay, a window's worth where only a window is kept, nothing where a
+                # model keeps no keys at all)
+                pages = [g.pages_for(plen, self.chunk_size) for g in cache.groups]
                 free = [f - d - o for f, d, o in zip(self._free_pages(), decode_pages, prompt_pages_outstanding())]
-                if any(pages > f for f in free):
-                    if not self.running and not entries and any(pages > g.num_pages for g in cache.groups):
+                if any(p > f for p, f in zip(pages, free)):
+                    if not self.running and not entries and any(p > g.num_pages for p, g in zip(pages, cache.groups)):
                         self.waiting.popleft()
                         events.append(Event("done", head.id, head.seq_index, tokens=head.resumed_tokens,
                                             reason="kv_cache_exhausted"))

@@ -26,9 +26,8 @@ def build_blocks(spec: ModelSpec) -> List[Block]:
     for ls in spec.layers:
         mixer = MIXERS.get(ls.mixer.kind)(**ls.mixer.params)
         ffn = FEED_FORWARDS.get(ls.feed_forward.kind)(**ls.feed_forward.params)
-        n1 = NORMS.get(ls.mixer_norm.kind)(**ls.mixer_norm.params)
-        n2 = NORMS.get(ls.ffn_norm.kind)(**ls.ffn_norm.params)
-        blocks.append(BLOCKS.get(ls.block.kind)(mixer, ffn, n1, n2, **ls.block.params))
+        norms = {name: NORMS.get(ns.kind)(**ns.params) for name, ns in ls.norms.items()}
+        blocks.append(BLOCKS.get(ls.block.kind)(mixer, ffn, norms, **ls.block.params))
     return blocks
 
 
@@ -177,6 +176,8 @@ class Model:
         T = batch.num_tokens
         hidden = torch.empty((T, self.spec.hidden_size), dtype=self.dtype, device=self.device)
         K.embed_gather(self.embedding, batch.token_ids, hidden, getattr(batch, "feedback", None))
+        if self.spec.embedding_scale != 1.0:
+            K.scale_softcap(hidden, self.spec.embedding_scale)
         delta = None
         for i, (call, slot) in enumerate(self.calls):
             block = self.blocks[call.layer]
@@ -204,4 +205,6 @@ class Model:
         else:
             x = self.final_norm.forward(hidden, delta=delta, row_idx=batch.logit_rows)
         self.head(x, out=logits)
+        if self.spec.logit_scale != 1.0 or self.spec.logit_softcap > 0.0:
+            K.scale_softcap(logits, self.spec.logit_scale, self.spec.logit_softcap)
         return logits

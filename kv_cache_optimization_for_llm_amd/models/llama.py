@@ -31,10 +31,12 @@ def llama_spec(cfg: LlamaConfig) -> ModelSpec:
             feed_forward=PartSpec("swiglu", dict(
                 prefix=p + "mlp.", hidden_size=cfg.hidden_size,
                 intermediate_size=cfg.intermediate_size)),
-            mixer_norm=PartSpec("rmsnorm", dict(prefix=p + "input_layernorm.", width=cfg.hidden_size,
-                                                eps=cfg.rms_norm_eps)),
-            ffn_norm=PartSpec("rmsnorm", dict(prefix=p + "post_attention_layernorm.",
-                                              width=cfg.hidden_size, eps=cfg.rms_norm_eps)),
+            norms={
+                "mixer": PartSpec("rmsnorm", dict(prefix=p + "input_layernorm.", width=cfg.hidden_size,
+                                                  eps=cfg.rms_norm_eps)),
+                "feed_forward": PartSpec("rmsnorm", dict(prefix=p + "post_attention_layernorm.",
+                                                         width=cfg.hidden_size, eps=cfg.rms_norm_eps)),
+            },
             prefix=p,
         ))
     return ModelSpec(

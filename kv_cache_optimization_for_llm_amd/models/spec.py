@@ -2,7 +2,7 @@
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional, Tuple
+from typing import Any, Dict, List, Mapping, Optional, Tuple
 
 
 @dataclass(frozen=True)
@@ -29,13 +29,17 @@ class TensorSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer: a block arrangement around a mixer and a feed-forward."""
+    """One layer: a block arrangement around a mixer and a feed-forward, with its norms by name.
+
+    ``norms`` maps the names the block arrangement knows (the pre-norm block: ``"mixer"`` and
+    ``"feed_forward"``, the norms in front of the two branches; an arrangement with norms after
+    its branches too, or with a single one, names its own) to their specs.  The order of the
+    mapping is the order in which the block's parts are listed."""
 
     block: PartSpec                      # e.g. PartSpec("pre_norm")
     mixer: PartSpec
     feed_forward: PartSpec
-    mixer_norm: PartSpec
-    ffn_norm: PartSpec
+    norms: Mapping[str, PartSpec]
     prefix: str                          # tensor-name prefix, e.g. "model.layers.3."
 
 
@@ -66,6 +70,12 @@ class ModelSpec:
     final_norm_prefix: str
     head_name: Optional[str]             # tensor name of the output matrix; None = tied to the table
     max_positions: int
+    # Constants around the layers (1 and 0 leave a value as it is): the rows taken from the token
+    # table are multiplied by ``embedding_scale``; logits are multiplied by ``logit_scale`` and
+    # then, with a positive ``logit_softcap`` c, replaced by c * tanh(logit / c).
+    embedding_scale: float = 1.0
+    logit_scale: float = 1.0
+    logit_softcap: float = 0.0
     eos_token_ids: Tuple[int, ...] = ()
     ignorable_tensors: Tuple[str, ...] = ()   # fnmatch patterns of tensors that may be present unused
 

@@ -116,6 +116,15 @@ def residual_add(hidden: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
     return hidden
 
 
+def scale_softcap(x: torch.Tensor, scale: float, cap: float = 0.0) -> torch.Tensor:
+    """In place: ``x *= scale``, then with ``cap > 0`` ``x = cap * tanh(x / cap)``."""
+    if cap < 0:
+        raise KernelError("scale_softcap: the cap must not be negative")
+    check(hip_lib().kva_scale_softcap(_dev(x, "x"), x.numel(), float(scale), float(cap), dtype_code(x.dtype),
+                                      _stream()), "scale_softcap")
+    return x
+
+
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]."""
     rows, inter = out.shape
@@ -211,8 +220,12 @@ def sample(logits: torch.Tensor, out_tokens: torch.Tensor, *, chunks: int = 128,
            inv_temperature: Optional[torch.Tensor] = None, seed: int = 0,
            rng_key: Optional[torch.Tensor] = None, rng_step: Optional[torch.Tensor] = None,
            penalty_mask: Optional[torch.Tensor] = None, row_seat: Optional[torch.Tensor] = None,
-           penalty: float = 1.0) -> torch.Tensor:
-    """Greedy (rows whose inv_temperature is 0 or absent) or temperature sampling per row."""
+           penalty: float = 1.0, mark_mask: Optional[torch.Tensor] = None,
+           mark_seat: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Greedy (rows whose inv_temperature is 0 or absent) or temperature sampling per row.
+    ``penalty_mask`` ``[seats, vocab]`` with ``row_seat`` (-1: none) names the logits that are
+    penalised; ``mark_mask`` with ``mark_seat`` (-1: none) gets ``mark_mask[seat, token] = 1`` for
+    every chosen token, in the same launch."""
     rows, vocab = logits.shape
     if out_tokens.shape != (rows,):
         raise KernelError("sample: one output token per row")
@@ -224,15 +237,19 @@ def sample(logits: torch.Tensor, out_tokens: torch.Tensor, *, chunks: int = 128,
         if row_seat is None or row_seat.shape != (rows,) or penalty_mask.dim() != 2 \
                 or penalty_mask.shape[1] != vocab:
             raise KernelError("sample: penalty mask [seats, vocab] needs a seat per row")
+    if (mark_mask is None) != (mark_seat is None) or (mark_mask is not None and (
+            mark_seat.shape != (rows,) or mark_mask.dim() != 2 or mark_mask.shape[1] != vocab)):
+        raise KernelError("sample: marking needs a mask [seats, vocab] and a seat per row")
     lib = hip_lib()
-    ws = torch.empty(lib.kva_sample_workspace_bytes(rows, chunks) // 4, dtype=torch.float32,
+    ws = torch.empty(max(1, lib.kva_sample_workspace_bytes(rows, chunks) // 4), dtype=torch.float32,
                      device=logits.device)
     check(lib.kva_sample(
         _dev(out_tokens, "out_tokens", torch.int32), _dev(logits, "logits", torch.float32), rows, vocab,
         chunks, _opt(penalty_mask, "penalty_mask", torch.uint8), _opt(row_seat, "row_seat", torch.int32),
         float(penalty), _opt(inv_temperature, "inv_temperature", torch.float32), int(seed) & 0xFFFFFFFF,
         _opt(rng_key, "rng_key", torch.int32), _opt(rng_step, "rng_step", torch.int32),
-        1 if any_sampled else 0, _dev(ws, "workspace"), _stream()), "sample")
+        1 if any_sampled else 0, _dev(ws, "workspace"), _opt(mark_mask, "mark_mask", torch.uint8),
+        _opt(mark_seat, "mark_seat", torch.int32), _stream()), "sample")
     return out_tokens
 
 

@@ -22,6 +22,43 @@ from .base import BranchTail, KVCacheSpec, Mixer, MixerContext, NormedRows
 from .linear import Linear
 
 
+class EncodedQKV:
+    """The joined Q/K/V projection with position encoding and cache write: what every mixer that
+    attends over cached keys does first.  It owns the choice between one product that does all of
+    it in its epilogue (few rows, an encoding that is a rotate-half rotation over the whole head,
+    or none) and the product followed by the encoding's own kernel, so that a mixer - this one or
+    another attention variant - only says ``qkv(x, batch, kv)``."""
+
+    def __init__(self, linear: Linear, position, hidden_size: int, num_heads: int, num_kv_heads: int,
+                 head_dim: int):
+        self.linear, self.position = linear, position
+        self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim = hidden_size, num_heads, num_kv_heads, head_dim
+
+    def __call__(self, x, batch, kv):
+        """``x`` [T, hidden] (plain or NormedRows).  Returns a tensor whose first ``nq * d`` columns
+        are the position-encoded queries; K (encoded) and V of the step's tokens are in the cache
+        when ``kv`` allows writing."""
+        tables = None
+        if self.linear.fusable(x) and K.gemm_skinny_qkv_rope_supported(x.shape[0], self.hidden_size, self.head_dim):
+            tables = self.position.rotate_half_tables(x.device, self.head_dim)
+        if tables is None:
+            qkv = self.linear(x)
+            self.position.apply_and_cache(qkv, batch.positions, self.num_heads, self.num_kv_heads,
+                                          self.head_dim, kv)
+            return qkv
+        write = kv is not None and kv.writes
+        q = torch.empty((x.shape[0], self.num_heads * self.head_dim), dtype=torch.bfloat16, device=x.device)
+        norm = {}
+        if isinstance(x, NormedRows):
+            norm = dict(sumsq=x.sumsq, norm_width=x.width, eps=x.eps)
+            x = x.scaled
+        K.gemm_skinny_qkv_rope(x, self.linear.tiled, q, self.num_heads, self.num_kv_heads, self.head_dim,
+                               batch.positions, tables[0], tables[1],
+                               kv.k_cache if write else None, kv.v_cache if write else None,
+                               kv.slot_mapping if write else None, kv.page_size if kv is not None else 0, **norm)
+        return q
+
+
 @MIXERS.register("gqa_attention")
 class GQAAttention(Mixer):
     graph_safe = True
@@ -34,7 +71,7 @@ class GQAAttention(Mixer):
         self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
         self.head_dim, self.scale, self.window = head_dim, float(scale), int(window)
         self.position = POSITION_ENCODINGS.get(position.kind)(**position.params)
-        self.qkv: Optional[Linear] = None
+        self.qkv: Optional[EncodedQKV] = None
         self.o: Optional[Linear] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
@@ -51,7 +88,8 @@ class GQAAttention(Mixer):
         q, k, v = (tensors[p + n + "_proj.weight"] for n in "qkv")
         if not (q.dtype == k.dtype == v.dtype):
             raise ValueError(f"{p}: q/k/v projection weights are stored in different dtypes")
-        self.qkv = Linear(torch.cat([q, k, v], dim=0))
+        self.qkv = EncodedQKV(Linear(torch.cat([q, k, v], dim=0)), self.position, self.hidden_size,
+                              self.num_heads, self.num_kv_heads, self.head_dim)
         self.o = Linear(tensors[p + "o_proj.weight"])
 
     def kv_cache_spec(self) -> KVCacheSpec:
@@ -64,37 +102,12 @@ class GQAAttention(Mixer):
         # the joined projection, the attention output and the output projection
         return (2 * self.num_heads + 2 * self.num_kv_heads) * self.head_dim + self.hidden_size
 
-    def _project_encode_cache(self, x, batch, kv):
-        """Q (position-encoded) for the attention kernel, with K and V of the step's tokens put
-        into the cache.  Few rows: one product does all of it in its epilogue; otherwise the
-        product is followed by the position encoding's own kernel.  Returns a tensor whose first
-        ``nq * d`` columns are the queries."""
-        tables = None
-        if self.qkv.fusable(x) and K.gemm_skinny_qkv_rope_supported(x.shape[0], self.hidden_size, self.head_dim):
-            tables = self.position.rotate_half_tables(x.device, self.head_dim)
-        if tables is None:
-            qkv = self.qkv(x)
-            self.position.apply_and_cache(qkv, batch.positions, self.num_heads, self.num_kv_heads,
-                                          self.head_dim, kv)
-            return qkv
-        write = kv is not None and kv.writes
-        q = torch.empty((x.shape[0], self.num_heads * self.head_dim), dtype=torch.bfloat16, device=x.device)
-        norm = {}
-        if isinstance(x, NormedRows):
-            norm = dict(sumsq=x.sumsq, norm_width=x.width, eps=x.eps)
-            x = x.scaled
-        K.gemm_skinny_qkv_rope(x, self.qkv.tiled, q, self.num_heads, self.num_kv_heads, self.head_dim,
-                               batch.positions, tables[0], tables[1],
-                               kv.k_cache if write else None, kv.v_cache if write else None,
-                               kv.slot_mapping if write else None, kv.page_size if kv is not None else 0, **norm)
-        return q
-
     def forward(self, x, ctx: MixerContext, tail: Optional[BranchTail] = None):
         """``x`` may be NormedRows (the input norm is then finished inside the QKV product); with
         a ``tail`` the output projection adds into the residual stream and prepares the next
         norm when the shapes allow, and NormedRows are returned instead of the plain output."""
         batch, kv = ctx.batch, ctx.kv
-        qkv = self._project_encode_cache(x, batch, kv)
+        qkv = self.qkv(x, batch, kv)
         out = torch.empty((x.shape[0], self.num_heads * self.head_dim), dtype=x.dtype, device=x.device)
         attn_ops.paged_attention(qkv, out, kv, batch, self.num_heads, self.num_kv_heads,
                                  self.head_dim, self.scale, self.window)

@@ -194,13 +194,21 @@ class FeedForward(Part):
 
 
 class Block(Part):
-    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, ffn_norm: Norm):
+    """The arrangement of a layer's parts.  ``norms`` holds the layer's norms by the names the
+    arrangement knows; ``NORM_NAMES`` lists the names a subclass needs (checked here)."""
+
+    NORM_NAMES: Tuple[str, ...] = ()
+
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward, norms: Dict[str, Norm]):
         super().__init__("")
         self.mixer, self.feed_forward = mixer, feed_forward
-        self.mixer_norm, self.ffn_norm = mixer_norm, ffn_norm
+        self.norms = dict(norms)
+        if set(self.norms) != set(self.NORM_NAMES):
+            raise ValueError(f"{type(self).__name__} arranges norms named {sorted(self.NORM_NAMES)}, "
+                             f"the layer gives {sorted(self.norms)}")
 
     def parts(self):
-        return (self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward)
+        return (*self.norms.values(), self.mixer, self.feed_forward)
 
     def forward(self, hidden: torch.Tensor, delta, ctx: MixerContext, next_norm: Optional[Norm] = None):
         """``delta`` is None, a plain branch output still to be added, or NormedRows prepared for
@@ -208,6 +216,8 @@ class Block(Part):
         block (the next block's first norm or the final norm)."""
         raise NotImplementedError
 
-    def first_norm(self) -> Norm:
-        """The norm that reads the residual stream first in this block."""
-        return self.mixer_norm
+    def first_norm(self) -> Optional[Norm]:
+        """The norm that reads the residual stream first in this block, if the block starts with
+        one: the block before may then prepare it in its last product.  ``None``: the stream is
+        handed over as it is."""
+        return None

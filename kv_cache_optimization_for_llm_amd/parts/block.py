@@ -18,6 +18,14 @@ from .base import Block, BranchTail, MixerContext, Norm, NormedRows
 @BLOCKS.register("pre_norm")
 class PreNormBlock(Block):
     graph_safe = True
+    NORM_NAMES = ("mixer", "feed_forward")
+
+    def __init__(self, mixer, feed_forward, norms):
+        super().__init__(mixer, feed_forward, norms)
+        self.mixer_norm, self.ffn_norm = self.norms["mixer"], self.norms["feed_forward"]
+
+    def first_norm(self) -> Norm:
+        return self.mixer_norm
 
     def forward(self, hidden: torch.Tensor, delta, ctx: MixerContext, next_norm: Optional[Norm] = None):
         # first norm: already prepared by the previous product, or add-and-normalise here

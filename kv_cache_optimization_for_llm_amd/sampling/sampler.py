@@ -133,12 +133,14 @@ class Sampler:
         if use_mask:
             seat_t = torch.tensor([r.seat if r.apply_penalty else -1 for r in rows],
                                   dtype=torch.int32).to(self.device)
+        # every token a request emits is marked in its mask row, by the launch that chooses it
+        mark_seat = None
+        if self.mask is not None:
+            mark_seat = torch.from_numpy(np.asarray([r.seat for r in rows], dtype=np.int32)).to(self.device)
         K.sample(logits, out, chunks=self.chunks, inv_temperature=inv_t, seed=self.seed, rng_key=key,
                  rng_step=step, penalty_mask=self.mask if use_mask else None, row_seat=seat_t,
-                 penalty=self.penalty)
+                 penalty=self.penalty, mark_mask=self.mask if mark_seat is not None else None,
+                 mark_seat=mark_seat)
         host[:n].copy_(out, non_blocking=True)
         event.record()
-        if self.mask is not None:
-            seats = torch.from_numpy(np.asarray([r.seat for r in rows], dtype=np.int32)).to(self.device)
-            K.mark_tokens(self.mask, seats, out)
         return PendingTokens(host, event, n)

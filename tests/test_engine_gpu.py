@@ -179,14 +179,17 @@ def test_random_workloads_emit_the_same_with_and_without_running_ahead(seed, mod
     from kv_cache_optimization_for_llm_amd.engine.runner import Runner
     rng = np.random.default_rng(100 + seed)
     cfg = TINY["A"][0]
-    eng = Engine(model_dirs["A"], EngineOptions(dtype="float32", max_seqs=3, max_seq_len=128, cache_tokens=160))
+    # room for the longest request alone (59 + 39 tokens) and little more: three live ones do not fit
+    eng = Engine(model_dirs["A"], EngineOptions(dtype="float32", max_seqs=3, max_seq_len=128, cache_tokens=112))
     requests = [([int(t) for t in rng.integers(0, cfg["vocab_size"], int(rng.integers(1, 60)))],
                  int(rng.integers(3, 40))) for _ in range(9)]
     probe = Runner(eng, ServeOptions(run_ahead=False, ignore_eos=True, temperature=0.8, sampling_seed=seed))
     for p, n in requests:
         probe.submit(p, n)
     seen = [ev.token for ev in probe.run_until_idle() if ev.kind == "token"]
-    eos = [int(t) for t in np.unique(seen)[:3]]               # ids that the requests do sample
+    ids_seen, counts = np.unique(seen, return_counts=True)
+    # ids that the requests do sample, but rarely: some requests stop early, most run on
+    eos = [int(t) for t in ids_seen[np.argsort(counts, kind="stable")[:3]]]
     results = {}
     for ahead in (False, True):
         runner = Runner(eng, ServeOptions(run_ahead=ahead, temperature=0.8, sampling_seed=seed,
@@ -207,7 +210,7 @@ def test_random_workloads_emit_the_same_with_and_without_running_ahead(seed, mod
     assert results[True][0] == results[False][0] and results[True][1] == results[False][1]
     assert set(results[True][1].values()) <= {"eos", "length"} and len(results[True][1]) == len(requests)
     assert not any(set(eos) & set(toks) for toks in results[True][0].values())
-    assert results[False][2] > 0 or results[True][2] > 0 or seed != 0     # pages do run out at least once
+    assert results[False][2] > 0 and results[True][2] > 0                 # pages do run out, for every seed
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -433,7 +433,7 @@ def test_choose_splits():
     assert choose_splits(1, 8, 100) == (1, 0)                     # too short to split
 
 
-@pytest.mark.parametrize("vocab", [1000, 128256])
+@pytest.mark.parametrize("vocab", [1000, 1001, 128256])
 def test_sampler_against_flat_cdf(vocab, gpu):
     """The reference's own check (python/sampling_reference.py:98-108): the chunked two-level walk
     picks the token of the flat CDF for the same draw; plus greedy ties and the penalty."""
@@ -447,7 +447,9 @@ def test_sampler_against_flat_cdf(vocab, gpu):
     inv_t = torch.tensor([1.0 / temps[i % 3] for i in range(rows)], device=gpu)
     key = torch.full((rows,), 7, dtype=torch.int32, device=gpu)
     step = torch.arange(rows, dtype=torch.int32, device=gpu)
-    K.sample(lg, out, chunks=128 if vocab > 4096 else 4, inv_temperature=inv_t, seed=1234, rng_key=key, rng_step=step)
+    # 1,001 tokens in 128 chunks of 8: the last two chunks are empty
+    chunks = {1000: 4, 1001: 128, 128256: 128}[vocab]
+    K.sample(lg, out, chunks=chunks, inv_temperature=inv_t, seed=1234, rng_key=key, rng_step=step)
     got = out.cpu().numpy()
     bad = 0
     for i in range(rows):
@@ -485,6 +487,13 @@ def test_sampler_against_flat_cdf(vocab, gpu):
     assert o2.cpu().tolist() == [20, 40]                  # 2/1.15 < 1.9 ; -1*1.15 < -1.1
     K.sample(pl, o2, chunks=8, penalty_mask=mask, row_seat=torch.tensor([-1, 0], dtype=torch.int32, device=gpu), penalty=1.15)
     assert o2.cpu().tolist() == [10, 30]                  # seat -1: no penalty; seat 0: nothing marked
+    # the launch that chooses a token marks it in the request's mask row (seat -1: nowhere); the
+    # mask it reads may be the mask it marks
+    K.sample(pl, o2, chunks=8, penalty_mask=mask, row_seat=torch.tensor([2, 3], dtype=torch.int32, device=gpu),
+             penalty=1.15, mark_mask=mask, mark_seat=torch.tensor([1, -1], dtype=torch.int32, device=gpu))
+    assert o2.cpu().tolist() == [20, 40]
+    marked = mask.nonzero().cpu().tolist()
+    assert marked == [[1, 20], [2, 10], [3, 30]]
 
 
 def test_sampler_distribution_and_boundaries(gpu):

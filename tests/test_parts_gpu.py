@@ -163,7 +163,7 @@ def test_pre_norm_block_adds_both_branches_to_the_stream(dtype, gpu):
                          position=PartSpec("rotary", dict(head_dim=d, max_positions=64, theta=10000.0)))
     ffn = SwiGLU("f.", hidden_size=H, intermediate_size=80)
     n1, n2 = RMSNorm("n1.", width=H, eps=1e-5), RMSNorm("n2.", width=H, eps=1e-5)
-    block = PreNormBlock(mixer, ffn, n1, n2)
+    block = PreNormBlock(mixer, ffn, {"mixer": n1, "feed_forward": n2})
     tensors = {}
     for i, part in enumerate(block.parts()):
         for k, s in part.tensor_specs().items():

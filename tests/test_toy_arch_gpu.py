@@ -17,15 +17,15 @@ import pytest
 import torch
 
 import plain_llama as plain
-from kv_cache_optimization_for_llm_amd.config.registry import (FEED_FORWARDS, MIXERS, POSITION_ENCODINGS,
+from kv_cache_optimization_for_llm_amd.config.registry import (BLOCKS, FEED_FORWARDS, MIXERS, POSITION_ENCODINGS,
                                                                register_architecture)
 from kv_cache_optimization_for_llm_amd.engine.batch import StepEntry
 from kv_cache_optimization_for_llm_amd.engine.engine import Engine, EngineOptions
 from kv_cache_optimization_for_llm_amd.models.spec import (LayerCall, LayerSpec, ModelSpec, PartSpec,
                                                            TensorSpec)
 from kv_cache_optimization_for_llm_amd.ops import kernels as K
-from kv_cache_optimization_for_llm_amd.parts.base import (FeedForward, Mixer, MixerContext, PositionEncoding,
-                                                          StateSpec)
+from kv_cache_optimization_for_llm_amd.parts.base import (Block, FeedForward, Mixer, MixerContext,
+                                                          PositionEncoding, StateSpec)
 from kv_cache_optimization_for_llm_amd.weights.random_init import write_random_model
 
 pytestmark = pytest.mark.gpu
@@ -138,7 +138,7 @@ def toy_layer(c, i, mixer):
     return LayerSpec(block=PartSpec("pre_norm"), mixer=mx,
                      feed_forward=PartSpec("swiglu", dict(prefix=p + "ffn.", hidden_size=c["hidden_size"],
                                                           intermediate_size=c["intermediate_size"])),
-                     mixer_norm=norm("n1"), ffn_norm=norm("n2"), prefix=p)
+                     norms={"mixer": norm("n1"), "feed_forward": norm("n2")}, prefix=p)
 
 
 def toy_spec(kind, mixers, order):
@@ -163,26 +163,66 @@ def routed_spec(c):
                                              head_dim=c["head_dim"], scale=1 / math.sqrt(c["head_dim"]), position=pos)),
         feed_forward=PartSpec("toy_routed", dict(prefix=p + "moe.", hidden_size=c["hidden_size"],
                                                  inner_size=c["intermediate_size"], experts=3)),
-        mixer_norm=norm("n1"), ffn_norm=norm("n2"), prefix=p)
+        norms={"mixer": norm("n1"), "feed_forward": norm("n2")}, prefix=p)
     return ModelSpec(architecture="ToyRoutedLM", hidden_size=c["hidden_size"], vocab_size=c["vocab_size"],
                      embedding_name="embed.weight", layers=(layer,), order=(LayerCall(0, 0),),
                      final_norm=PartSpec("rmsnorm", dict(prefix="final.", width=c["hidden_size"], eps=c["eps"])),
                      final_norm_prefix="final.", head_name="head.weight", max_positions=c["max_position_embeddings"])
 
 
+class ToySandwichBlock(Block):
+    """Another arrangement of a layer, with four norms: each branch is normalised before AND after,
+    ``h += post(branch(pre(h)))``.  It does not start with a norm that a product could prepare
+    (``first_norm`` stays None), so it takes the stream and a plain branch output as they are."""
+
+    graph_safe = True
+    NORM_NAMES = ("pre_mixer", "post_mixer", "pre_ffn", "post_ffn")
+
+    def forward(self, hidden, delta, ctx, next_norm=None):
+        if delta is not None:
+            K.residual_add(hidden, delta)
+        a = self.mixer.forward(self.norms["pre_mixer"].forward(hidden), ctx)
+        K.residual_add(hidden, self.norms["post_mixer"].forward(a))
+        f = self.feed_forward.forward(self.norms["pre_ffn"].forward(hidden), ctx)
+        return hidden, self.norms["post_ffn"].forward(f)
+
+
+SANDWICH = dict(embedding_scale=6.5, logit_scale=3.0, logit_softcap=3.0)
+
+
+def sandwich_spec(c):
+    layers = []
+    for i in range(2):
+        base = toy_layer(c, i, "gqa_attention")
+        p = base.prefix
+        norm = lambda n: PartSpec("rmsnorm", dict(prefix=p + n + ".", width=c["hidden_size"], eps=c["eps"]))
+        layers.append(LayerSpec(block=PartSpec("toy_sandwich"), mixer=base.mixer, feed_forward=base.feed_forward,
+                                norms={n: norm(n) for n in ToySandwichBlock.NORM_NAMES}, prefix=p))
+    return ModelSpec(architecture="ToySandwichLM", hidden_size=c["hidden_size"], vocab_size=c["vocab_size"],
+                     embedding_name="embed.weight", layers=tuple(layers), order=(LayerCall(0, 0), LayerCall(1, 1)),
+                     final_norm=PartSpec("rmsnorm", dict(prefix="final.", width=c["hidden_size"], eps=c["eps"])),
+                     final_norm_prefix="final.", head_name="head.weight", max_positions=c["max_position_embeddings"],
+                     **SANDWICH)
+
+
 @pytest.fixture(scope="module", autouse=True)
 def registered():
+    BLOCKS.register("toy_sandwich", ToySandwichBlock, replace=True)
+    register_architecture("ToySandwichLM", dict, sandwich_spec, replace=True)
     MIXERS.register("toy_decay", ToyDecayMixer, replace=True)
     POSITION_ENCODINGS.register("toy_neighbour_rotary", ToyNeighbourRotary, replace=True)
     FEED_FORWARDS.register("toy_routed", ToyRoutedFFN, replace=True)
     register_architecture("ToyRoutedLM", dict, routed_spec, replace=True)
     register_architecture("ToyStateLM", dict, toy_spec(
         "ToyStateLM", ["toy_decay", "gqa_attention"], [LayerCall(0, 0), LayerCall(1, 1)]), replace=True)
+    register_architecture("ToyStateOnlyLM", dict, toy_spec(
+        "ToyStateOnlyLM", ["toy_decay", "toy_decay"], [LayerCall(0, 0), LayerCall(1, 1)]), replace=True)
     register_architecture("ToyOrderLM", dict, toy_spec(
         "ToyOrderLM", ["gqa_attention", "gqa_attention"],
         [LayerCall(0, 0), LayerCall(1, 1), LayerCall(0, 2), LayerCall(1, 1, writes_cache=False)]), replace=True)
     yield
     MIXERS.unregister("toy_decay")
+    BLOCKS.unregister("toy_sandwich")
     POSITION_ENCODINGS.unregister("toy_neighbour_rotary")
     FEED_FORWARDS.unregister("toy_routed")
 
@@ -281,6 +321,56 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(dtype, tol, tmp_pa
     eng.cache.check()
 
 
+def test_a_model_that_keeps_no_keys_at_all(tmp_path, gpu):
+    """Two layers of the stateful toy mixer and no attention: the cache manager has no paged group,
+    only state slots; the pool is sized from nothing, admission asks no group for pages, and the
+    serving loop generates through the same scheduler."""
+    from kv_cache_optimization_for_llm_amd.engine.runner import Runner, ServeOptions
+    c = toy_config("ToyStateOnlyLM", "bfloat16")
+    d = write_random_model(str(tmp_path / "toy"), c, seed=17, gain=1.0)
+    W = load_plain(d)
+
+    def ref(toks):
+        h = W["embed.weight"][torch.tensor(toks)]
+        for i in range(2):
+            p = f"blocks.{i}."
+            u = plain.rms_norm(h, W[p + "n1.weight"], c["eps"]) @ W[p + "mix.in.weight"].t()
+            s, ys = torch.zeros(c["state_size"]), []
+            for t in range(len(toks)):
+                s = DECAY * s + u[t]
+                ys.append(s)
+            h = ref_ffn(c, W, p, h + torch.stack(ys) @ W[p + "mix.out.weight"].t())
+        return plain.rms_norm(h, W["final.weight"], c["eps"]) @ W["head.weight"].t()
+
+    eng = Engine(d, EngineOptions(dtype="float32", max_seqs=2, max_seq_len=96))       # no pool size given
+    assert eng.cache.groups == [] and sorted(eng.cache.state) == [0, 1]
+    rng = np.random.default_rng(4)
+    toks = [int(t) for t in rng.integers(0, 97, 40)]
+    want = ref(toks)
+    rows, i = [], 0
+    for n in (11, 1, 1, 20, 7):
+        rows.append(eng.step([StepEntry("p", toks[i:i + n], list(range(n)))]).cpu())
+        i += n
+    assert err(torch.cat(rows), want) <= 3e-5
+    eng.release("p")
+    # generation: three requests through two seats; greedy tokens are the plain model's
+    runner = Runner(eng, ServeOptions(ignore_eos=True, max_batch_tokens=32, chunk_size=16))
+    prompts = [[int(t) for t in rng.integers(0, 97, n)] for n in (5, 33, 18)]
+    ids = [runner.submit(p, 6) for p in prompts]
+    out = {i: [] for i in ids}
+    for ev in runner.run_until_idle():
+        if ev.kind == "token":
+            out[ev.request_id].append(ev.token)
+    for rid, p in zip(ids, prompts):
+        seq = list(p)
+        for tok in out[rid]:
+            assert tok == int(ref(seq)[-1].argmax())
+            seq.append(tok)
+        assert len(out[rid]) == 6
+    eng.cache.check()
+    assert eng.cache.free_seats == 2
+
+
 @pytest.mark.parametrize("dtype, tol", [("float32", 3e-5), ("bfloat16", 2e-2)])
 def test_run_order_names_a_layer_twice_and_shares_a_cache(dtype, tol, tmp_path, gpu):
     c = toy_config("ToyOrderLM", "bfloat16")
@@ -350,6 +440,55 @@ def test_another_position_encoding_and_a_routed_feed_forward(dtype, tol, tmp_pat
         i += n
     assert err(torch.cat(rows)[sure], ref[sure]) <= tol
     eng.cache.check()
+
+
+def ref_sandwich_model(c, W, toks):
+    T, eps = len(toks), c["eps"]
+    h = W["embed.weight"][torch.tensor(toks)] * SANDWICH["embedding_scale"]
+    for i in range(2):
+        p = f"blocks.{i}."
+        x = plain.rms_norm(h, W[p + "pre_mixer.weight"], eps)
+        q, k, v = ref_qkv(c, W, p, x, T)
+        o = plain.causal_gqa_attention(q, k, v, 1 / math.sqrt(c["head_dim"])).reshape(T, -1)
+        h = h + plain.rms_norm(plain.linear(o, W[p + "attn.o_proj.weight"]), W[p + "post_mixer.weight"], eps)
+        x = plain.rms_norm(h, W[p + "pre_ffn.weight"], eps)
+        f = plain.swiglu(x, W[p + "ffn.gate_proj.weight"], W[p + "ffn.up_proj.weight"], W[p + "ffn.down_proj.weight"])
+        h = h + plain.rms_norm(f, W[p + "post_ffn.weight"], eps)
+    raw = plain.rms_norm(h, W["final.weight"], eps) @ W["head.weight"].t()
+    logits = raw * SANDWICH["logit_scale"]
+    return SANDWICH["logit_softcap"] * torch.tanh(logits / SANDWICH["logit_softcap"]), float(raw.abs().max())
+
+
+@pytest.mark.parametrize("dtype, tol", [("float32", 3e-5), ("bfloat16", 2e-2)])
+def test_a_block_with_four_norms_and_constants_on_embedding_and_logits(dtype, tol, tmp_path, gpu):
+    """A layer arrangement with norms after its branches too, a multiplier on the embeddings, a
+    scale and a soft cap on the logits: a block class and a ModelSpec in this file, nothing changed
+    in the framework.  Decoded tokens run from captured graphs (the toy block says it may)."""
+    c = toy_config("ToySandwichLM", "bfloat16")
+    d = write_random_model(str(tmp_path / "toy"), c, seed=21, gain=1.0)
+    W = load_plain(d)
+    eng = Engine(d, EngineOptions(dtype=dtype, max_seqs=2, max_seq_len=128, cache_tokens=256))
+    assert (eng.graphs is not None) == (dtype == "bfloat16")
+    rng = np.random.default_rng(3)
+    toks = [int(t) for t in rng.integers(0, 97, 64)]
+    ref, raw_scale = ref_sandwich_model(c, W, toks)
+    assert ref.abs().max() > 0.8 * SANDWICH["logit_softcap"] and ref.abs().max() <= SANDWICH["logit_softcap"]
+    # A rounding error of the head's product is a fraction of ITS scale (raw_scale); the logit scale
+    # multiplies it, the cap (slope at most 1) does not shrink it, but the cap does shrink the scale
+    # the result is measured by, to logit_softcap.
+    tol = tol * max(1.0, SANDWICH["logit_scale"] * raw_scale / SANDWICH["logit_softcap"])
+    assert err(eng.step([StepEntry("w", toks, list(range(64)))]), ref) <= tol
+    rows, i = [], 0
+    for n in (9, 30, 2) + (1,) * 23:
+        rows.append(eng.step([StepEntry("p", toks[i:i + n], list(range(n)))]).cpu().clone())
+        i += n
+    assert i == 64 and err(torch.cat(rows), ref) <= tol
+    if eng.graphs is not None:
+        assert eng.graphs.replays > 0
+    # the arrangement is checked against the names it is given
+    with pytest.raises(ValueError) as e:
+        ToySandwichBlock(None, None, {"pre_mixer": None})
+    assert "post_ffn" in str(e.value)
 
 
 def test_garbage_of_an_earlier_engine_is_not_collected_inside_a_graph_capture(tmp_path, gpu):
