@@ -559,3 +559,78 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
                                           num_kv_heads, all_rows, stream);
     return KVA_OK;
 }
+
+// ---------------------------------------------------------------------------------------------
+// The same attention for callers that cannot allocate (declared in attention_static.h).
+//
+// kva_attention_mfma takes the partial results of its key splits in two buffers that the caller
+// allocates per call.  Here they live in one file-scope device array instead: each GPU the
+// library runs on holds its own copy, at its own address, until the process ends.  The array's
+// name is only a host-side handle; the address kernels can use is asked for once per device
+// (hipGetSymbolAddress, with that device current) and kept.
+#include "attention_static.h"
+#include <mutex>
+
+static __device__ __align__(256) unsigned char scratch[KVA_ATTENTION_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int STATIC_MAX_DEVICES = 64;
+std::mutex static_scratch_lock;
+unsigned char *static_scratch_of_device[STATIC_MAX_DEVICES] = {};
+}  // namespace
+
+// The device address of `scratch` on the current device, looked up at the first call there.
+static int static_scratch_address(unsigned char **out) {
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    KVA_REQUIRE(e == hipSuccess && device >= 0 && device < STATIC_MAX_DEVICES,
+                "attention_mfma_static: no current device (%s)", hipGetErrorString(e));
+    std::lock_guard<std::mutex> hold(static_scratch_lock);
+    if (static_scratch_of_device[device] == nullptr) {
+        unsigned char *ptr = nullptr;
+        e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+        KVA_REQUIRE(e == hipSuccess && ptr != nullptr,
+                    "attention_mfma_static: the scratch array has no address on device %d (%s)", device,
+                    hipGetErrorString(e));
+        static_scratch_of_device[device] = ptr;
+    }
+    *out = static_scratch_of_device[device];
+    return KVA_OK;
+}
+
+extern "C" long long kva_attention_mfma_static_scratch_bytes(int total_rows, int head_dim, int splits) {
+    if (splits <= 1) return 0;
+    // partial outputs [rows, splits, head_dim] fp32, then (max, sum) pairs [rows, splits, 2] fp32
+    const long long outputs = ((long long)total_rows * splits * head_dim * 4 + 255) / 256 * 256;
+    return outputs + (long long)total_rows * splits * 2 * 4;
+}
+
+extern "C" int kva_attention_mfma_static(void *out, const void *q, int q_row_stride, const void *k_cache,
+                                         const void *v_cache, const int *block_table, int max_blocks,
+                                         const int *item_meta, const int *item_entry, const int *item_row0,
+                                         int num_items, int row_tiles, const int *entry_seat,
+                                         const int *entry_q_start, const int *entry_start_pos, int total_rows,
+                                         int num_q_heads, int num_kv_heads, int head_dim, int page_size,
+                                         float scale, int window, int splits, int keys_per_split, int pair,
+                                         int all_rows, hipStream_t stream) {
+    KVA_REQUIRE(total_rows >= 0 && head_dim > 0 && splits >= 1, "attention_mfma_static: bad sizes");
+    float *part_o = nullptr, *part_ml = nullptr;
+    if (splits > 1) {
+        const long long need = kva_attention_mfma_static_scratch_bytes(total_rows, head_dim, splits);
+        KVA_REQUIRE(need <= (long long)KVA_ATTENTION_STATIC_SCRATCH_BYTES,
+                    "attention_mfma_static: %d rows x %d splits x head size %d need %lld bytes of scratch, the "
+                    "static array holds %lld; use fewer splits or kva_attention_mfma with buffers of your own",
+                    total_rows, splits, head_dim, need, (long long)KVA_ATTENTION_STATIC_SCRATCH_BYTES);
+        unsigned char *base = nullptr;
+        const int rc = static_scratch_address(&base);
+        if (rc != KVA_OK) return rc;
+        part_o = reinterpret_cast<float *>(base);
+        part_ml = reinterpret_cast<float *>(base + ((long long)total_rows * splits * head_dim * 4 + 255) / 256 * 256);
+        // Nothing in the array has to start at zero: every (row, split) partial that the merge reads
+        // is written by the attention launch before it, ranges without keys included.
+    }
+    return kva_attention_mfma(out, part_o, part_ml, q, q_row_stride, k_cache, v_cache, block_table, max_blocks,
+                              item_meta, item_entry, item_row0, num_items, row_tiles, entry_seat, entry_q_start,
+                              entry_start_pos, total_rows, num_q_heads, num_kv_heads, head_dim, page_size, scale,
+                              window, splits, keys_per_split, pair, all_rows, stream);
+}
