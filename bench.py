@@ -5,9 +5,13 @@
 
 Prints ONE JSON line.  ``value`` is decoded tokens per second of the default run: a batch of 8
 requests whose contexts end at 8,192 tokens, driven by the serving loop; a "step" is one decode
-step (scheduling, model forward over the paged cache, greedy sampling, token ids back on the host).  The same line carries the
-2,048-token prefill, the decode roofline (bytes the step has to read / time / HBM peak) and the
-batch-1 and batch-64 points.
+step (scheduling, model forward over the paged cache, greedy sampling, token ids back on the host).
+The same line carries the 2,048-token prefill; the decode roofline (bytes the step has to read /
+time / HBM peak, and against what a plain read stream gets from this GPU); ``points``: batch 1 and
+batch 64 at the same context and batches 1, 8 and 64 with 512-token prompts and 256 generated
+tokens, each with its step time, bytes and fraction of the HBM peak, and the serving loop at the
+3B and 8B layer sizes (mixed prompt lengths; paged against contiguous cache occupancy).
+``--kernel-classes`` adds device time per class of kernel.
 """
 import argparse
 import json
@@ -68,6 +72,11 @@ def main():
     ap.add_argument("--no-gemm-tuning", action="store_true",
                     help="leave the vendor GEMM library its own choice of algorithm (no timing at start-up)")
     ap.add_argument("--skip-points", action="store_true", help="only the default decode run and the prefill")
+    ap.add_argument("--skip-large", action="store_true",
+                    help="leave out the serving runs at the 3B and 8B layer sizes (about a minute together)")
+    ap.add_argument("--kernel-classes", action="store_true",
+                    help="also time one decode step and the prefill kernel class by kernel class (events around "
+                         "every launch, steps launched one by one instead of replayed from graphs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")
@@ -159,15 +168,93 @@ def main():
                "ms": round(p_ms, 3), "frac": round(flops / (p_ms * 1e-3) / (PEAK_TFLOPS["bf16"] * 1e12), 4)}
 
     points = {}
+
+    def add_point(name, batch, steps, seconds, mean_context):
+        """tok/s under the name itself; beside it the step's time, the bytes it has to read (every
+        weight once, the cache of the live requests) and the fraction of the HBM peak that is."""
+        ms = seconds / steps * 1e3
+        gb = (weight_bytes(cfg) + batch * mean_context * kv_bytes_per_token(cfg)) / 1e9
+        points[name] = round(batch * steps / seconds, 1)
+        points[name + "_ms"] = round(ms, 4)
+        points[name + "_gb"] = round(gb, 3)
+        points[name + "_frac"] = round(gb / (ms * 1e-3) / HBM_PEAK_GBS, 4)
+
     if not args.skip_points:
         for b in (1, 64):
             k = max(16, args.steps // 2)
-            d, _ = decode_run(b, k, 8, ctx)
-            points[f"decode_b{b}"] = round(b * k / d, 1)
+            d, c = decode_run(b, k, 8, ctx)
+            add_point(f"decode_b{b}", b, k, d, c)
         # the serving workload of the comparison: 512-token prompts, 256 generated tokens
         for b in (1, 8, 64):
-            d, _ = decode_run(b, 240, 8, 512 + 256)
-            points[f"decode_b{b}_p512_g256"] = round(b * 240 / d, 1)
+            d, c = decode_run(b, 240, 8, 512 + 256)
+            add_point(f"decode_b{b}_p512_g256", b, 240, d, c)
+
+    # what a plain read stream gets from this GPU's memory (the published peak is 8 TB/s)
+    from kv_cache_optimization_for_llm_amd.ops import kernels as K
+    probed_gbs = K.probe_read_bandwidth(dev)
+
+    kernel_ms = None
+    if args.kernel_classes:
+        graphs, portion_graphs = engine.graphs, engine.portion_graphs
+        engine.graphs = engine.portion_graphs = None           # launched one by one, so that events fit between
+        kernel_ms = {}
+        try:
+            # eight requests decoding at the context's end
+            ids = [f"k{i}" for i in range(args.batch)]
+            base = [int(t) for t in torch.randint(0, engine.vocab_size, (ctx - 8,), generator=gen)]
+            for rid in ids:
+                for lo in range(0, len(base), 4096):
+                    engine.step([StepEntry(rid, base[lo:lo + 4096], [])])
+            step = [StepEntry(rid, [5], [0]) for rid in ids]
+            engine.step(step)
+            with K.KernelClassTimer() as timer:
+                engine.step(step)
+            kernel_ms[f"decode_b{args.batch}_eager"] = timer.milliseconds()
+            for rid in ids:
+                engine.release(rid)
+            engine.step([StepEntry("kp0", prompt, [PREFILL_TOKENS - 1])])
+            engine.release("kp0")
+            with K.KernelClassTimer() as timer:
+                engine.step([StepEntry("kp1", prompt, [PREFILL_TOKENS - 1])])
+            kernel_ms[f"prefill_{PREFILL_TOKENS}_eager"] = timer.milliseconds()
+            engine.release("kp1")
+        finally:
+            engine.graphs, engine.portion_graphs = graphs, portion_graphs
+
+    # The serving loop at the layer sizes of the larger configurations (random weights, seeded
+    # uniform token ids): 32 requests with prompts of 128 to 4,096 tokens and 128 new tokens each,
+    # portions of 512, at the 3B sizes; 64 concurrent requests of 8,192 + 512 tokens at the 8B
+    # sizes, once over the paged cache and once over the contiguous one (what is reserved against
+    # what holds a token is the comparison the reference's paper makes).
+    if not args.skip_large:
+        import gc
+        from kv_cache_optimization_for_llm_amd.cli import sweep
+        del engine
+        gc.collect()
+        torch.cuda.empty_cache()
+        mixed = sweep.build_parser().parse_args(
+            ["--workload", "mixed", "--prompt-len", "4096", "--prompt-min", "128", "--new-tokens", "128",
+             "--chunk-size", "512", "--max-batch-tokens", "4096", "--tune-gemm"])
+        r = sweep.run_one(mixed, "3b", 32, "paged")
+        points.update({"serve_3b_mixed_b32_tok_s": round(r["tokens_emitted"] / r["wall_s"], 1),
+                       "serve_3b_mixed_b32_wall_s": r["wall_s"], "serve_3b_mixed_b32_prefill_tok_s": r["prefill_tok_s"],
+                       "serve_3b_mixed_b32_decode_tok_s": r["decode_tok_s"],
+                       "serve_3b_mixed_b32_decode_frac": r.get("decode_hbm_frac")})
+        gc.collect()
+        torch.cuda.empty_cache()
+        long = sweep.build_parser().parse_args(
+            ["--prompt-len", "8192", "--new-tokens", "512", "--max-batch-tokens", "8192", "--chunk-size", "2048",
+             "--reserve-policy", "pow2", "--tune-gemm"])
+        for mode in ("paged", "contiguous"):
+            r = sweep.run_one(long, "8b", 64, mode)
+            key = f"serve_8b_b64_ctx8704_{mode}"
+            points.update({key + "_decode_tok_s": r["decode_tok_s"], key + "_decode_frac": r.get("decode_hbm_frac"),
+                           key + "_prefill_tok_s": r["prefill_tok_s"], key + "_wall_s": r["wall_s"],
+                           key + "_kv_tokens_reserved": r["peak_kv_tokens_reserved"],
+                           key + "_kv_tokens_live": r["peak_kv_tokens_live"],
+                           key + "_reserved_over_live": r["reserved_over_live"]})
+            gc.collect()
+            torch.cuda.empty_cache()
 
     out = {
         "metric": f"decode tok/s at batch {args.batch} (context {ctx}), Llama-3.2-1B shape", "value": round(value, 1),
@@ -183,9 +270,12 @@ def main():
                    "rope": "llama3 factor 32", "sampling": "greedy on device"},
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "bytes_gb": round(step_bytes / 1e9, 3),
+                     "probed_read_stream": round(probed_gbs, 1), "frac_of_probed": round(achieved / probed_gbs, 4)},
         "points": points,
     }
+    if kernel_ms is not None:
+        out["kernel_ms"] = kernel_ms
     print(json.dumps(out))
     return 0
 

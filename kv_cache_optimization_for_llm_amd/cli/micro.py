@@ -4,6 +4,7 @@
     python -m kv_cache_optimization_for_llm_amd.cli.micro attention --batch 8 --context 8192 --splits 32
     python -m kv_cache_optimization_for_llm_amd.cli.micro gemm --rows 8 --shape gate_up
     python -m kv_cache_optimization_for_llm_amd.cli.micro prompt --tokens 8192 --portion 512
+    python -m kv_cache_optimization_for_llm_amd.cli.micro stream --megabytes 8.4,67,525
 
 The reference keeps a harness that runs its attention kernels alone over made-up caches
 (``micro/harness.cuh``); this is the same idea for the kernels here.  Sizes default to the
@@ -158,6 +159,38 @@ def prompt(args) -> None:
           f"{args.tokens / best:9.0f} tok/s", flush=True)
 
 
+def stream(args) -> None:
+    """The floor for kernels that stream weights: a kernel that only reads N bytes once, each call
+    on another buffer so that every byte comes from memory, launched one by one and from a graph
+    of 200 such kernels (as decode steps run)."""
+    import torch
+    from ..ops import kernels as K
+
+    dev = torch.device("cuda:0")
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    print(f"plain read stream over 2 GiB: {K.probe_read_bandwidth(dev):.0f} GB/s")
+    for mb in [float(x) for x in args.megabytes.split(",")]:
+        n = int(mb * 1e6) // 16 * 16
+        copies = max(2, min(200, int(3e9 // n)))
+        bufs = [torch.zeros(n, dtype=torch.uint8, device=dev) for _ in range(copies)]
+        for wgs in [int(w) for w in args.workgroups.split(",")]:
+            eager = _time([(lambda b=b: K.stream_read(b, wgs, sink)) for b in bufs], 200)
+            g = torch.cuda.CUDAGraph()
+            torch.cuda.synchronize()
+            with torch.cuda.graph(g):
+                for i in range(200):
+                    K.stream_read(bufs[i % copies], wgs, sink)
+            g.replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(5):
+                g.replay()
+            torch.cuda.synchronize()
+            in_graph = (time.perf_counter() - t0) / (5 * 200) * 1e6
+            print(f"read {mb:g} MB, {wgs} workgroups of 256: {eager:.2f} us launched one by one, "
+                  f"{in_graph:.2f} us in a graph = {n / in_graph / 1e6:.2f} TB/s")
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description="one kernel in a loop")
     sub = ap.add_subparsers(dest="what", required=True)
@@ -185,9 +218,15 @@ def main(argv=None) -> int:
     pr.add_argument("--layers", type=int, default=0, help="fewer layers than the 16 of the shape")
     pr.add_argument("--reps", type=int, default=4)
     pr.add_argument("--no-graphs", action="store_true")
+    st = sub.add_parser("stream", help="a kernel that only reads: the floor for weight-streaming kernels")
+    st.add_argument("--megabytes", default="8.4,12.6,33.5,67,525", help="comma list of sizes to read")
+    st.add_argument("--workgroups", default="256,1024,2048")
     args = ap.parse_args(argv)
     if args.what == "prompt":
         prompt(args)
+        return 0
+    if args.what == "stream":
+        stream(args)
         return 0
     if args.what == "attention":
         if args.kernel == "lds" and not args.tokens:

@@ -16,6 +16,9 @@ reached.
 Workloads: ``uniform`` (every prompt ``--prompt-len`` long) and ``mixed`` (prompt lengths uniform
 in ``[--prompt-min, --prompt-len]``, the shape of the reference's trace-driven runs without their
 datasets).  ``--layers`` runs fewer layers than the shape has (the line then names both numbers).
+With ``--out FILE`` the sweep can be resumed: a run whose line the file already holds is skipped
+unless ``--force`` is given (the reference's driver skips finished runs the same way,
+``sweep.py:270-288``).
 """
 from __future__ import annotations
 
@@ -159,7 +162,38 @@ def run_one(args, shape: str, batch: int, mode: str) -> dict:
     return out
 
 
-def main(argv=None) -> int:
+RUN_KEY = ("shape", "layers_asked", "batch", "cache_mode", "reserve_policy", "workload", "prompt_len",
+           "prompt_min", "new_tokens_each", "page_size", "max_seqs", "cache_tokens_asked", "max_batch_tokens",
+           "chunk_size", "seed")
+
+
+def run_key(args, shape: str, batch: int, mode: str) -> dict:
+    """What identifies a run: a line with the same key in the output file is that run's result."""
+    return {"shape": shape, "layers_asked": args.layers, "batch": batch, "cache_mode": mode,
+            "reserve_policy": args.reserve_policy if mode == "contiguous" else None, "workload": args.workload,
+            "prompt_len": args.prompt_len, "prompt_min": args.prompt_min if args.workload == "mixed" else None,
+            "new_tokens_each": args.new_tokens, "page_size": args.page_size, "max_seqs": args.max_seqs,
+            "cache_tokens_asked": args.cache_tokens, "max_batch_tokens": args.max_batch_tokens,
+            "chunk_size": args.chunk_size, "seed": args.seed}
+
+
+def finished_runs(path: str) -> list:
+    """Keys of the runs whose lines a file of earlier results holds (a cut-off last line is ignored)."""
+    import os
+    done = []
+    if path and os.path.isfile(path):
+        with open(path) as f:
+            for line in f:
+                try:
+                    rec = json.loads(line)
+                except json.JSONDecodeError:
+                    continue
+                if isinstance(rec, dict) and rec.get("requests_done") is not None:
+                    done.append({k: rec.get(k) for k in RUN_KEY})
+    return done
+
+
+def build_parser() -> argparse.ArgumentParser:
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("--shapes", default="1b",
                     help="comma list of " + ", ".join(SHAPES) + ", or paths of config.json files")
@@ -182,16 +216,29 @@ def main(argv=None) -> int:
     ap.add_argument("--no-graphs", action="store_true", help="launch every step's kernels one by one")
     ap.add_argument("--no-run-ahead", action="store_true")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--out", default=None, help="also append the lines to this file")
+    ap.add_argument("--out", default=None, help="also append the lines to this file; a run whose line is "
+                                                 "there already is skipped (the sweep can be resumed)")
+    ap.add_argument("--force", action="store_true", help="run again what the --out file already holds")
+    return ap
+
+
+def main(argv=None) -> int:
+    ap = build_parser()
     args = ap.parse_args(argv)
     import os
+    done = [] if args.force else finished_runs(args.out)
     for shape in args.shapes.split(","):
         if shape not in SHAPES and not os.path.isfile(shape):
             ap.error(f"shape {shape!r} is neither one of {', '.join(SHAPES)} nor a config.json file")
     for shape in args.shapes.split(","):
         for mode in args.cache_modes.split(","):
             for batch in (int(b) for b in args.batches.split(",")):
-                line = json.dumps(run_one(args, shape, batch, mode))
+                key = run_key(args, shape, batch, mode)
+                if key in done:
+                    print(f"[sweep] {shape} batch {batch} {mode}: already in {args.out}, skipped (--force runs it again)",
+                          file=sys.stderr, flush=True)
+                    continue
+                line = json.dumps({**run_one(args, shape, batch, mode), **key})
                 print(line, flush=True)
                 if args.out:
                     with open(args.out, "a") as f:

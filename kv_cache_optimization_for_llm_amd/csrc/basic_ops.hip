@@ -237,6 +237,35 @@ extern "C" int kva_residual_add(void *hidden, const void *delta, long long n, in
 }
 
 // ---------------------------------------------------------------------------------------
+// A probe, not a part of the model: reads `count` 16-byte units once (non-temporal loads, four in
+// flight per lane) and stores nothing.  Its time is the floor for any kernel that has to read as
+// many bytes, and bytes / time the memory bandwidth this GPU gives a plain stream.
+__global__ void __launch_bounds__(256) stream_read_kernel(const uint4 *__restrict__ p, size_t count,
+                                                          unsigned *__restrict__ sink) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    unsigned acc = 0;
+    for (; i + 3 * stride < count; i += 4 * stride) {
+        const uint4 a = load_streamed_u4(p + i), b = load_streamed_u4(p + i + stride);
+        const uint4 c = load_streamed_u4(p + i + 2 * stride), d = load_streamed_u4(p + i + 3 * stride);
+        acc ^= a.x ^ b.y ^ c.z ^ d.w;
+    }
+    for (; i < count; i += stride) acc ^= load_streamed_u4(p + i).x;
+    // practically never true; it keeps the loads from being dropped
+    if (acc == 0x9E3779B9u && threadIdx.x == 255 && sink != nullptr) *sink = acc;
+}
+
+extern "C" int kva_stream_read(const void *p, long long bytes, int workgroups, void *sink, hipStream_t stream) {
+    KVA_REQUIRE(workgroups >= 1 && workgroups <= 65535, "stream_read: 1..65535 workgroups");
+    KVA_REQUIRE(bytes >= 0 && p != nullptr && ((uintptr_t)p % 16) == 0, "stream_read: a 16-byte aligned range is needed");
+    if (bytes < 16) return KVA_OK;
+    hipLaunchKernelGGL(stream_read_kernel, dim3(workgroups), dim3(256), 0, stream, (const uint4 *)p,
+                       (size_t)(bytes / 16), (unsigned *)sink);
+    KVA_CHECK_LAUNCH("stream_read");
+    return KVA_OK;
+}
+
+// ---------------------------------------------------------------------------------------
 // x <- x * scale, and then, with cap > 0, x <- cap * tanh(x / cap): the constants a model may put
 // on its embeddings and on its logits.  fp32 arithmetic, rounded to the storage type.
 template <typename T>

@@ -141,10 +141,22 @@ class Model:
         head = tensors[self.spec.head_name] if self.spec.head_name is not None else self.embedding
         self.head = Linear(head)
 
+    @staticmethod
+    def block_linears(block) -> List[Linear]:
+        """Every Linear the block's parts hold as an attribute, or inside an attribute that wraps
+        one as ``.linear``."""
+        out = []
+        for part in block.parts():
+            for v in vars(part).values():
+                if isinstance(v, Linear):
+                    out.append(v)
+                elif isinstance(getattr(v, "linear", None), Linear):
+                    out.append(v.linear)
+        return out
+
     def linears(self) -> List[Linear]:
-        """Every Linear a block's parts hold as an attribute, in layer order."""
-        return [v for b in self.blocks for part in b.parts() for v in vars(part).values()
-                if isinstance(v, Linear)]
+        """Every Linear of every block, in layer order."""
+        return [lin for b in self.blocks for lin in self.block_linears(b)]
 
     def tune_products(self, row_counts, say=None) -> List[dict]:
         """For every row count, has the vendor GEMM library's algorithms timed for each shape of

@@ -116,6 +116,30 @@ def residual_add(hidden: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
     return hidden
 
 
+def stream_read(x: torch.Tensor, workgroups: int, sink: torch.Tensor) -> None:
+    """A probe: reads ``x`` once and stores nothing (``sink``: any int32 device tensor, practically
+    never written).  Its time is the floor of any kernel that reads as many bytes."""
+    check(hip_lib().kva_stream_read(_dev(x, "x"), x.numel() * x.element_size(), int(workgroups),
+                                    _dev(sink, "sink", torch.int32), _stream()), "stream_read")
+
+
+def probe_read_bandwidth(device, megabytes: int = 2048, workgroups: int = 2048, reps: int = 5) -> float:
+    """GB/s of a plain read stream over a buffer far larger than every cache, best of ``reps``."""
+    x = torch.empty(megabytes << 20, dtype=torch.uint8, device=device)
+    x.zero_()
+    sink = torch.zeros(4, dtype=torch.int32, device=device)
+    stream_read(x, workgroups, sink)
+    best = 0.0
+    for _ in range(reps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        stream_read(x, workgroups, sink)
+        b.record()
+        b.synchronize()
+        best = max(best, x.numel() / (a.elapsed_time(b) * 1e-3) / 1e9)
+    return best
+
+
 def scale_softcap(x: torch.Tensor, scale: float, cap: float = 0.0) -> torch.Tensor:
     """In place: ``x *= scale``, then with ``cap > 0`` ``x = cap * tanh(x / cap)``."""
     if cap < 0:
@@ -623,3 +647,62 @@ def normed_rows_finish(scaled: torch.Tensor, sumsq: torch.Tensor, norm_width: in
         _dev(out, "out"), _dev(scaled, "scaled"), _dev(sumsq, "sumsq", torch.float32), sumsq.shape[1],
         rows, _opt(row_idx, "row_idx", torch.int32), width, float(eps), _stream()), "normed_rows_finish")
     return out
+
+
+# --------------------------------------------------------------------------------------
+# Measurement: device time per class of kernel, from events around every launch.
+KERNEL_CLASSES = {
+    "embed_gather": "embedding", "rmsnorm": "norm", "normed_rows_finish": "norm",
+    "residual_add": "elementwise", "scale_softcap": "elementwise", "cast": "elementwise",
+    "silu_mul": "activation", "rope_kv_write": "rope + cache write",
+    "attention_rowwise": "attention", "attention_mfma": "attention", "attention_lds": "attention",
+    "gemm_nt_f32": "gemm fp32", "gemm_vendor": "gemm (vendor library)",
+    "gemm_skinny": "gemm (few rows)", "gemm_skinny_qkv_rope": "gemm (few rows)",
+    "sample": "sampling", "mark_tokens": "sampling",
+}
+
+
+class KernelClassTimer:
+    """``with KernelClassTimer() as t: ...`` brackets every kernel entry point of this module
+    with a pair of events on the current stream; ``t.milliseconds()`` then gives the device time
+    per class of kernel (the reference times its attention micro-benchmark the same way,
+    ``micro/main_paged.cu:102-114``).  Launches one by one - a step replayed from a graph shows
+    nothing here - so a class's time includes the gaps between its launches and their
+    predecessors; it tells where a step's time goes, not how fast a kernel can be."""
+
+    def __init__(self):
+        self._marks = []
+        self._saved = {}
+
+    def __enter__(self):
+        module = globals()
+        for name, cls in KERNEL_CLASSES.items():
+            fn = module[name]
+            self._saved[name] = fn
+            module[name] = self._wrap(fn, cls)
+        return self
+
+    def _wrap(self, fn, cls):
+        marks = self._marks
+
+        def timed(*args, **kwargs):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            try:
+                return fn(*args, **kwargs)
+            finally:
+                b.record()
+                marks.append((cls, a, b))
+        return timed
+
+    def __exit__(self, *exc):
+        globals().update(self._saved)
+        self._saved = {}
+        return False
+
+    def milliseconds(self) -> dict:
+        torch.cuda.synchronize()
+        out: dict = {}
+        for cls, a, b in self._marks:
+            out[cls] = out.get(cls, 0.0) + a.elapsed_time(b)
+        return {k: round(v, 4) for k, v in sorted(out.items(), key=lambda kv: -kv[1])}

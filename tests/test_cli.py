@@ -28,6 +28,24 @@ def test_checksum_is_order_sensitive():
     assert checksum([1, 2]) == (1 * 1000003 + 2) & 0xFFFFFFFF
 
 
+def test_a_sweep_knows_which_of_its_runs_a_results_file_already_holds(tmp_path):
+    """Resuming (reference sweep.py:270-288): a run is identified by its parameters; a finished
+    run's line in the --out file stands for it, a cut-off line or another run's line does not."""
+    from kv_cache_optimization_for_llm_amd.cli import sweep
+    out = tmp_path / "runs.jsonl"
+    args = sweep.build_parser().parse_args(["--out", str(out), "--prompt-len", "64", "--new-tokens", "8"])
+    key = sweep.run_key(args, "1b", 8, "paged")
+    assert sweep.finished_runs(str(out)) == []                      # no file yet
+    out.write_text(json.dumps({**key, "requests_done": 8, "decode_tok_s": 1.0}) + "\n"
+                   + json.dumps({**sweep.run_key(args, "1b", 64, "paged"), "requests_done": 64})[:40] + "\n")
+    done = sweep.finished_runs(str(out))
+    assert key in done and len(done) == 1                           # the cut-off line does not count
+    assert sweep.run_key(args, "1b", 64, "paged") not in done
+    assert sweep.run_key(args, "1b", 8, "contiguous") not in done   # the same batch in the other mode is another run
+    other = sweep.build_parser().parse_args(["--out", str(out), "--prompt-len", "128", "--new-tokens", "8"])
+    assert sweep.run_key(other, "1b", 8, "paged") not in done       # and so is another prompt length
+
+
 @pytest.mark.gpu
 def test_served_tokens_are_the_same_in_both_cache_modes(sharp_model_dirs, tmp_path, gpu):
     """The reference's cross-build gate (bench.py:226-237): the paged and the contiguous engine
@@ -72,6 +90,11 @@ def test_sweep_reports_both_cache_modes_on_a_small_shape(sharp_model_dirs, tmp_p
     paged, contiguous = lines[1], lines[3]
     assert paged["reserved_over_live"] < contiguous["reserved_over_live"]
     assert paged["pages_reused"] > 0                  # six requests through three seats
+    # started again with the same file, nothing is run again: every run's line is there already
+    assert sweep.main(["--shapes", cfg, "--batches", "3,6", "--cache-modes", "paged,contiguous", "--prompt-len", "40",
+                       "--prompt-min", "5", "--workload", "mixed", "--new-tokens", "12", "--max-seqs", "3",
+                       "--reserve-policy", "pow2", "--out", str(out)]) == 0
+    assert len(out.read_text().splitlines()) == 4
 
 
 @pytest.mark.gpu
