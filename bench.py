@@ -101,7 +101,8 @@ def main():
     tune_rows = [] if args.no_gemm_tuning else [PREFILL_TOKENS] + [b for b in {args.batch, max_batch} if b > 16]
     engine = Engine(None, EngineOptions(dtype="bfloat16", page_size=PAGE, cache_tokens=pool,
                                         max_seqs=max_batch, max_seq_len=cfg["max_position_embeddings"],
-                                        max_batch_tokens=32768, gemm_tune_rows=tune_rows),
+                                        max_batch_tokens=32768, max_logit_rows=max(64, args.batch),
+                                        gemm_tune_rows=tune_rows),
                     config_dict=cfg, random_seed=0)
     dev = engine.device
     gen = torch.Generator().manual_seed(0)

@@ -134,6 +134,7 @@ def main(argv=None) -> int:
     engine = Engine(args.model_dir, EngineOptions(
         dtype=args.dtype, cache_mode=args.cache_mode, page_size=args.page_size, max_seqs=args.max_seqs,
         max_seq_len=args.max_seq_len, cache_tokens=args.cache_tokens, max_batch_tokens=args.max_batch_tokens,
+        max_logit_rows=args.max_seqs,         # one sampled token per request and step
         gemm_tune_rows=([args.max_seqs] if args.max_seqs > 16 else []) if args.gemm_tune_rows == "auto"
         else [int(r) for r in args.gemm_tune_rows.split(",") if r.strip()]))
     runner = Runner(engine, ServeOptions(

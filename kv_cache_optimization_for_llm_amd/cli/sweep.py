@@ -80,7 +80,7 @@ def run_one(args, shape: str, batch: int, mode: str) -> dict:
     engine = Engine(None, EngineOptions(dtype="bfloat16", cache_mode=mode, page_size=args.page_size,
                                         cache_tokens=pool, max_seqs=seats, max_seq_len=longest,
                                         use_graphs=not args.no_graphs,
-                                        max_batch_tokens=max(8192, args.max_batch_tokens),
+                                        max_batch_tokens=max(8192, args.max_batch_tokens), max_logit_rows=seats,
                                         gemm_tune_rows=[seats] if args.tune_gemm and seats > 16 else []),
                     config_dict=cfg, random_seed=args.seed)
     runner = Runner(engine, ServeOptions(ignore_eos=True, max_batch_tokens=args.max_batch_tokens,

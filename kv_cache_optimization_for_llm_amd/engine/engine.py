@@ -49,6 +49,8 @@ class EngineOptions:
     max_seqs: int = 8                   # seats (reference: MAX_SEQUENCES)
     max_seq_len: Optional[int] = None   # longest request (default: max_position_embeddings)
     max_batch_tokens: int = 8192        # most tokens one step may bring (reference: MAX_BATCH_TOKENS)
+    max_logit_rows: Optional[int] = None  # most places a step may want logits at (default: max_batch_tokens;
+                                          # a server that samples one token per request needs max_seqs)
     use_graphs: bool = True             # replay decode-only steps, and steps with prompt portions whose
                                         # shape comes back, as HIP graphs (bfloat16 engine)
     # Row counts (tokens per step) for which the vendor GEMM library's algorithms are timed at
@@ -127,6 +129,9 @@ class Engine:
         if options.max_batch_tokens < 1:
             raise EngineError("max_batch_tokens must be at least 1")
         self.max_batch_tokens = int(options.max_batch_tokens)
+        self.max_logit_rows = int(options.max_logit_rows or options.max_batch_tokens)
+        if self.max_logit_rows < 1:
+            raise EngineError("max_logit_rows must be at least 1")
         groups, states = self.model.cache_requirements()
         if options.cache_tokens:
             num_pages = (options.cache_tokens + options.page_size - 1) // options.page_size
@@ -144,11 +149,18 @@ class Engine:
                 num_pages = pool_pages_from_memory(
                     free_bytes - tables, page_bytes, page_size=options.page_size, max_seqs=options.max_seqs,
                     max_seq_len=max_seq_len, margin_bytes=options.memory_margin_bytes,
-                    step_bytes=self.model.step_activation_bytes(self.max_batch_tokens))
+                    step_bytes=self.model.step_activation_bytes(self.max_batch_tokens, self.max_logit_rows))
         self.cache = CacheManager(groups, states, page_size=options.page_size, num_pages=num_pages,
                                   max_seqs=options.max_seqs, max_seq_len=max_seq_len,
                                   mode=options.cache_mode, device=self.device, dtype=self.dtype)
         self.max_seq_len = max_seq_len
+        # The step's arena (reference: one block of scratch for MAX_BATCH_TOKENS rows,
+        # base/src/engine.cu:62-122): what the largest step needs for its intermediate results is
+        # taken from the device once, here, and handed to torch's caching allocator, which cuts
+        # every later step's tensors out of this block instead of asking the device again.
+        self.step_arena_bytes = self.model.step_activation_bytes(self.max_batch_tokens, self.max_logit_rows)
+        arena = torch.empty(self.step_arena_bytes, dtype=torch.uint8, device=self.device)
+        del arena
         self._seat_of: Dict[object, int] = {}
         self.steps_run = 0
         # tokens that stay on the device between steps: a sampler leaves its output here and the
@@ -283,6 +295,10 @@ class Engine:
         if total > self.max_batch_tokens:
             raise EngineError(f"a step of {total} tokens is larger than max_batch_tokens "
                               f"({self.max_batch_tokens}); cut the prompts into smaller portions")
+        wanted = sum(len(w) for w in wants)
+        if wanted > self.max_logit_rows:
+            raise EngineError(f"a step that wants logits at {wanted} places is larger than max_logit_rows "
+                              f"({self.max_logit_rows})")
         seat_of, cache = self._seat_of, self.cache
         for e in entries:
             seat = seat_of.get(e.request_id)

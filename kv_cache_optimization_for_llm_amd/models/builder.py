@@ -107,15 +107,16 @@ class Model:
             groups.setdefault(slot_spec[slot], []).append(slot)
         return list(groups.items()), states
 
-    def step_activation_bytes(self, tokens: int) -> int:
+    def step_activation_bytes(self, tokens: int, logit_rows: Optional[int] = None) -> int:
         """Upper estimate of the device memory one step of ``tokens`` tokens needs beside weights
         and cache: the residual stream and a branch output, twice the widest layer's intermediate
-        results (one layer's are freed while the next one's are made) and fp32 logits for every
-        token.  Used when the cache pool is sized from leftover memory."""
+        results (one layer's are freed while the next one's are made) and fp32 logits at
+        ``logit_rows`` places (default: every token).  The engine reserves this much once, and
+        leaves it out when it sizes the cache pool from leftover memory."""
         elem = torch.empty((), dtype=self.dtype).element_size()
         widest = max((sum(part.activation_elements() for part in b.parts()) for b in self.blocks), default=0)
-        per_token = (3 * self.spec.hidden_size + 2 * widest) * elem + 4 * self.spec.vocab_size
-        return int(tokens) * per_token
+        rows = int(tokens if logit_rows is None else logit_rows)
+        return int(tokens) * (3 * self.spec.hidden_size + 2 * widest) * elem + rows * 4 * self.spec.vocab_size
 
     def graph_safe(self) -> bool:
         """Whether every part may be captured into a HIP graph."""

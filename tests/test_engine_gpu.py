@@ -544,11 +544,16 @@ def test_pool_comes_from_free_memory_and_a_step_is_bounded(gpu):
     from conftest import MID_F
     from kv_cache_optimization_for_llm_amd.engine.engine import EngineError
     cfg = dict(MID_F, max_position_embeddings=131072)
+    torch.cuda.empty_cache()               # what earlier tests left in torch's cache is free memory too
     free, _ = torch.cuda.mem_get_info(gpu)
     page_bytes = 2 * 2 * 2 * 128 * 16 * 2                      # layers x (K, V) x kv heads x head size x tokens x bf16
     # as on a device with 3 GiB to spare: the margin takes the rest
     eng = Engine(None, EngineOptions(dtype="bfloat16", max_seqs=64, memory_margin_bytes=free - 3 * 2 ** 30,
-                                     max_batch_tokens=256, use_graphs=False), config_dict=cfg, random_seed=1)
+                                     max_batch_tokens=256, max_logit_rows=4, use_graphs=False),
+                 config_dict=cfg, random_seed=1)
+    # the largest step's intermediate results have their memory already (taken once, kept by torch's allocator)
+    assert eng.step_arena_bytes == eng.model.step_activation_bytes(256, 4) > 256 * 640 * 2
+    assert torch.cuda.memory_reserved(gpu) - torch.cuda.memory_allocated(gpu) >= eng.step_arena_bytes
     pool_bytes = eng.cache.num_pages * page_bytes
     assert eng.max_seq_len == 131072 and eng.cache.num_pages < 64 * 131072 // 16
     assert 2 * 2 ** 30 < pool_bytes <= 3 * 2 ** 30
@@ -560,6 +565,9 @@ def test_pool_comes_from_free_memory_and_a_step_is_bounded(gpu):
     with pytest.raises(EngineError) as e:
         eng.step([StepEntry("a", list(range(200)), []), StepEntry("b", list(range(57)), [])])
     assert "max_batch_tokens" in str(e.value)
+    with pytest.raises(EngineError) as e:
+        eng.step([StepEntry("a", list(range(8)), [0, 1, 2, 3, 4])])
+    assert "max_logit_rows" in str(e.value)
     assert not eng.has_request("b") and eng.length("a") == 256 and eng.cache.free_seats == 63
     eng.cache.check()
     del eng

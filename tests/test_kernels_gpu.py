@@ -61,6 +61,24 @@ def test_rmsnorm_plain_fused_and_gathered(dtype, width, gpu):
     # a weight stored in 32-bit is used in 32-bit
     K.rmsnorm(x.to(gpu), w.float().to(gpu), eps, out)
     close(out, plain.rms_norm(x.float(), w.float(), eps), dt, "rmsnorm fp32 weight", tol16=5e-3)
+    # many rows (a prompt portion): the same three forms
+    R = 515
+    X, D = rnd(R, width, dtype=dt, seed=5), rnd(R, width, dtype=dt, seed=6)
+    O = torch.full((R, width), float("nan"), dtype=dt, device=gpu)
+    H = X.clone().to(gpu)
+    K.rmsnorm(H, w.to(gpu), eps, O)
+    close(O, plain.rms_norm(X.float(), w.float(), eps), dt, "rmsnorm, many rows", tol16=5e-3)
+    assert torch.equal(H.cpu(), X)
+    K.rmsnorm(H, w.to(gpu), eps, O, delta=D.to(gpu))
+    S = (X.float() + D.float()).to(dt)
+    assert torch.equal(H.cpu(), S)
+    close(O, plain.rms_norm(S.float(), w.float(), eps), dt, "add+rmsnorm, many rows", tol16=5e-3)
+    idx = torch.arange(R - 1, -1, -1, dtype=torch.int32)
+    idx[7] = idx[8]
+    H = X.clone().to(gpu)
+    K.rmsnorm(H, w.float().to(gpu), eps, O, delta=D.to(gpu), row_idx=idx.to(gpu))
+    assert torch.equal(H.cpu(), X)
+    close(O, plain.rms_norm(S.float()[idx.long()], w.float(), eps), dt, "gather+add+rmsnorm, many rows", tol16=5e-3)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
