@@ -38,6 +38,28 @@ def _time(calls, reps: int) -> float:
     return (time.perf_counter() - t0) / reps * 1e6
 
 
+def _time_in_graph(calls, reps: int) -> float:
+    """Microseconds per call when the calls run from a HIP graph, one after the other, as the
+    kernels of a decode step do (no host launch cost between them)."""
+    import torch
+    for f in calls:
+        f()
+    n = max(len(calls), min(reps, 64))
+    g = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(g):
+        for i in range(n):
+            calls[i % len(calls)]()
+    g.replay()
+    torch.cuda.synchronize()
+    rounds = max(1, reps // n)
+    t0 = time.perf_counter()
+    for _ in range(rounds):
+        g.replay()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / (rounds * n) * 1e6
+
+
 def attention(args) -> None:
     import numpy as np
     import torch
@@ -86,7 +108,7 @@ def attention(args) -> None:
         pair = bool(args.tokens) and len(meta) * nkv >= 2048 and not args.no_pair
         calls = [lambda c=c: K.attention_mfma(qkv, nq * d, out, c[0], c[1], table, ent, row0, seat, qs, sp, nq, nkv,
                                               d, scale, 0, splits, per, tiles, pair, meta_d) for c in caches]
-    us = _time(calls, args.reps)
+    us = _time_in_graph(calls, args.reps) if args.graph else _time(calls, args.reps)
     flops = sum(4.0 * nq * d * n * (2 * s + n + 1) / 2 for s, n in entries)
     kv_bytes = sum((s + n) * nkv * d * 4 for s, n in entries)
     what = f"prompt of {args.tokens}" if args.tokens else f"batch {args.batch} at context {args.context}, {splits} splits"
@@ -207,6 +229,7 @@ def main(argv=None) -> int:
     a.add_argument("--reps", type=int, default=20)
     a.add_argument("--no-pair", action="store_true", help="wave kernel: never give a wave two items")
     a.add_argument("--pair", action="store_true", help="workgroup kernel: a workgroup takes item i and item n-1-i")
+    a.add_argument("--graph", action="store_true", help="time the calls inside a HIP graph (no host launch cost)")
     g = sub.add_parser("gemm")
     g.add_argument("--shape", choices=sorted(GEMM_SHAPES), default="gate_up")
     g.add_argument("--rows", type=int, default=8)

@@ -10,9 +10,23 @@ import torch
 
 from . import kernels as K
 
-# wavefronts wanted in flight: 256 compute units, a few waves each
+# Wavefronts wanted in flight when keys are split.  Prompt portions (two row tiles per wavefront,
+# keys shared through L2): a few per compute unit.  Decoded tokens stream their keys once and pay
+# 4-5 us for the merge kernel as soon as there is more than one split: with three wavefronts for
+# every two compute units they are not split at all, below that until there are four per unit,
+# in ranges of at least 64 keys (128 for long contexts).  Whole decode steps of the 1B shape
+# (8 kv heads, head size 64) in one process, ms per step, old rule (2,048 wavefronts, ranges of at
+# least 128 keys) against this one:
+#   contexts of 768: batch 1 0.890 -> 0.845, batch 8 0.915 -> 0.911, batch 32 1.384 -> 1.370,
+#   batch 64 1.583 -> 1.510 (one range, no merge); contexts of 8,192: batch 1 0.919 -> 0.919,
+#   batch 8 1.298 -> 1.269 (16 ranges instead of 32), batch 64 4.13 -> 4.10
 _TARGET_WAVES = 2048
 _MIN_KEYS_PER_SPLIT = 128
+_TARGET_WAVES_DECODE = 1024
+_UNSPLIT_WAVES_DECODE = 384
+_MIN_KEYS_PER_SPLIT_DECODE = 64
+_LONG_CONTEXT_DECODE = 2048         # above it a range holds at least _MIN_KEYS_PER_SPLIT keys
+
 # wide items (two row tiles per wave) are used when they alone give this many waves
 _WIDE_MIN_WAVES = 1024
 _PAIR_MIN_WAVES = 2048      # two items per wavefront once that still leaves a wavefront per SIMD
@@ -39,14 +53,22 @@ def _cut_keys(want: int, max_context: int, max_splits: int) -> tuple:
     return (splits, per) if splits > 1 else (1, 0)
 
 
-def choose_splits(num_items: int, num_kv_heads: int, max_context: int, max_splits: int = None) -> tuple:
+def choose_splits(num_items: int, num_kv_heads: int, max_context: int, max_splits: int = None,
+                  decoding: bool = False) -> tuple:
     """(splits, keys_per_split) for the matrix-core kernel; never more splits than the kernels
-    and their merge take (``max_splits``, by default what the library says)."""
+    and their merge take (``max_splits``, by default what the library says).  ``decoding``: the
+    items are decoded tokens (one row tile each)."""
     if max_splits is None:
         max_splits = K.attention_max_splits()
     waves = max(1, num_items * num_kv_heads)
-    want = max(1, _TARGET_WAVES // waves)
-    most = max(1, (max_context + _MIN_KEYS_PER_SPLIT - 1) // _MIN_KEYS_PER_SPLIT)
+    target, least = _TARGET_WAVES, _MIN_KEYS_PER_SPLIT
+    if decoding:
+        if waves >= _UNSPLIT_WAVES_DECODE:
+            return 1, 0
+        target = _TARGET_WAVES_DECODE
+        least = _MIN_KEYS_PER_SPLIT_DECODE if max_context <= _LONG_CONTEXT_DECODE else _MIN_KEYS_PER_SPLIT
+    want = max(1, target // waves)
+    most = max(1, (max_context + least - 1) // least)
     return _cut_keys(min(want, most), max_context, max_splits)
 
 
@@ -88,7 +110,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
 
     def decoded(which):
         items = batch.attention_items(group, 1, which)
-        splits, per = choose_splits(items[0].shape[0], num_kv_heads, batch.max_context)
+        splits, per = choose_splits(items[0].shape[0], num_kv_heads, batch.max_context, decoding=True)
         wave_kernel(items, 1, splits, per, False, which)
 
     if batch.max_q_len * group <= 16:

@@ -404,8 +404,9 @@ def test_attention_of_one_decoded_token_over_a_very_long_context(nkv, ctx, gpu):
     key ranges than the kernels take and must stop at their limit.  One key at a range's edge is
     made to dominate, so a range that is dropped or counted twice shows."""
     nq, d, page = 2 * nkv, 64, 16
-    splits, per = choose_splits(1, nkv, ctx)
-    assert splits == K.attention_max_splits() == 256 and splits * per >= ctx
+    splits, per = choose_splits(1, nkv, ctx, decoding=True)
+    assert K.attention_max_splits() == 256 and splits * per >= ctx
+    assert splits == 256           # 1,024 wavefronts are wanted: more splits than the kernels take
     far = per * 101 - 1                                   # the last key of range 100
     g = torch.Generator().manual_seed(ctx + nkv)
     k = torch.randn(ctx, nkv, d, generator=g) * 0.1
@@ -449,6 +450,13 @@ def test_choose_splits():
     s, per = choose_splits(1, 8, 8192)
     assert s > 16 and per % 32 == 0 and s * per >= 8192 and (s - 1) * per < 8192
     assert choose_splits(1, 8, 100) == (1, 0)                     # too short to split
+    # decoded tokens: not split at all when they alone give three wavefronts per two compute units,
+    # else until there are four per unit, in ranges of at least 64 keys (128 in long contexts)
+    assert choose_splits(64, 8, 1024, decoding=True) == (1, 0) == choose_splits(48, 8, 8192, decoding=True)
+    assert choose_splits(32, 8, 1024, decoding=True) == (4, 256)
+    assert choose_splits(1, 8, 1024, decoding=True) == (16, 64)
+    assert choose_splits(1, 8, 8192, decoding=True) == (64, 128)
+    assert choose_splits(8, 8, 8192, decoding=True) == (16, 512)
 
 
 @pytest.mark.parametrize("vocab", [1000, 1001, 128256])

@@ -15,6 +15,7 @@ def test_key_splits_never_exceed_what_the_kernels_take(nkv, items, context):
     """Few kv heads, one or two decoding requests and a long context ask for many splits; the
     policy must stop at the kernels' limit, and its ranges must still cover every key."""
     for splits, per in (choose_splits(items, nkv, context, KERNEL_MAX_SPLITS),
+                        choose_splits(items, nkv, context, KERNEL_MAX_SPLITS, decoding=True),
                         choose_lds_splits(items * nkv, context, KERNEL_MAX_SPLITS)):
         assert 1 <= splits <= KERNEL_MAX_SPLITS
         if splits > 1:
