@@ -95,7 +95,7 @@ def main():
     ctx = args.context
     cfg["max_position_embeddings"] = max(cfg["max_position_embeddings"], ctx)      # a longer --context
     # room for max_batch requests at the context, one more page each for the tokens decoded
-    pool = max_batch * (ctx + 2 * PAGE)
+    pool = max(max_batch * (ctx + 2 * PAGE), PREFILL_TOKENS + PAGE)      # and room for the prefill's prompt
     # the vendor library's algorithms are timed once, at start-up, for the row counts whose
     # products go to it here: the prefill's 2,048 tokens and decode batches above 16
     tune_rows = [] if args.no_gemm_tuning else [PREFILL_TOKENS] + [b for b in {args.batch, max_batch} if b > 16]

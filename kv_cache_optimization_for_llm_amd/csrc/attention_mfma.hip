@@ -52,7 +52,7 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
     constexpr int NKS = D / KSTEP;
     constexpr int NDT = D / 16;                      // 16-wide tiles of the value dimension
 
-    const int lane = threadIdx.x, r = lane & 15, g = lane >> 4;
+    const int lane = threadIdx.x & (KVA_WAVE - 1), r = lane & 15, g = lane >> 4;   // (a workgroup may hold several wavefronts)
     const int G = num_q_heads / num_kv_heads;
 
     // Everything about the item is uniform over the wavefront: keep it in scalar registers.  Every

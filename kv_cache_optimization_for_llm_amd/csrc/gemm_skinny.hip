@@ -830,16 +830,29 @@ extern "C" int kva_gemm_skinny_qkv_rope(void *q_out, int ldq, const void *X, con
     a.k_cache = (bf16_t *)k_cache; a.v_cache = (bf16_t *)v_cache;
     a.nq = nq; a.nkv = nkv; a.head_dim = head_dim; a.page_size = page_size;
     int groups = a.N / 32;
-    a.half = choose_half_tiles(groups);
+    // More than 16 tokens: workgroups of several tile groups share X through LDS, as in
+    // kva_gemm_skinny (17 / 32 / 48 / 64 tokens of the 1B shape: 12.3 / 12.8 / 16.2 / 20.1 us -> 11.5 /
+    // 11.8 / 14.2 / 16.3 us), without half tiles.
+    const bool xl = M > 16 && groups >= 2;
+    a.half = xl ? 0 : choose_half_tiles(groups);
     if (a.half) groups *= 2;
-    const int kw = choose_k_waves(groups, K, 2);
+    int kw = choose_k_waves(groups, K, 2);
+    int groups_per_wg = kw >= 4 ? 1 : 4 / kw;
+    if (xl) {
+        kw = kw < 4 ? kw : 4;
+        groups_per_wg = kw == 4 ? 2 : 4;
+    }
     a.k_waves = kw;
-    const int groups_per_wg = kw >= 4 ? 1 : 4 / kw;
     const int waves = kw * groups_per_wg;
     size_t lds = kw > 1 ? (size_t)waves * 2 * 64 * 4 * sizeof(float) : 0;
+    if (xl) {
+        const size_t stage = (size_t)kw * 2 * ((M + 15) / 16 * 16) * 128;
+        lds = lds > stage ? lds : stage;
+    }
     KVA_REQUIRE(lds <= 64 * 1024, "gemm_skinny_qkv_rope: LDS buffer of %zu bytes does not fit", lds);
     dim3 grid((groups + groups_per_wg - 1) / groups_per_wg), block(64 * waves);
-    launch_mt<2, EPI_ROPE>(a, grid, block, lds, stream);
+    if (xl) launch_xl<2, EPI_ROPE>(a, grid, block, lds, stream);
+    else launch_mt<2, EPI_ROPE>(a, grid, block, lds, stream);
     KVA_CHECK_LAUNCH("gemm_skinny_qkv_rope");
     return KVA_OK;
 }

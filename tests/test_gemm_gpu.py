@@ -133,7 +133,7 @@ def test_wide_matrices_give_a_wave_several_tiles(gpu):
         assert (out.cpu().double() - want).abs().max() <= 1e-5 * want.abs().max()
 
 
-@pytest.mark.parametrize("m", [1, 7, 16, 35])
+@pytest.mark.parametrize("m", [1, 7, 16, 17, 35, 64])
 @pytest.mark.parametrize("nq, nkv, d, page, k", [(4, 2, 32, 16, 64), (6, 1, 96, 8, 160), (3, 3, 64, 4, 2048),
                                                  (32, 8, 64, 16, 2048)])
 @pytest.mark.parametrize("rotate, normed", [(True, False), (True, True), (False, False)])
