@@ -37,7 +37,8 @@
 #include <type_traits>
 #include <math.h>
 
-template <int D, int RT, bool FAST>
+// STREAM: keys and values are loaded with the non-temporal hint (see load_block).
+template <int D, int RT, bool FAST, bool STREAM>
 __device__ __forceinline__ void
 attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
                       const bf16_t *__restrict__ q, int q_row_stride,
@@ -146,10 +147,11 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
     const uint32_t k_lane = (uint32_t)(r * D + g * (KSTEP / 4)) * 2u;          // bytes
     const uint32_t v_lane = (uint32_t)(r * 16 + 4 * g) * 2u;                   // bytes
     constexpr uint32_t v_tile_stride = 16u * 16u * 2u;                         // 16 value dims
-    // One row tile per item is how decoded tokens (and short portions) run: their keys and values
-    // are read once per step, by this wave alone, and go past the caches.  Prompt items share
-    // theirs with the other row tiles of the request, through L2.
-    constexpr bool STREAM = RT == 1;
+    // STREAM: keys and values go past the caches (non-temporal loads).  Right for decoded tokens
+    // whose keys and values are read once per step and are too many to still be in the
+    // memory-side cache at the next step; prompt items share theirs with the other row tiles of
+    // the request through L2, and the keys of a few short requests (a few tens of megabytes over
+    // all layers) survive a step in the memory-side cache if they are allowed in.
     auto load_block = [&](BlockFrags &f, int kstart) {
         if constexpr (FAST) {
             // the index is uniform: said so explicitly, the lookups are scalar loads (both issued
@@ -361,7 +363,7 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
 // same heads' keys and values.  With `pair`, a wavefront takes item w and then item n-1-w of the
 // list: the caller orders the list by the number of keys an item visits (most first), so every
 // wavefront gets about the same work - rows late in a prompt visit many keys, early rows few.
-template <int D, int RT, bool FAST>
+template <int D, int RT, bool FAST, bool STREAM>
 __global__ void __launch_bounds__(KVA_WAVE)
 attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
                       const bf16_t *__restrict__ q, int q_row_stride,
@@ -374,12 +376,12 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
                       int page_size, float scale, int window, int splits, int keys_per_split, int num_items, int pair) {
     const int kvh = blockIdx.x % num_kv_heads, split = blockIdx.z;
     const int w = blockIdx.x / num_kv_heads;
-    attention_item<D, RT, FAST>(out, part_o, part_ml, q, q_row_stride, k_cache, v_cache, block_table, max_blocks,
+    attention_item<D, RT, FAST, STREAM>(out, part_o, part_ml, q, q_row_stride, k_cache, v_cache, block_table, max_blocks,
                                 item_meta, item_entry, item_row0, entry_seat, entry_q_start, entry_start_pos, num_q_heads,
                                 num_kv_heads, page_size, scale, window, splits, keys_per_split, w, kvh, split);
     const int other = num_items - 1 - w;
     if (pair && other > w)
-        attention_item<D, RT, FAST>(out, part_o, part_ml, q, q_row_stride, k_cache, v_cache, block_table, max_blocks,
+        attention_item<D, RT, FAST, STREAM>(out, part_o, part_ml, q, q_row_stride, k_cache, v_cache, block_table, max_blocks,
                                     item_meta, item_entry, item_row0, entry_seat, entry_q_start, entry_start_pos, num_q_heads,
                                     num_kv_heads, page_size, scale, window, splits, keys_per_split, other, kvh, split);
 }
@@ -507,7 +509,7 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
                                   const int *entry_start_pos, int total_rows, int num_q_heads,
                                   int num_kv_heads, int head_dim, int page_size, float scale, int window,
                                   int splits, int keys_per_split, int pair, int all_rows,
-                                  hipStream_t stream) {
+                                  int keep_cached, hipStream_t stream) {
     KVA_REQUIRE(num_items >= 0 && num_q_heads > 0 && num_kv_heads > 0 && max_blocks > 0,
                 "attention_mfma: bad sizes");
     KVA_REQUIRE(num_q_heads % num_kv_heads == 0, "attention_mfma: %d query heads is not a multiple of %d kv heads",
@@ -529,8 +531,8 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
     const int waves_x = pair ? (num_items + 1) / 2 : num_items;
     dim3 grid(waves_x * num_kv_heads, 1, splits), block(KVA_WAVE);
     const bool fast = page_size == 16;
-#define LAUNCH(DD, RR, FF)                                                                      \
-    hipLaunchKernelGGL((attention_mfma_kernel<DD, RR, FF>), grid, block, 0, stream, (bf16_t *)out, \
+#define LAUNCH(DD, RR, FF, SS)                                                                  \
+    hipLaunchKernelGGL((attention_mfma_kernel<DD, RR, FF, SS>), grid, block, 0, stream, (bf16_t *)out, \
                        part_o, part_ml, (const bf16_t *)q, q_row_stride, (const bf16_t *)k_cache, \
                        (const bf16_t *)v_cache, block_table, max_blocks, item_meta, item_entry,  \
                        item_row0,                                                               \
@@ -539,9 +541,11 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
 #define CASE(DD, WIDE)                                                                          \
     case DD:                                                                                    \
         if (row_tiles == 1) {                                                                   \
-            if (fast) LAUNCH(DD, 1, true); else LAUNCH(DD, 1, false);                           \
+            if (fast && keep_cached) LAUNCH(DD, 1, true, false);                                \
+            else if (fast) LAUNCH(DD, 1, true, true);                                           \
+            else LAUNCH(DD, 1, false, false);                                                   \
         } else {                                                                                \
-            if (fast) LAUNCH(DD, WIDE, true); else LAUNCH(DD, WIDE, false);                     \
+            if (fast) LAUNCH(DD, WIDE, true, false); else LAUNCH(DD, WIDE, false, false);       \
         }                                                                                       \
         break
     switch (head_dim) {
@@ -632,5 +636,5 @@ extern "C" int kva_attention_mfma_static(void *out, const void *q, int q_row_str
     return kva_attention_mfma(out, part_o, part_ml, q, q_row_stride, k_cache, v_cache, block_table, max_blocks,
                               item_meta, item_entry, item_row0, num_items, row_tiles, entry_seat, entry_q_start,
                               entry_start_pos, total_rows, num_q_heads, num_kv_heads, head_dim, page_size, scale,
-                              window, splits, keys_per_split, pair, all_rows, stream);
+                              window, splits, keys_per_split, pair, all_rows, /*keep_cached=*/0, stream);
 }

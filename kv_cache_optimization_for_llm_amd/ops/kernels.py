@@ -312,7 +312,8 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
                    entry_start_pos: torch.Tensor, num_q_heads: int, num_kv_heads: int, head_dim: int,
                    scale: float, window: int = 0, splits: int = 1, keys_per_split: int = 0,
                    row_tiles: int = 1, pair: bool = False,
-                   item_meta: Optional[torch.Tensor] = None, covers_all_rows: bool = True) -> torch.Tensor:
+                   item_meta: Optional[torch.Tensor] = None, covers_all_rows: bool = True,
+                   keep_cached: bool = False) -> torch.Tensor:
     """bf16 matrix-core attention over the paged cache.  Items are (entry, first query row) pairs
     of ``16 * row_tiles`` query rows each, row = token_in_step * (nq / nkv) + head_in_group.
     With ``pair`` one wavefront takes item i and item n-1-i of the list (give the list ordered by
@@ -320,7 +321,9 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
     ``[items, 8]`` int32 (q_start, q_len, start_pos, seat, row0, 0, 0, 0 per item) saves the
     kernel the chain of lookups item -> entry -> entry arrays; it must say the same as they do.
     ``covers_all_rows=False``: the items are only some of the step's rows (the others belong to
-    another launch) and a split merge must leave those alone."""
+    another launch) and a split merge must leave those alone.  ``keep_cached`` (items of one row
+    tile): keys and values are loaded through the caches instead of past them - for the few
+    short contexts that are still in the memory-side cache when the next step reads them."""
     tokens = out.shape[0]
     if out.dtype != torch.bfloat16 or q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16:
         raise KernelError("attention_mfma: bfloat16 only")
@@ -349,7 +352,8 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
         int(row_tiles), _dev(entry_seat, "entry_seat", torch.int32), _dev(entry_q_start, "entry_q_start", torch.int32),
         _dev(entry_start_pos, "entry_start_pos", torch.int32), tokens * num_q_heads, num_q_heads,
         num_kv_heads, head_dim, k_cache.shape[2], float(scale), int(window), int(splits),
-        int(keys_per_split), 1 if pair else 0, 1 if covers_all_rows else 0, _stream()), "attention_mfma")
+        int(keys_per_split), 1 if pair else 0, 1 if covers_all_rows else 0, 1 if keep_cached else 0,
+        _stream()), "attention_mfma")
     return out
 
 

@@ -263,6 +263,12 @@ def test_attention_mfma(nq, nkv, d, page, window, splits, wide, pair, gpu):
                      dev["entry_seat"], dev["q_start"], dev["start_pos"], nq, nkv, d, scale, window,
                      splits, per, tiles, pair, meta.to(gpu))
     assert torch.equal(out2, out)
+    # keys and values loaded through the caches instead of past them: the same bits
+    out4 = torch.full_like(out, float("nan"))
+    K.attention_mfma(dev["qkv"], stride, out4, dev["kc"], dev["vc"], dev["table"], ent, row0,
+                     dev["entry_seat"], dev["q_start"], dev["start_pos"], nq, nkv, d, scale, window,
+                     splits, per, tiles, pair, keep_cached=True)
+    assert torch.equal(out4, out)
     # a launch over some of the entries only (the others belong to another launch of the same
     # step): their rows are right, every other row keeps what it held, split merge included
     keep = (ent.cpu() % 2 == 0)
