@@ -114,6 +114,25 @@ __device__ inline float quad_rows_max(float x) {
     return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 
+// Sum over the 16 lanes of a row (lanes 16 i .. 16 i + 15), every one of them getting it: four
+// rotations within the row, done by the data-parallel-primitive path of the vector ALU.
+template <int ROTATE>
+__device__ inline float row16_rotated(float v) {
+    return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x120 | ROTATE, 0xf, 0xf, false));
+}
+__device__ inline float row16_sum(float v) {
+    v += row16_rotated<8>(v);
+    v += row16_rotated<4>(v);
+    v += row16_rotated<2>(v);
+    v += row16_rotated<1>(v);
+    return v;
+}
+
+// wave_sum without a trip through LDS: a chain of about a hundred cycles instead of six shuffles
+// of about a hundred each, for kernels that are as short as that chain.  The additions are in
+// another order than wave_sum's.
+__device__ inline float wave_sum_valu(float v) { return quad_rows_sum(row16_sum(v)); }
+
 // Sum over a whole workgroup of `nwaves` wavefronts; `scratch` holds at least nwaves floats.
 // Every thread gets the result.  The order of the additions is fixed.
 __device__ inline float block_sum(float v, float *scratch, int nwaves) {

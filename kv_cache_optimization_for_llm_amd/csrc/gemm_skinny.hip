@@ -14,7 +14,7 @@
 // (NTW = 1, 2 or 4: wide matrices give a wave several n-tiles so that a loaded X fragment is
 // used several times), so W is read once whatever M is.  K is split over `k_waves` wavefronts of
 // a workgroup (partials summed through LDS in a fixed order) so that narrow matrices still put
-// about 2048 waves on the 256 compute units.
+// about 2048 waves on the 256 compute units.  A wave keeps up to 8 steps of its K range in flight.
 //
 // A column of the result depends only on its own token's row of X, and with at most 16 rows the
 // order of its sum does not depend on M: bitwise the same result in any batch that small.
@@ -164,7 +164,7 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
     // issued here, ahead of the main loop, and (for up to 32 tokens) their values are only added
     // after it, so this wave starts streaming W as early as the others; with more token tiles
     // there are no registers to hold them and they are added at once.
-    constexpr int DV = (MT == 1 && NTW <= 2) ? 16 : ((MT == 1 || (MT == 2 && NTW <= 2)) ? 8 : 0);   // vectors of 4 sums held per token tile
+    constexpr int DV = (MT == 1 && NTW <= 2) ? 8 : ((MT == 1 || (MT == 2 && NTW <= 2)) ? 4 : 0);   // vectors of 4 sums held per token tile
     float4 dv[MT][DV > 0 ? DV : 1];
     int dv_end[MT];
     float ssum[MT];
@@ -261,12 +261,7 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
     }
 
     // ---- the main loop.  Rows of X past M are read from row 0 instead (their columns of the
-    // result are never stored), so the loop body has no branch.  One step per turn and wave: what
-    // bounds these products is how much a compute unit can have in flight (about 32 KiB, or
-    // 33 GB/s per unit at the latency seen here), which its 16 waves reach with one step each;
-    // chunks of 2-8 steps with all loads up front were measured equal for the per-layer matrices
-    // and 10-20 % slower for the vocabulary-sized one.  What counts is that every compute unit
-    // has a workgroup.
+    // result are never stored), so the loop body has no branch.
     if constexpr (XL) {
         // More than 16 tokens: every wave needs MT fragments of X per fragment of W, and loading
         // them per wave makes X (from L2, in half-used cache lines) the larger stream.  Here the
@@ -382,19 +377,58 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
         }
         __syncthreads();                                        // the sums below reuse the buffer
     } else if (group_ok) {
+        // S steps are in flight at any time: all of a chunk's loads are asked for before its first
+        // product, and as soon as a step's product has used its registers they are asked for
+        // again, for the same step of the next chunk.  (A plain loop of load, wait, product - what
+        // the compiler makes of `for k` here, its trip count being a vector register's - costs one
+        // trip to memory per step, 0.43 us each.)  What is left after the whole chunks goes in
+        // chunks of S/2, S/4, .. 1 steps, each with its loads up front.
+        constexpr int S = NTW + MT <= 2 ? 8 : ((MT == 1 && NTW == 2) ? 4 : (NTW * MT >= 12 ? 1 : 2));   // by registers
         const size_t xstep = a.x_tiled ? 16 : 1;               // a step of 32 columns is 4 chunks of 16 rows x 8
-#pragma unroll 8
-        for (int k = kbeg; k < kend; k += 32) {
-            GFrag8 w[NTW];
+        const int kb = __builtin_amdgcn_readfirstlane(kbeg), ke = __builtin_amdgcn_readfirstlane(kend);
+        const int steps = (ke - kb) / 32, full = steps / S;
+        GFrag8 w[S][NTW], x[S][MT];
+        auto ask = [&](int st, int k) {
 #pragma unroll
-            for (int t = 0; t < NTW; ++t) w[t].u4 = load_streamed_u4(wp[t] + (size_t)k * 16);
+            for (int t = 0; t < NTW; ++t) w[st][t].u4 = load_streamed_u4(wp[t] + (size_t)k * 16);
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                GFrag8 x;
-                x.u4 = *reinterpret_cast<const uint4 *>(xr[mt] + (size_t)k * xstep);
+            for (int mt = 0; mt < MT; ++mt) x[st][mt].u4 = *reinterpret_cast<const uint4 *>(xr[mt] + (size_t)k * xstep);
+        };
+        auto multiply = [&](int st) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                 for (int t = 0; t < NTW; ++t)
-                    acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[t].v, x.v, acc[t][mt], 0, 0, 0);
+                    acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[st][t].v, x[st][mt].v, acc[t][mt], 0, 0, 0);
+        };
+        int k = kb;
+        if (full > 0) {
+#pragma unroll
+            for (int st = 0; st < S; ++st) ask(st, k + 32 * st);
+            for (int c = 1; c < full; ++c) {
+                k += 32 * S;
+#pragma unroll
+                for (int st = 0; st < S; ++st) {
+                    multiply(st);
+                    ask(st, k + 32 * st);
+                    __builtin_amdgcn_sched_barrier(0);        // in this order: S - 1 steps stay in flight
+                }
+            }
+#pragma unroll
+            for (int st = 0; st < S; ++st) multiply(st);
+            k += 32 * S;
+        }
+        const int left = steps - full * S;
+#pragma unroll
+        for (int part = S / 2; part >= 1; part /= 2) {
+            if (left & part) {
+#pragma unroll
+                for (int st = 0; st < (S > 1 ? S / 2 : 1); ++st)
+                    if (st < part) ask(st, k + 32 * st);
+#pragma unroll
+                for (int st = 0; st < (S > 1 ? S / 2 : 1); ++st)
+                    if (st < part) multiply(st);
+                k += 32 * part;
             }
         }
     }

@@ -638,6 +638,102 @@ def gemm_skinny_sumsq_parts(n: int) -> int:
     return int(hip_lib().kva_gemm_skinny_sumsq_parts(int(n)))
 
 
+def gemv_supported(m: int, n: int, k: int) -> bool:
+    return bool(hip_lib().kva_gemv_supported(int(m), int(n), int(k)))
+
+
+def gemv_sumsq_parts(n: int, k: int) -> int:
+    """Partial sums of squares per token that :func:`gemv` writes with its residual epilogue."""
+    return int(hip_lib().kva_gemv_sumsq_parts(int(n), int(k)))
+
+
+def gemv(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor], swiglu: bool = False, *,
+         sumsq: Optional[torch.Tensor] = None, norm_width: int = 0, eps: float = 0.0,
+         hidden: Optional[torch.Tensor] = None, next_weight: Optional[torch.Tensor] = None,
+         scaled_out: Optional[torch.Tensor] = None, sumsq_out: Optional[torch.Tensor] = None):
+    """out = x @ W^T for one or two rows of x over the plain row-major bf16 weight ``w`` [N, K]
+    (fp32 accumulation).  The options are :func:`gemm_skinny`'s: ``swiglu`` for a joined
+    ``[gate; up]`` matrix, ``sumsq`` to finish the input's norm, ``hidden`` / ``next_weight`` /
+    ``scaled_out`` / ``sumsq_out`` [M, :func:`gemv_sumsq_parts`] for the residual epilogue."""
+    if x.dim() != 2 or w.dim() != 2 or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 \
+            or x.shape[1] != w.shape[1] or not w.is_contiguous() or x.stride(1) != 1:
+        raise KernelError(f"gemv: bf16 x {tuple(x.shape)} does not fit a row-major bf16 weight {tuple(w.shape)}")
+    m, k = x.shape
+    n = w.shape[0]
+    lib = hip_lib()
+    if sumsq is not None and (sumsq.dim() != 2 or sumsq.shape[0] != m or norm_width <= 0):
+        raise KernelError("gemv: sumsq must be [M, parts] and norm_width positive")
+    parts = sumsq.shape[1] if sumsq is not None else 0
+    norm = (_opt(sumsq, "sumsq", torch.float32), parts, int(norm_width), float(eps))
+    if hidden is not None:
+        if swiglu or out is not None:
+            raise KernelError("gemv: the residual epilogue has no other output")
+        p_out = gemv_sumsq_parts(n, k)
+        if hidden.shape != (m, n) or hidden.dtype != torch.bfloat16 or scaled_out is None \
+                or scaled_out.shape != (m, n) or scaled_out.dtype != torch.bfloat16 \
+                or sumsq_out is None or sumsq_out.shape != (m, p_out):
+            raise KernelError(f"gemv: hidden / scaled_out [M, N] bf16 and sumsq_out [M, {p_out}] needed")
+        if next_weight is not None and next_weight.shape != (n,):
+            raise KernelError("gemv: the next norm's weight must be [N]")
+        check(lib.kva_gemv(None, _dev(x, "x", contiguous=False), _dev(w, "w"), m, n, k, x.stride(0), n, 3, *norm,
+                           _dev(hidden, "hidden"), _opt(next_weight, "next_weight"),
+                           1 if next_weight is not None and next_weight.dtype == torch.float32 else 0,
+                           _dev(scaled_out, "scaled_out"), _dev(sumsq_out, "sumsq_out", torch.float32), _stream()),
+              "gemv")
+        return hidden
+    cols = n // 2 if swiglu else n
+    if out.shape != (m, cols) or (swiglu and out.dtype != torch.bfloat16) \
+            or out.dtype not in (torch.bfloat16, torch.float32) or not out.is_contiguous():
+        raise KernelError(f"gemv: out {tuple(out.shape)} {out.dtype} does not fit")
+    mode = 2 if swiglu else (1 if out.dtype == torch.float32 else 0)
+    check(lib.kva_gemv(_dev(out, "out"), _dev(x, "x", contiguous=False), _dev(w, "w"), m, n, k, x.stride(0), cols, mode, *norm,
+                       None, None, 0, None, None, _stream()), "gemv")
+    return out
+
+
+def gemv_qkv_rope_supported(m: int, k: int, head_dim: int) -> bool:
+    return bool(hip_lib().kva_gemv_qkv_rope_supported(int(m), int(k), int(head_dim)))
+
+
+def gemv_qkv_rope(x: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, num_q_heads: int,
+                  num_kv_heads: int, head_dim: int, positions: torch.Tensor,
+                  cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+                  k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                  slot_mapping: Optional[torch.Tensor], page_size: int, *,
+                  sumsq: Optional[torch.Tensor] = None, norm_width: int = 0, eps: float = 0.0):
+    """:func:`gemm_skinny_qkv_rope` for one or two rows, over the plain row-major weight."""
+    m, k = x.shape
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or not w.is_contiguous() \
+            or w.shape != ((num_q_heads + 2 * num_kv_heads) * head_dim, k):
+        raise KernelError(f"gemv_qkv_rope: bf16 x {tuple(x.shape)} does not fit weight {tuple(w.shape)} "
+                          f"for {num_q_heads}+2*{num_kv_heads} heads of {head_dim}")
+    if q_out.shape != (m, num_q_heads * head_dim) or q_out.dtype != torch.bfloat16 or not q_out.is_contiguous():
+        raise KernelError("gemv_qkv_rope: q_out must be bf16 [M, nq * d]")
+    if positions.shape != (m,):
+        raise KernelError("gemv_qkv_rope: one position per row")
+    if (cos is None) != (sin is None) or (cos is not None and (
+            cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] * 2 != head_dim)):
+        raise KernelError("gemv_qkv_rope: cos and sin tables must both be [positions, d/2]")
+    if sumsq is not None and (sumsq.dim() != 2 or sumsq.shape[0] != m or norm_width <= 0):
+        raise KernelError("gemv_qkv_rope: sumsq must be [M, parts] and norm_width positive")
+    write = k_cache is not None
+    if write:
+        if v_cache is None or slot_mapping is None or slot_mapping.shape != (m,):
+            raise KernelError("gemv_qkv_rope: K and V cache and one slot per row are all needed")
+        check_cache_shapes("gemv_qkv_rope", k_cache, v_cache, num_kv_heads, head_dim)
+        if k_cache.shape[2] != page_size or k_cache.dtype != torch.bfloat16:
+            raise KernelError("gemv_qkv_rope: cache page size or dtype does not fit")
+    check(hip_lib().kva_gemv_qkv_rope(
+        _dev(q_out, "q_out"), q_out.shape[1], _dev(x, "x"), _dev(w, "w"), m, k, x.stride(0), num_q_heads,
+        num_kv_heads, head_dim, _opt(sumsq, "sumsq", torch.float32), sumsq.shape[1] if sumsq is not None else 0,
+        int(norm_width), float(eps), _opt(cos, "cos", torch.float32), _opt(sin, "sin", torch.float32),
+        _dev(positions, "positions", torch.int32),
+        _dev(slot_mapping, "slot_mapping", torch.int32) if write else None,
+        _opt(k_cache, "k_cache") if write else None, _opt(v_cache, "v_cache") if write else None,
+        int(page_size), _stream()), "gemv_qkv_rope")
+    return q_out
+
+
 def normed_rows_finish(scaled: torch.Tensor, sumsq: torch.Tensor, norm_width: int, eps: float,
                        out: torch.Tensor, row_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[i] = scaled[row] * rsqrt(sum(sumsq[row]) / norm_width + eps), row = row_idx[i] or i."""
@@ -662,6 +758,7 @@ KERNEL_CLASSES = {
     "attention_rowwise": "attention", "attention_mfma": "attention", "attention_lds": "attention",
     "gemm_nt_f32": "gemm fp32", "gemm_vendor": "gemm (vendor library)",
     "gemm_skinny": "gemm (few rows)", "gemm_skinny_qkv_rope": "gemm (few rows)",
+    "gemv": "gemm (few rows)", "gemv_qkv_rope": "gemm (few rows)",
     "sample": "sampling", "mark_tokens": "sampling",
 }
 

@@ -53,6 +53,11 @@ _HIP_SIGNATURES = {
     "kva_gemm_skinny_supported": [I, I, I],
     "kva_gemm_skinny_qkv_rope_supported": [I, I, I],
     "kva_gemm_skinny_qkv_rope": [P, I, P, P, I, I, I, I, I, I, P, I, I, F, P, P, P, P, P, P, I, P],
+    "kva_gemv": [P, P, P, I, I, I, I, I, I, P, I, I, F, P, P, I, P, P, P],
+    "kva_gemv_supported": [I, I, I],
+    "kva_gemv_sumsq_parts": [I, I],
+    "kva_gemv_qkv_rope_supported": [I, I, I],
+    "kva_gemv_qkv_rope": [P, I, P, P, I, I, I, I, I, I, P, I, I, F, P, P, P, P, P, P, I, P],
     "kva_gemm_nt_f32": [P, P, P, I, I, I, I, I, I, P],
     "kva_gemm_vendor": [P, P, P, I, I, I, I, I, I, P],
     "kva_gemm_vendor_init": [],

@@ -38,8 +38,13 @@ class EncodedQKV:
         """``x`` [T, hidden] (plain or NormedRows).  Returns a tensor whose first ``nq * d`` columns
         are the position-encoded queries; K (encoded) and V of the step's tokens are in the cache
         when ``kv`` allows writing."""
-        tables = None
-        if self.linear.fusable(x) and K.gemm_skinny_qkv_rope_supported(x.shape[0], self.hidden_size, self.head_dim):
+        tables, rows = None, x.shape[0]
+        kernel = self.linear.fused_kernel(rows, x.dtype)
+        if kernel == Linear.GEMV and not K.gemv_qkv_rope_supported(rows, self.hidden_size, self.head_dim):
+            kernel = Linear.FEW_ROWS if self.linear.tiled is not None else None
+        if kernel == Linear.FEW_ROWS and not K.gemm_skinny_qkv_rope_supported(rows, self.hidden_size, self.head_dim):
+            kernel = None
+        if kernel is not None:
             tables = self.position.rotate_half_tables(x.device, self.head_dim)
         if tables is None:
             qkv = self.linear(x)
@@ -47,15 +52,17 @@ class EncodedQKV:
                                           self.head_dim, kv)
             return qkv
         write = kv is not None and kv.writes
-        q = torch.empty((x.shape[0], self.num_heads * self.head_dim), dtype=torch.bfloat16, device=x.device)
+        q = torch.empty((rows, self.num_heads * self.head_dim), dtype=torch.bfloat16, device=x.device)
         norm = {}
         if isinstance(x, NormedRows):
             norm = dict(sumsq=x.sumsq, norm_width=x.width, eps=x.eps)
             x = x.scaled
-        K.gemm_skinny_qkv_rope(x, self.linear.tiled, q, self.num_heads, self.num_kv_heads, self.head_dim,
-                               batch.positions, tables[0], tables[1],
-                               kv.k_cache if write else None, kv.v_cache if write else None,
-                               kv.slot_mapping if write else None, kv.page_size if kv is not None else 0, **norm)
+        product, weight = ((K.gemv_qkv_rope, self.linear.weight) if kernel == Linear.GEMV
+                           else (K.gemm_skinny_qkv_rope, self.linear.tiled))
+        product(x, weight, q, self.num_heads, self.num_kv_heads, self.head_dim,
+                batch.positions, tables[0], tables[1],
+                kv.k_cache if write else None, kv.v_cache if write else None,
+                kv.slot_mapping if write else None, kv.page_size if kv is not None else 0, **norm)
         return q
 
 

@@ -33,50 +33,84 @@ class Linear:
             if self.in_features % 32 == 0:
                 self.tiled = K.TiledWeight(self.weight, halves)
 
+    GEMV, FEW_ROWS = "gemv", "few_rows"
+
+    def fused_kernel(self, rows: int, dtype) -> Optional[str]:
+        """The hand-written product that takes ``rows`` rows of ``dtype`` with a norm on its input
+        and/or the residual stream in its epilogue: ``GEMV`` (one token: a matrix-vector product
+        over the plain weight), ``FEW_ROWS`` (the matrix-core kernel over the tiled copy) or None."""
+        from ..ops.gemm_bf16 import use_gemv, use_skinny
+        if dtype != torch.bfloat16 or self.weight.dtype != torch.bfloat16 or not self.weight.is_cuda:
+            return None
+        if use_gemv(rows, self.out_features, self.in_features):
+            return self.GEMV
+        if self.tiled is not None and use_skinny(rows, self.out_features, self.in_features, self.halves == 2):
+            return self.FEW_ROWS
+        return None
+
     def fusable(self, x) -> bool:
         """Whether this product can finish a norm on its input and/or feed the residual stream
         in its epilogue for these rows (bf16 everywhere, few rows)."""
-        from ..ops.gemm_bf16 import use_skinny
-        return (self.tiled is not None and x.dtype == torch.bfloat16
-                and use_skinny(x.shape[0], self.out_features, self.in_features, self.halves == 2))
+        return self.fused_kernel(x.shape[0], x.dtype) is not None
 
-    def will_fuse_residual(self, rows: int, dtype, tail: Optional[BranchTail]) -> bool:
-        """Whether :meth:`into_residual` will fuse for ``rows`` rows of ``dtype`` (then its input may
-        come as ``ops.kernels.TiledRows``)."""
-        from ..ops.gemm_bf16 import use_skinny
+    def residual_kernel(self, rows: int, dtype, tail: Optional[BranchTail]) -> Optional[str]:
+        """The kernel with which :meth:`into_residual` will fuse ``rows`` rows of ``dtype``, or None
+        (with ``FEW_ROWS`` its input may come as ``ops.kernels.TiledRows``)."""
         prep = tail.norm.prepared_by_product() if tail is not None and tail.norm is not None else None
-        return (prep is not None and prep[1] == self.out_features and self.tiled is not None
-                and dtype == torch.bfloat16 and tail.hidden.dtype == torch.bfloat16
-                and use_skinny(rows, self.out_features, self.in_features, self.halves == 2))
+        if prep is None or prep[1] != self.out_features or tail.hidden.dtype != torch.bfloat16:
+            return None
+        return self.fused_kernel(rows, dtype)
 
     def into_residual(self, x, tail: BranchTail) -> Optional[NormedRows]:
         """hidden += x @ W^T in place and the sum prepared for ``tail.norm``; ``None`` when this
         cannot be fused (the caller then takes the plain product)."""
-        prep = tail.norm.prepared_by_product() if tail is not None and tail.norm is not None else None
-        if prep is None or not self.fusable(x) or tail.hidden.dtype != torch.bfloat16:
+        kernel = self.residual_kernel(x.shape[0], x.dtype, tail)
+        if kernel is None:
             return None
-        next_w, width, eps = prep
-        if width != self.out_features:
-            return None
+        next_w, width, eps = tail.norm.prepared_by_product()
         rows = x.shape[0]
         scaled = torch.empty((rows, self.out_features), dtype=torch.bfloat16, device=x.device)
-        sumsq = torch.empty((rows, K.gemm_skinny_sumsq_parts(self.out_features)), dtype=torch.float32,
-                            device=x.device)
+        norm = {}
         if isinstance(x, NormedRows):
-            K.gemm_skinny(x.scaled, self.tiled, None, sumsq=x.sumsq, norm_width=x.width, eps=x.eps,
-                          hidden=tail.hidden, next_weight=next_w, scaled_out=scaled, sumsq_out=sumsq)
+            norm = dict(sumsq=x.sumsq, norm_width=x.width, eps=x.eps)
+            x = x.scaled
+        if kernel == self.GEMV:
+            if isinstance(x, K.TiledRows):
+                x = x.to_rows()
+            sumsq = torch.empty((rows, K.gemv_sumsq_parts(self.out_features, self.in_features)),
+                                dtype=torch.float32, device=x.device)
+            K.gemv(x, self.weight, None, hidden=tail.hidden, next_weight=next_w, scaled_out=scaled,
+                   sumsq_out=sumsq, **norm)
         else:
-            K.gemm_skinny(x, self.tiled, None, hidden=tail.hidden, next_weight=next_w,
-                          scaled_out=scaled, sumsq_out=sumsq, x_tiled=isinstance(x, K.TiledRows))
+            sumsq = torch.empty((rows, K.gemm_skinny_sumsq_parts(self.out_features)), dtype=torch.float32,
+                                device=x.device)
+            K.gemm_skinny(x, self.tiled, None, hidden=tail.hidden, next_weight=next_w, scaled_out=scaled,
+                          sumsq_out=sumsq, x_tiled=isinstance(x, K.TiledRows), **norm)
         return NormedRows(scaled, sumsq, width, eps, tail.norm)
+
+    def gated(self, x, out) -> None:
+        """``out`` = silu(x gate^T) * (x up^T) for a joined [gate; up] weight whose rows
+        :meth:`fusable` accepts; ``out`` is [rows, out_features / 2] or, for the few-rows kernel,
+        an ``ops.kernels.TiledRows`` of that size."""
+        norm = {}
+        if isinstance(x, NormedRows):
+            norm = dict(sumsq=x.sumsq, norm_width=x.width, eps=x.eps)
+            x = x.scaled
+        if self.fused_kernel(x.shape[0], x.dtype) == self.GEMV:
+            K.gemv(x, self.weight, out, swiglu=True, **norm)
+        else:
+            K.gemm_skinny(x, self.tiled, out, swiglu=True, out_tiled=isinstance(out, K.TiledRows), **norm)
 
     def __call__(self, x, out: Optional[torch.Tensor] = None,
                  out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
         if isinstance(x, NormedRows):
-            if self.fusable(x):
+            kernel = self.fused_kernel(x.shape[0], x.dtype)
+            if kernel is not None:
                 if out is None:
                     out = torch.empty((x.shape[0], self.out_features), dtype=out_dtype or x.dtype,
                                       device=x.device)
+                if kernel == self.GEMV:
+                    return K.gemv(x.scaled, self.weight, out, sumsq=x.sumsq, norm_width=x.width, eps=x.eps)
                 return K.gemm_skinny(x.scaled, self.tiled, out, sumsq=x.sumsq, norm_width=x.width, eps=x.eps)
             x = x.materialize()
         w = self.weight

@@ -52,23 +52,18 @@ class SwiGLU(FeedForward):
         """``x`` may be NormedRows; with a ``tail`` the down projection adds into the residual
         stream and prepares the next norm when the shapes allow (NormedRows are returned)."""
         rows = x.shape[0]
-        w = self.gate_up.tiled
-        fused_up = self.gate_up.fusable(x)
+        up_kernel = self.gate_up.fused_kernel(rows, x.dtype)
         # Both products in their few-rows form and at most 16 rows: the activations go from one to
         # the other in the order the second one's lanes read them (ops.kernels.TiledRows).
-        tiled = (fused_up and rows <= K.TiledRows.MAX_ROWS and self.intermediate_size % 8 == 0
-                 and self.down.will_fuse_residual(rows, x.dtype, tail))
+        tiled = (up_kernel == Linear.FEW_ROWS and rows <= K.TiledRows.MAX_ROWS and self.intermediate_size % 8 == 0
+                 and self.down.residual_kernel(rows, x.dtype, tail) == Linear.FEW_ROWS)
         if tiled:
             act = K.TiledRows(rows, self.intermediate_size, x.device)
         else:
             act = torch.empty((rows, self.intermediate_size), dtype=x.dtype, device=x.device)
-        if fused_up:
+        if up_kernel is not None:
             # activation fused into the product; an unfinished input norm is finished there too
-            if isinstance(x, NormedRows):
-                K.gemm_skinny(x.scaled, w, act, swiglu=True, sumsq=x.sumsq, norm_width=x.width, eps=x.eps,
-                              out_tiled=tiled)
-            else:
-                K.gemm_skinny(x, w, act, swiglu=True, out_tiled=tiled)
+            self.gate_up.gated(x, act)
         else:
             K.silu_mul(self.gate_up(x), act)
         if tail is not None:

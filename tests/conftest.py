@@ -54,7 +54,7 @@ TINY_D = dict(
 # products with their fused epilogues and the vendor products are the ones that run.
 MID_E = dict(
     architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=2003, hidden_size=512,
-    intermediate_size=1376, num_hidden_layers=2, num_attention_heads=8, num_key_value_heads=2,
+    intermediate_size=1536, num_hidden_layers=2, num_attention_heads=8, num_key_value_heads=2,
     head_dim=64, rms_norm_eps=1e-5, rope_theta=500000.0, max_position_embeddings=2048,
     rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
                       original_max_position_embeddings=512),
