@@ -84,7 +84,8 @@ def attention(args) -> None:
     qkv = torch.randn(T, nq * d, device=dev).bfloat16()
     out = torch.empty(T, nq * d, dtype=torch.bfloat16, device=dev)
     q_start = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
-    rows_per_item = {"lds": 128, "wave": 32 if args.tokens else 16}[args.kernel]
+    tiles = args.tiles or (2 if args.tokens else 1)
+    rows_per_item = {"lds": 128, "wave": 16 * tiles}[args.kernel]
     meta = []
     for e, (start, n) in enumerate(entries):
         for r0 in range(0, n * group, rows_per_item):
@@ -104,7 +105,6 @@ def attention(args) -> None:
         calls = [lambda c=c: K.attention_lds(qkv, nq * d, out, c[0], c[1], table, meta_d, nq, nkv, d, scale, 0, args.pair)
                  for c in caches]
     else:
-        tiles = 2 if args.tokens else 1
         pair = bool(args.tokens) and len(meta) * nkv >= 2048 and not args.no_pair
         calls = [lambda c=c: K.attention_mfma(qkv, nq * d, out, c[0], c[1], table, ent, row0, seat, qs, sp, nq, nkv,
                                               d, scale, 0, splits, per, tiles, pair, meta_d) for c in caches]
@@ -228,6 +228,7 @@ def main(argv=None) -> int:
     a.add_argument("--head-dim", type=int, default=64)
     a.add_argument("--reps", type=int, default=20)
     a.add_argument("--no-pair", action="store_true", help="wave kernel: never give a wave two items")
+    a.add_argument("--tiles", type=int, default=0, help="wave kernel: row tiles of 16 per item (default 2 for a prompt, 1 for decoded tokens)")
     a.add_argument("--pair", action="store_true", help="workgroup kernel: a workgroup takes item i and item n-1-i")
     a.add_argument("--graph", action="store_true", help="time the calls inside a HIP graph (no host launch cost)")
     g = sub.add_parser("gemm")
