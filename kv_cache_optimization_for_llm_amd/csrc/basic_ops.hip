@@ -120,6 +120,57 @@ template <> __device__ inline void load_weight8<float>(const float *w, float (&f
     f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
 }
 
+// The gather for a few tokens of a bf16 model, with the first norm prepared in the same pass, as a
+// product's residual epilogue prepares the norm after it: hidden[t, :] = table[id, :],
+// scaled[t, :] = round(hidden * w_norm), sumsq[t] = sum hidden^2.  A decode step saves the
+// norm kernel that would read back what this one has just written.
+template <typename TW>
+__global__ void __launch_bounds__(256)
+embed_gather_prep_kernel(bf16_t *__restrict__ hidden, bf16_t *__restrict__ scaled, float *__restrict__ sumsq,
+                         const bf16_t *__restrict__ table, const int *__restrict__ ids,
+                         const int *__restrict__ feedback, const TW *__restrict__ norm_w, int width) {
+    __shared__ float scratch[4];
+    const int row = blockIdx.x;
+    int id = ids[row];
+    if (id < 0) id = feedback[-1 - id];
+    const bf16_t *src = table + (size_t)id * width;
+    float ss = 0.f;
+    for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8) {
+        const uint4 raw = *reinterpret_cast<const uint4 *>(src + i);
+        float v[8], w[8];
+        unpack8(raw, v);
+        load_weight8<TW>(norm_w + i, w);
+        *reinterpret_cast<uint4 *>(hidden + (size_t)row * width + i) = raw;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            ss += v[j] * v[j];
+            v[j] *= w[j];
+        }
+        *reinterpret_cast<uint4 *>(scaled + (size_t)row * width + i) = pack8(v);
+    }
+    const float total = block_sum(ss, scratch, blockDim.x / KVA_WAVE);
+    if (threadIdx.x == 0) sumsq[row] = total;
+}
+
+// bf16 table and outputs, width a multiple of 8; norm_w [width] bf16 or fp32.
+extern "C" int kva_embed_gather_prep(void *hidden, void *scaled, float *sumsq, const void *table, const int *ids,
+                                     const int *feedback, const void *norm_w, int norm_w_f32, int rows, int width,
+                                     hipStream_t stream) {
+    KVA_REQUIRE(rows >= 0 && width > 0 && width % 8 == 0, "embed_gather_prep: bad sizes rows=%d width=%d (a multiple of 8)",
+                rows, width);
+    KVA_REQUIRE(hidden && scaled && sumsq && table && ids && norm_w, "embed_gather_prep: a pointer is missing");
+    if (rows == 0) return KVA_OK;
+    dim3 grid(rows), block(256);
+    if (norm_w_f32)
+        hipLaunchKernelGGL(embed_gather_prep_kernel<float>, grid, block, 0, stream, (bf16_t *)hidden, (bf16_t *)scaled,
+                           sumsq, (const bf16_t *)table, ids, feedback, (const float *)norm_w, width);
+    else
+        hipLaunchKernelGGL(embed_gather_prep_kernel<bf16_t>, grid, block, 0, stream, (bf16_t *)hidden, (bf16_t *)scaled,
+                           sumsq, (const bf16_t *)table, ids, feedback, (const bf16_t *)norm_w, width);
+    KVA_CHECK_LAUNCH("embed_gather_prep");
+    return KVA_OK;
+}
+
 #define RMS_VEC_CACHE 4   // vectors of 8 a thread keeps between the passes
 template <typename TW>
 __global__ void rmsnorm_vec_kernel(bf16_t *__restrict__ out, bf16_t *__restrict__ hidden,

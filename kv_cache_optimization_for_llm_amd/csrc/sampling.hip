@@ -177,7 +177,7 @@ sample_pick_kernel(const float *__restrict__ logits, int vocab, int chunk_tokens
                    const ChunkRecord *__restrict__ records, unsigned int seed,
                    const unsigned int *__restrict__ rng_key, const unsigned int *__restrict__ rng_step,
                    unsigned char *mark_mask /* may be penalty_mask */, const int *__restrict__ mark_seat,
-                   int *__restrict__ out_tokens) {
+                   int *__restrict__ out_tokens, int *__restrict__ host_tokens) {
     const int row = blockIdx.x, lane = threadIdx.x;
     const ChunkRecord *rec = records + (size_t)row * chunks;
     // this lane's chunks: a contiguous run, so that lane order is chunk order
@@ -269,6 +269,7 @@ sample_pick_kernel(const float *__restrict__ logits, int vocab, int chunk_tokens
     }
     if (lane == 0) {
         out_tokens[row] = token;
+        if (host_tokens != nullptr) host_tokens[row] = token;      // pinned host memory, mapped for the device
         if (mark_mask != nullptr && mark_seat != nullptr) {
             const int seat = mark_seat[row];
             if (seat >= 0 && token >= 0 && token < vocab) mark_mask[(size_t)seat * vocab + token] = 1;
@@ -284,12 +285,24 @@ extern "C" long long kva_sample_workspace_bytes(int rows, int chunks) {
 // out_tokens[row] = the sampled (inv_temperature[row] > 0) or the best token of logits[row, :].
 // penalty_mask [seats, vocab] with row_seat[row] (-1: none) says which logits are penalised;
 // mark_mask / mark_seat (may be the same mask, -1: none) get the chosen token marked afterwards.
+// host_tokens (optional): pinned host memory (hipHostMalloc, torch's pin_memory) with room for a token
+// per row; the kernel that chooses the tokens writes them there as well, which saves the copy
+// that would otherwise follow it on the stream.  Refused unless the runtime says the memory is
+// mapped for the device.
 extern "C" int kva_sample(int *out_tokens, const float *logits, int rows, int vocab, int chunks,
                           const unsigned char *penalty_mask, const int *row_seat, float penalty,
                           const float *inv_temperature, unsigned int seed,
                           const unsigned int *rng_key, const unsigned int *rng_step, int any_sampled,
                           void *workspace, unsigned char *mark_mask, const int *mark_seat,
-                          hipStream_t stream) {
+                          int *host_tokens, hipStream_t stream) {
+    int *host_mapped = nullptr;
+    if (host_tokens != nullptr) {
+        void *dev = nullptr;
+        const hipError_t e = hipHostGetDevicePointer(&dev, host_tokens, 0);
+        KVA_REQUIRE(e == hipSuccess && dev != nullptr, "sample: host_tokens is not pinned host memory mapped for the device (%s)",
+                    hipGetErrorString(e));
+        host_mapped = (int *)dev;
+    }
     KVA_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", rows, vocab);
     KVA_REQUIRE(chunks >= 1 && chunks <= SAMPLE_MAX_CHUNKS, "sample: chunk count %d is not in 1..%d", chunks,
                 SAMPLE_MAX_CHUNKS);
@@ -306,7 +319,7 @@ extern "C" int kva_sample(int *out_tokens, const float *logits, int rows, int vo
                        vocab, chunk_tokens, penalty_mask, row_seat, penalty, inv_t, records);
     hipLaunchKernelGGL(sample_pick_kernel, dim3(rows), dim3(KVA_WAVE), 0, stream, logits, vocab,
                        chunk_tokens, chunks, penalty_mask, row_seat, penalty, inv_t, records, seed, rng_key,
-                       rng_step, mark_mask, mark_seat, out_tokens);
+                       rng_step, mark_mask, mark_seat, out_tokens, host_mapped);
     KVA_CHECK_LAUNCH("sample");
     return KVA_OK;
 }

@@ -183,15 +183,30 @@ class Model:
         return report
 
     # ---- forward
+    GATHER_PREP_MAX_ROWS = 64       # steps of at most this many tokens gather and prepare the first norm in one kernel
+
     def forward(self, batch, cache) -> torch.Tensor:
         """Runs the batch's tokens through every layer call and returns fp32 logits
         ``[len(batch.logit_rows), vocab]``."""
         T = batch.num_tokens
         hidden = torch.empty((T, self.spec.hidden_size), dtype=self.dtype, device=self.device)
-        K.embed_gather(self.embedding, batch.token_ids, hidden, getattr(batch, "feedback", None))
-        if self.spec.embedding_scale != 1.0:
-            K.scale_softcap(hidden, self.spec.embedding_scale)
         delta = None
+        first_norm = self.blocks[self.calls[0][0].layer].first_norm() if self.calls else self.final_norm
+        prep = first_norm.prepared_by_product() if first_norm is not None else None
+        if (T <= self.GATHER_PREP_MAX_ROWS and prep is not None and prep[1] == self.spec.hidden_size
+                and self.dtype == torch.bfloat16 and self.embedding.dtype == torch.bfloat16
+                and self.spec.hidden_size % 8 == 0 and self.spec.embedding_scale == 1.0):
+            # a few tokens: the gather prepares the first norm as a product's epilogue would, and
+            # the first product finishes it (or one kernel does, as the norm kernel would have)
+            scaled = torch.empty_like(hidden)
+            sumsq = torch.empty((T, 1), dtype=torch.float32, device=self.device)
+            K.embed_gather_prep(self.embedding, batch.token_ids, hidden, scaled, sumsq, prep[0],
+                                getattr(batch, "feedback", None))
+            delta = NormedRows(scaled, sumsq, prep[1], prep[2], first_norm)
+        else:
+            K.embed_gather(self.embedding, batch.token_ids, hidden, getattr(batch, "feedback", None))
+            if self.spec.embedding_scale != 1.0:
+                K.scale_softcap(hidden, self.spec.embedding_scale)
         for i, (call, slot) in enumerate(self.calls):
             block = self.blocks[call.layer]
             # the norm that reads the residual stream after this block

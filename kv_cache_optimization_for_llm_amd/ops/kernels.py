@@ -6,6 +6,7 @@ a tensor that is not on the GPU, or a missing kernel library, is an error.
 """
 from __future__ import annotations
 
+import ctypes
 from typing import Optional
 
 import torch
@@ -81,6 +82,26 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor,
                                      dtype_code(table.dtype), dtype_code(out.dtype), _stream()),
           "embed_gather")
     return out
+
+
+def embed_gather_prep(table: torch.Tensor, ids: torch.Tensor, hidden: torch.Tensor, scaled: torch.Tensor,
+                      sumsq: torch.Tensor, norm_weight: torch.Tensor,
+                      feedback: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """:func:`embed_gather` for a bf16 table and stream that prepares the first norm in the same
+    pass: ``scaled = round(hidden * norm_weight)`` and ``sumsq[t, 0] = sum(hidden[t]^2)``."""
+    rows, width = hidden.shape
+    if table.dim() != 2 or table.shape[1] != width or ids.shape != (rows,) or scaled.shape != (rows, width) \
+            or sumsq.shape != (rows, 1) or norm_weight.shape != (width,):
+        raise KernelError(f"embed_gather_prep: shapes table {tuple(table.shape)} ids {tuple(ids.shape)} hidden "
+                          f"{tuple(hidden.shape)} scaled {tuple(scaled.shape)} sumsq {tuple(sumsq.shape)} do not fit")
+    if not (table.dtype == hidden.dtype == scaled.dtype == torch.bfloat16) or width % 8 \
+            or norm_weight.dtype not in (torch.bfloat16, torch.float32):
+        raise KernelError("embed_gather_prep: bf16 table and outputs, a width that is a multiple of 8")
+    check(hip_lib().kva_embed_gather_prep(
+        _dev(hidden, "hidden"), _dev(scaled, "scaled"), _dev(sumsq, "sumsq", torch.float32), _dev(table, "table"),
+        _dev(ids, "ids", torch.int32), _opt(feedback, "feedback", torch.int32), _dev(norm_weight, "norm_weight"),
+        1 if norm_weight.dtype == torch.float32 else 0, rows, width, _stream()), "embed_gather_prep")
+    return hidden
 
 
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
@@ -245,11 +266,13 @@ def sample(logits: torch.Tensor, out_tokens: torch.Tensor, *, chunks: int = 128,
            rng_key: Optional[torch.Tensor] = None, rng_step: Optional[torch.Tensor] = None,
            penalty_mask: Optional[torch.Tensor] = None, row_seat: Optional[torch.Tensor] = None,
            penalty: float = 1.0, mark_mask: Optional[torch.Tensor] = None,
-           mark_seat: Optional[torch.Tensor] = None) -> torch.Tensor:
+           mark_seat: Optional[torch.Tensor] = None, host_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Greedy (rows whose inv_temperature is 0 or absent) or temperature sampling per row.
     ``penalty_mask`` ``[seats, vocab]`` with ``row_seat`` (-1: none) names the logits that are
     penalised; ``mark_mask`` with ``mark_seat`` (-1: none) gets ``mark_mask[seat, token] = 1`` for
-    every chosen token, in the same launch."""
+    every chosen token, in the same launch.  ``host_tokens``: a pinned host int32 tensor with a
+    place per row that takes the tokens too, written by the kernel itself (valid once the stream
+    has passed the launch)."""
     rows, vocab = logits.shape
     if out_tokens.shape != (rows,):
         raise KernelError("sample: one output token per row")
@@ -264,6 +287,10 @@ def sample(logits: torch.Tensor, out_tokens: torch.Tensor, *, chunks: int = 128,
     if (mark_mask is None) != (mark_seat is None) or (mark_mask is not None and (
             mark_seat.shape != (rows,) or mark_mask.dim() != 2 or mark_mask.shape[1] != vocab)):
         raise KernelError("sample: marking needs a mask [seats, vocab] and a seat per row")
+    if host_tokens is not None and (host_tokens.is_cuda or not host_tokens.is_pinned() or host_tokens.dtype != torch.int32
+                                    or host_tokens.dim() != 1 or host_tokens.shape[0] < rows
+                                    or not host_tokens.is_contiguous()):
+        raise KernelError("sample: host_tokens must be a pinned host int32 vector with a place per row")
     lib = hip_lib()
     ws = torch.empty(max(1, lib.kva_sample_workspace_bytes(rows, chunks) // 4), dtype=torch.float32,
                      device=logits.device)
@@ -273,7 +300,8 @@ def sample(logits: torch.Tensor, out_tokens: torch.Tensor, *, chunks: int = 128,
         float(penalty), _opt(inv_temperature, "inv_temperature", torch.float32), int(seed) & 0xFFFFFFFF,
         _opt(rng_key, "rng_key", torch.int32), _opt(rng_step, "rng_step", torch.int32),
         1 if any_sampled else 0, _dev(ws, "workspace"), _opt(mark_mask, "mark_mask", torch.uint8),
-        _opt(mark_seat, "mark_seat", torch.int32), _stream()), "sample")
+        _opt(mark_seat, "mark_seat", torch.int32),
+        ctypes.c_void_p(host_tokens.data_ptr()) if host_tokens is not None else None, _stream()), "sample")
     return out_tokens
 
 
@@ -752,7 +780,7 @@ def normed_rows_finish(scaled: torch.Tensor, sumsq: torch.Tensor, norm_width: in
 # --------------------------------------------------------------------------------------
 # Measurement: device time per class of kernel, from events around every launch.
 KERNEL_CLASSES = {
-    "embed_gather": "embedding", "rmsnorm": "norm", "normed_rows_finish": "norm",
+    "embed_gather": "embedding", "embed_gather_prep": "embedding", "rmsnorm": "norm", "normed_rows_finish": "norm",
     "residual_add": "elementwise", "scale_softcap": "elementwise", "cast": "elementwise",
     "silu_mul": "activation", "rope_kv_write": "rope + cache write",
     "attention_rowwise": "attention", "attention_mfma": "attention", "attention_lds": "attention",

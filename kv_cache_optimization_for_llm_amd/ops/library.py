@@ -33,6 +33,7 @@ U = c_uint
 
 _HIP_SIGNATURES = {
     "kva_embed_gather": [P, P, P, P, I, I, I, I, P],
+    "kva_embed_gather_prep": [P, P, P, P, P, P, P, I, I, I, P],
     "kva_rmsnorm": [P, P, P, P, P, I, I, F, I, I, P],
     "kva_residual_add": [P, P, LL, I, P],
     "kva_scale_softcap": [P, LL, F, F, I, P],
@@ -63,7 +64,7 @@ _HIP_SIGNATURES = {
     "kva_gemm_vendor_init": [],
     "kva_gemm_vendor_tune": [P, P, P, I, I, I, I, I, I, I, P, P, P, P],
     "kva_gemm_vendor_forget": [I, I, I, I, I, I],
-    "kva_sample": [P, P, I, I, I, P, P, F, P, U, P, P, I, P, P, P, P],
+    "kva_sample": [P, P, I, I, I, P, P, F, P, U, P, P, I, P, P, P, P, P],
     "kva_mark_tokens": [P, P, P, I, I, P],
 }
 

@@ -51,8 +51,8 @@ def _as_i32(values: Sequence[int]) -> np.ndarray:
 
 
 class PendingTokens:
-    """Sampled tokens on their way to the host: the copy into pinned memory has been queued and
-    :meth:`wait` blocks until it has arrived."""
+    """Sampled tokens on their way to the host: the kernel that chooses them writes them into
+    pinned memory as well, and :meth:`wait` blocks until the stream has passed it."""
 
     def __init__(self, host: torch.Tensor, event: "torch.cuda.Event", n: int):
         self._host, self._event, self._n = host, event, n
@@ -66,6 +66,10 @@ class PendingTokens:
 
 
 class Sampler:
+    # the kernel that chooses the tokens writes them to the pinned host buffer itself (no copy
+    # kernel behind it on the stream)
+    KERNEL_WRITES_HOST = True
+
     def __init__(self, vocab_size: int, max_seqs: int, device, *, seed: int = 0,
                  repetition_penalty: float = 1.0, chunks: int = 128):
         if repetition_penalty <= 0:
@@ -102,8 +106,8 @@ class Sampler:
 
     def sample_async(self, logits: torch.Tensor, rows: Sequence[SampleRow],
                      out: Optional[torch.Tensor] = None) -> PendingTokens:
-        """Queues the sampling of one token per logits row and their copy to the host, without
-        waiting for either.  ``out`` (device int32, at least ``len(rows)`` long) takes the tokens,
+        """Queues the sampling of one token per logits row (the tokens land in pinned host memory
+        too), without waiting for it.  ``out`` (device int32, at least ``len(rows)`` long) takes the tokens,
         row by row, and may be read by later work on the same stream."""
         n = len(rows)
         if logits.shape != (n, self.vocab_size):
@@ -140,7 +144,8 @@ class Sampler:
         K.sample(logits, out, chunks=self.chunks, inv_temperature=inv_t, seed=self.seed, rng_key=key,
                  rng_step=step, penalty_mask=self.mask if use_mask else None, row_seat=seat_t,
                  penalty=self.penalty, mark_mask=self.mask if mark_seat is not None else None,
-                 mark_seat=mark_seat)
-        host[:n].copy_(out, non_blocking=True)
+                 mark_seat=mark_seat, host_tokens=host if self.KERNEL_WRITES_HOST else None)
+        if not self.KERNEL_WRITES_HOST:
+            host[:n].copy_(out, non_blocking=True)
         event.record()
         return PendingTokens(host, event, n)

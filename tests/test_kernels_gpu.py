@@ -36,6 +36,31 @@ def test_embed_gather(dtype, table_dtype, gpu):
     assert torch.equal(out.cpu(), want)
 
 
+@pytest.mark.parametrize("width", [8, 520, 2048, 4104])
+@pytest.mark.parametrize("weight_dtype", ["float32", "bfloat16"])
+def test_embed_gather_that_prepares_the_first_norm(width, weight_dtype, gpu):
+    """hidden = table[ids] (ids from the feedback buffer too), scaled = round(hidden * w), the sum of
+    squares per row; finished, it is the norm of the gathered rows."""
+    table = rnd(91, width, dtype=torch.bfloat16)
+    w = (1 + 0.1 * rnd(width, seed=2)).to(DT[weight_dtype])
+    ids = torch.tensor([3, -1, 90, 0, -2, 3], dtype=torch.int32)
+    feedback = torch.tensor([55, 7], dtype=torch.int32)
+    real = torch.tensor([3, 55, 90, 0, 7, 3])
+    hidden = torch.full((6, width), float("nan"), dtype=torch.bfloat16, device=gpu)
+    scaled, sumsq = torch.empty_like(hidden), torch.full((6, 1), float("nan"), device=gpu)
+    K.embed_gather_prep(table.to(gpu), ids.to(gpu), hidden, scaled, sumsq, w.to(gpu), feedback.to(gpu))
+    want = table[real]
+    assert torch.equal(hidden.cpu(), want)
+    assert torch.equal(scaled.cpu(), (want.float() * w.float()).to(torch.bfloat16))
+    assert torch.allclose(sumsq.cpu()[:, 0], (want.float() ** 2).sum(-1), rtol=1e-5)
+    eps = 2e-6
+    fin = torch.empty_like(hidden)
+    K.normed_rows_finish(scaled, sumsq, width, eps, fin)
+    close(fin, plain.rms_norm(want.float(), w.float(), eps), torch.bfloat16, "gather + norm", tol16=1.2e-2)
+    with pytest.raises(K.KernelError):
+        K.embed_gather_prep(table.float().to(gpu), ids.to(gpu), hidden, scaled, sumsq, w.to(gpu), feedback.to(gpu))
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("width", [50, 64, 520, 1000, 2048, 2050, 4096, 4104])
 def test_rmsnorm_plain_fused_and_gathered(dtype, width, gpu):
@@ -547,3 +572,19 @@ def test_sampler_distribution_and_boundaries(gpu):
     counts = np.bincount(got, minlength=vocab)
     for t in np.argsort(probs)[-8:]:
         assert abs(counts[t] / draws - probs[t]) / probs[t] < 0.05
+
+
+def test_sampler_writes_the_tokens_to_pinned_host_memory_too(gpu):
+    """The kernel that chooses the tokens leaves them in the host's pinned buffer as well: the same
+    values as in the device vector once the stream has passed the launch; memory that is not
+    pinned is refused before anything is launched."""
+    g = torch.Generator().manual_seed(11)
+    logits = torch.randn(5, 1001, generator=g).to(gpu)
+    out = torch.full((5,), -1, dtype=torch.int32, device=gpu)
+    host = torch.full((8,), -7, dtype=torch.int32).pin_memory()
+    K.sample(logits, out, chunks=16, host_tokens=host)
+    torch.cuda.synchronize()
+    assert torch.equal(host[:5], out.cpu()) and torch.equal(out.cpu().long(), logits.cpu().argmax(-1))
+    assert (host[5:] == -7).all()
+    with pytest.raises(K.KernelError):
+        K.sample(logits, out, chunks=16, host_tokens=torch.zeros(8, dtype=torch.int32))
