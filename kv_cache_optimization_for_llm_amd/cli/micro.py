@@ -162,7 +162,9 @@ def prompt(args) -> None:
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
     eng = Engine(None, EngineOptions(dtype="bfloat16", cache_tokens=args.tokens + 64, max_seqs=2,
-                                     max_seq_len=cfg["max_position_embeddings"], use_graphs=not args.no_graphs),
+                                     max_seq_len=cfg["max_position_embeddings"], use_graphs=not args.no_graphs,
+                                     max_batch_tokens=max(8192, args.tokens),
+                                     gemm_tune_rows=[args.portion] if args.tune_gemm else []),
                  config_dict=cfg, random_seed=0)
     gen = torch.Generator().manual_seed(0)
     tokens = [int(t) for t in torch.randint(0, eng.vocab_size, (args.tokens,), generator=gen)]
@@ -242,6 +244,7 @@ def main(argv=None) -> int:
     pr.add_argument("--layers", type=int, default=0, help="fewer layers than the 16 of the shape")
     pr.add_argument("--reps", type=int, default=4)
     pr.add_argument("--no-graphs", action="store_true")
+    pr.add_argument("--tune-gemm", action="store_true", help="time the vendor library's algorithms for the portion's rows first")
     st = sub.add_parser("stream", help="a kernel that only reads: the floor for weight-streaming kernels")
     st.add_argument("--megabytes", default="8.4,12.6,33.5,67,525", help="comma list of sizes to read")
     st.add_argument("--workgroups", default="256,1024,2048")
