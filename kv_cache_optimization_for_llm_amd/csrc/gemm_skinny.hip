@@ -23,8 +23,8 @@
 // of a workgroup that work on the same K range stage X through LDS, once for all of them, instead
 // of each loading MT fragments of X per fragment of W.  Matrices with at most half as many tile
 // groups as the chip has compute units are cut into half tiles: two workgroups share a tile, each
-// taking 8 of its 16 rows, because a compute unit sustains only some 25 GB/s of a stream from
-// memory and the chip's bandwidth needs all of them.
+// taking 8 of its 16 rows, because the chip's 6 TB/s are 24 GB/s from each of 256 compute units and
+// a matrix that leaves half of them without a workgroup gets half of it.
 //
 // Row scaling.  With `sumsq` the rows of X are un-normalised norm inputs: X = round(h * w_norm)
 // and sumsq[m, 0..parts) are partial sums of h[m,:]^2; the product is multiplied by
@@ -709,8 +709,8 @@ static int choose_k_waves(int groups, int K, int ntw) {
     return kw;
 }
 
-// A compute unit streams some 25 GB/s of weights whatever its waves do, so a matrix with at most
-// half as many tile groups as the chip has compute units is spread over twice as many workgroups:
+// Every compute unit has its share of the chip's bandwidth to give (24 GB/s each), so a matrix with
+// at most half as many tile groups as the chip has compute units is spread over twice as many workgroups:
 // each takes half (8) of the rows of its tiles.  Depends on the matrix only, never on M.
 static int compute_units() {
     static int cus = 0;
