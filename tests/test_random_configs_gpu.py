@@ -63,9 +63,26 @@ def wide_group_config(nq, nkv, d):
                 tie_word_embeddings=False, hidden_act="silu", torch_dtype="bfloat16")
 
 
-@pytest.mark.parametrize("case", list(range(12)) + ["32 heads on 1", "40 heads on 2", "17 heads on 1"])
+def wide_config(hidden, inter, nq, nkv, d, tied):
+    """Widths that are multiples of 512: one or two decoded tokens take the matrix-vector kernel
+    (with its rotation epilogue where half a head is a multiple of the pairs a wavefront works on,
+    whatever the attention kernel needs), the other row counts the few-rows kernel or the library."""
+    return dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=1003, hidden_size=hidden,
+                intermediate_size=inter, num_hidden_layers=2, num_attention_heads=nq, num_key_value_heads=nkv,
+                head_dim=d, rms_norm_eps=1e-5, rope_theta=10000.0, max_position_embeddings=1024,
+                tie_word_embeddings=tied, hidden_act="silu", torch_dtype="bfloat16")
+
+
+WIDE = {"512 wide, head 64": (512, 1024, 8, 2, 64, True), "1024 wide, head 24": (1024, 1000, 6, 3, 24, False),
+        "1536 wide, head 96": (1536, 512, 4, 1, 96, True)}
+
+
+@pytest.mark.parametrize("case", list(range(12)) + ["32 heads on 1", "40 heads on 2", "17 heads on 1"] + list(WIDE))
 def test_random_configuration_under_two_cuts(case, tmp_path, gpu):
-    if isinstance(case, str):
+    if case in WIDE:
+        rng = np.random.default_rng(sum(WIDE[case][:5]))
+        cfg, case = wide_config(*WIDE[case]), WIDE[case][0]
+    elif isinstance(case, str):
         nq, nkv, d = {"32 heads on 1": (32, 1, 64), "40 heads on 2": (40, 2, 32), "17 heads on 1": (17, 1, 16)}[case]
         rng = np.random.default_rng(nq * 100 + d)
         cfg, case = wide_group_config(nq, nkv, d), nq
