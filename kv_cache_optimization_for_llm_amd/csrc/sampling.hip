@@ -285,6 +285,16 @@ extern "C" long long kva_sample_workspace_bytes(int rows, int chunks) {
 // out_tokens[row] = the sampled (inv_temperature[row] > 0) or the best token of logits[row, :].
 // penalty_mask [seats, vocab] with row_seat[row] (-1: none) says which logits are penalised;
 // mark_mask / mark_seat (may be the same mask, -1: none) get the chosen token marked afterwards.
+// Whether a kernel may write to this host memory: pinned and mapped for the current device.
+extern "C" int kva_host_memory_is_mapped(void *host) {
+    void *dev = nullptr;
+    if (host == nullptr || hipHostGetDevicePointer(&dev, host, 0) != hipSuccess) {
+        (void)hipGetLastError();                                    // the query's failure is an answer, not an error to keep
+        return 0;
+    }
+    return dev != nullptr ? 1 : 0;
+}
+
 // host_tokens (optional): pinned host memory (hipHostMalloc, torch's pin_memory) with room for a token
 // per row; the kernel that chooses the tokens writes them there as well, which saves the copy
 // that would otherwise follow it on the stream.  Refused unless the runtime says the memory is

@@ -261,6 +261,13 @@ def gemm_nt_f32(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Te
     return out
 
 
+def host_memory_is_mapped(t: torch.Tensor) -> bool:
+    """Whether a kernel may write into this host tensor (pinned memory mapped for the device)."""
+    if t.is_cuda or not t.is_pinned():
+        return False
+    return bool(hip_lib().kva_host_memory_is_mapped(ctypes.c_void_p(t.data_ptr())))
+
+
 def sample(logits: torch.Tensor, out_tokens: torch.Tensor, *, chunks: int = 128,
            inv_temperature: Optional[torch.Tensor] = None, seed: int = 0,
            rng_key: Optional[torch.Tensor] = None, rng_step: Optional[torch.Tensor] = None,

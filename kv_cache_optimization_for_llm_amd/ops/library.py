@@ -64,6 +64,7 @@ _HIP_SIGNATURES = {
     "kva_gemm_vendor_init": [],
     "kva_gemm_vendor_tune": [P, P, P, I, I, I, I, I, I, I, P, P, P, P],
     "kva_gemm_vendor_forget": [I, I, I, I, I, I],
+    "kva_host_memory_is_mapped": [P],
     "kva_sample": [P, P, I, I, I, P, P, F, P, U, P, P, I, P, P, P, P, P],
     "kva_mark_tokens": [P, P, P, I, I, P],
 }

@@ -82,6 +82,7 @@ class Sampler:
             self.mask = torch.zeros((max_seqs, vocab_size), dtype=torch.uint8, device=device)
         # pinned landing buffers for sample_async, used in turn (two samplings may be in flight)
         self._landing: List[torch.Tensor] = []
+        self._kernel_writes_host = False
         self._landing_next = 0
 
     def reset_seat(self, seat: int, emitted: Sequence[int] = ()) -> None:
@@ -120,6 +121,8 @@ class Sampler:
         if len(self._landing) < 3 or self._landing[0].shape[0] < n:
             size = max(64, n)
             self._landing = [torch.zeros(size, dtype=torch.int32, pin_memory=True) for _ in range(3)]
+            # where the runtime does not map pinned memory for the device, a copy follows the kernels instead
+            self._kernel_writes_host = self.KERNEL_WRITES_HOST and all(K.host_memory_is_mapped(t) for t in self._landing)
         host = self._landing[self._landing_next]
         self._landing_next = (self._landing_next + 1) % len(self._landing)
         event = torch.cuda.Event()
@@ -144,8 +147,8 @@ class Sampler:
         K.sample(logits, out, chunks=self.chunks, inv_temperature=inv_t, seed=self.seed, rng_key=key,
                  rng_step=step, penalty_mask=self.mask if use_mask else None, row_seat=seat_t,
                  penalty=self.penalty, mark_mask=self.mask if mark_seat is not None else None,
-                 mark_seat=mark_seat, host_tokens=host if self.KERNEL_WRITES_HOST else None)
-        if not self.KERNEL_WRITES_HOST:
+                 mark_seat=mark_seat, host_tokens=host if self._kernel_writes_host else None)
+        if not self._kernel_writes_host:
             host[:n].copy_(out, non_blocking=True)
         event.record()
         return PendingTokens(host, event, n)

@@ -588,3 +588,9 @@ def test_sampler_writes_the_tokens_to_pinned_host_memory_too(gpu):
     assert (host[5:] == -7).all()
     with pytest.raises(K.KernelError):
         K.sample(logits, out, chunks=16, host_tokens=torch.zeros(8, dtype=torch.int32))
+
+
+def test_which_host_memory_a_kernel_may_write(gpu):
+    assert K.host_memory_is_mapped(torch.zeros(8, dtype=torch.int32).pin_memory())
+    assert not K.host_memory_is_mapped(torch.zeros(8, dtype=torch.int32))
+    assert not K.host_memory_is_mapped(torch.zeros(8, dtype=torch.int32, device=gpu))
