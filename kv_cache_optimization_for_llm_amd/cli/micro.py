@@ -126,22 +126,27 @@ def gemm(args) -> None:
     copies = min(48, max(4, int(600e6 / (n * k * 2)) + 1))
     x = torch.randn(m, k, device=dev).bfloat16()
     ws = [torch.randn(n, k, device=dev).bfloat16() * 0.02 for _ in range(copies)]
-    tiled = [K.TiledWeight(w, 2 if mode == "swiglu" else 1) for w in ws]
+    gemv = args.kernel == "gemv"
+    if gemv and not K.gemv_supported(m, n, k):
+        raise SystemExit(f"the matrix-vector kernel does not take {m} rows of [{n} x {k}]")
+    tiled = ws if gemv else [K.TiledWeight(w, 2 if mode == "swiglu" else 1) for w in ws]
+    product = K.gemv if gemv else K.gemm_skinny
     if mode == "resid":
         hidden = torch.zeros(m, n, device=dev).bfloat16()
         scaled = torch.empty_like(hidden)
-        ss = torch.empty(m, K.gemm_skinny_sumsq_parts(n), device=dev)
+        ss = torch.empty(m, K.gemv_sumsq_parts(n, k) if gemv else K.gemm_skinny_sumsq_parts(n), device=dev)
         nw = torch.ones(n, device=dev).bfloat16()
-        calls = [lambda w=w: K.gemm_skinny(x, w, None, hidden=hidden, next_weight=nw, scaled_out=scaled, sumsq_out=ss)
+        calls = [lambda w=w: product(x, w, None, hidden=hidden, next_weight=nw, scaled_out=scaled, sumsq_out=ss)
                  for w in tiled]
     elif mode == "swiglu":
         out = torch.empty(m, n // 2, device=dev).bfloat16()
-        calls = [lambda w=w: K.gemm_skinny(x, w, out, swiglu=True) for w in tiled]
+        calls = [lambda w=w: product(x, w, out, swiglu=True) for w in tiled]
     else:
         out = torch.empty(m, n, device=dev, dtype=torch.float32 if mode == "f32" else torch.bfloat16)
-        calls = [lambda w=w: K.gemm_skinny(x, w, out) for w in tiled]
-    us = _time(calls, args.reps)
-    line = f"gemm {args.shape:8s} rows {m:3d} [{n} x {k}] few-rows kernel {us:8.2f} us  {n * k * 2 / us / 1e6:6.2f} TB/s of weights"
+        calls = [lambda w=w: product(x, w, out) for w in tiled]
+    us = _time_in_graph(calls, args.reps) if args.graph else _time(calls, args.reps)
+    name = "matrix-vector kernel" if gemv else "few-rows kernel"
+    line = f"gemm {args.shape:8s} rows {m:3d} [{n} x {k}] {name} {us:8.2f} us  {n * k * 2 / us / 1e6:6.2f} TB/s of weights"
     if args.vendor:
         out_v = torch.empty(m, n, device=dev, dtype=torch.bfloat16)
         us_v = _time([lambda w=w: K.gemm_vendor(x, w, out_v) for w in ws], args.reps)
@@ -237,6 +242,9 @@ def main(argv=None) -> int:
     g.add_argument("--shape", choices=sorted(GEMM_SHAPES), default="gate_up")
     g.add_argument("--rows", type=int, default=8)
     g.add_argument("--vendor", action="store_true", help="also time the vendor GEMM on the plain weight")
+    g.add_argument("--kernel", choices=["few-rows", "gemv"], default="few-rows",
+                   help="the matrix-core kernel over the tiled weight, or the matrix-vector kernel (one or two rows)")
+    g.add_argument("--graph", action="store_true", help="time the launches inside a captured graph")
     g.add_argument("--reps", type=int, default=48)
     pr = sub.add_parser("prompt")
     pr.add_argument("--tokens", type=int, default=8192)
