@@ -104,7 +104,8 @@ def main(argv=None) -> int:
     ap.add_argument("--gemm-tune-rows", default="auto",
                     help="comma list of row counts (tokens per step) for which the vendor GEMM library's "
                          "algorithms are timed at start-up (a few seconds); smaller row counts down to half "
-                         "share what is found.  'auto': the number of seats when above 16; '' for none")
+                         "share what is found.  'auto': the powers of two from 32 up to the number of seats, "
+                         "and that number; '' for none")
     args = ap.parse_args(argv)
     if not args.model_dir:
         print("no model folder: pass it as the first argument or set MODEL_DIR", file=sys.stderr)
@@ -130,12 +131,13 @@ def main(argv=None) -> int:
 
     from ..engine.engine import Engine, EngineOptions
     from ..engine.runner import Runner, ServeOptions
+    from ..ops.gemm_bf16 import decode_tune_rows
 
     engine = Engine(args.model_dir, EngineOptions(
         dtype=args.dtype, cache_mode=args.cache_mode, page_size=args.page_size, max_seqs=args.max_seqs,
         max_seq_len=args.max_seq_len, cache_tokens=args.cache_tokens, max_batch_tokens=args.max_batch_tokens,
         max_logit_rows=args.max_seqs,         # one sampled token per request and step
-        gemm_tune_rows=([args.max_seqs] if args.max_seqs > 16 else []) if args.gemm_tune_rows == "auto"
+        gemm_tune_rows=decode_tune_rows(args.max_seqs) if args.gemm_tune_rows == "auto"
         else [int(r) for r in args.gemm_tune_rows.split(",") if r.strip()]))
     runner = Runner(engine, ServeOptions(
         temperature=temperature, sampling_seed=seed, ignore_eos=ignore_eos, repetition_penalty=penalty,

@@ -64,6 +64,7 @@ def run_one(args, shape: str, batch: int, mode: str) -> dict:
     import torch
     from ..engine.engine import Engine, EngineOptions
     from ..engine.runner import Runner, ServeOptions
+    from ..ops.gemm_bf16 import decode_tune_rows
 
     cfg = dict(SHAPES[shape]) if shape in SHAPES else json.load(open(shape))
     full_layers = cfg["num_hidden_layers"]
@@ -81,7 +82,7 @@ def run_one(args, shape: str, batch: int, mode: str) -> dict:
                                         cache_tokens=pool, max_seqs=seats, max_seq_len=longest,
                                         use_graphs=not args.no_graphs,
                                         max_batch_tokens=max(8192, args.max_batch_tokens), max_logit_rows=seats,
-                                        gemm_tune_rows=[seats] if args.tune_gemm and seats > 16 else []),
+                                        gemm_tune_rows=decode_tune_rows(seats) if args.tune_gemm else []),
                     config_dict=cfg, random_seed=args.seed)
     runner = Runner(engine, ServeOptions(ignore_eos=True, max_batch_tokens=args.max_batch_tokens,
                                          chunk_size=args.chunk_size, reserve_policy=args.reserve_policy,

@@ -55,6 +55,22 @@ def use_gemv(m: int, n: int, k: int) -> bool:
     return m <= GEMV_MAX_ROWS and K.gemv_supported(m, n, k)
 
 
+def decode_tune_rows(max_rows: int) -> list:
+    """Row counts for which a server with ``max_rows`` seats has the vendor library's algorithms
+    timed at start-up: the powers of two from 32 and ``max_rows`` itself.  A row count that was not
+    timed takes what was found for the nearest timed one above it, up to twice its size, so these
+    cover every decode batch above the few-rows kernels' 16 (a shape costs a fraction of a second;
+    decode steps of 17 / 24 / 32 requests at the 1B sizes: 1.22 / 1.27 / 1.36 ms with the library's
+    own choice, 1.19 / 1.25 / 1.31 with 32 rows timed)."""
+    rows, r = [], 32
+    while r < max_rows:
+        rows.append(r)
+        r *= 2
+    if max_rows > SKINNY_MAX_ROWS:
+        rows.append(int(max_rows))
+    return rows
+
+
 def linear_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, tiled=None) -> torch.Tensor:
     """``tiled`` is the weight's :class:`~.kernels.TiledWeight` when it has one."""
     if not (x.is_cuda and w.is_cuda and out.is_cuda):

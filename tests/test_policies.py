@@ -48,3 +48,16 @@ def test_pool_from_leftover_memory():
         pool_pages_from_memory(3 * GiB, page_bytes, page_size=16, max_seqs=8, max_seq_len=8192,
                                margin_bytes=2 * GiB, step_bytes=2 * GiB)
     assert "no room for a cache pool" in str(e.value)
+
+
+def test_row_counts_timed_for_decode_batches_cover_every_batch_above_the_few_rows_kernels():
+    """Every batch from 17 seats up to the largest has a timed row count at or above it and at
+    most twice its size (the sharing rule of the vendor product's plans)."""
+    from kv_cache_optimization_for_llm_amd.ops.gemm_bf16 import decode_tune_rows
+    assert decode_tune_rows(1) == [] and decode_tune_rows(16) == []
+    assert decode_tune_rows(17) == [17] and decode_tune_rows(32) == [32]
+    assert decode_tune_rows(64) == [32, 64] and decode_tune_rows(100) == [32, 64, 100]
+    for seats in (17, 40, 64, 200, 384):
+        rows = decode_tune_rows(seats)
+        for batch in range(17, seats + 1):
+            assert any(batch <= r <= 2 * batch for r in rows), (seats, batch)
