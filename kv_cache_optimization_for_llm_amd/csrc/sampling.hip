@@ -21,6 +21,7 @@
 #include <math.h>
 
 #define SAMPLE_THREADS 256
+#define SCAN_IN_FLIGHT 8
 #define SAMPLE_MAX_CHUNKS 1024
 #define PICK_CHUNKS_PER_LANE (SAMPLE_MAX_CHUNKS / KVA_WAVE)
 
@@ -138,10 +139,25 @@ sample_scan_kernel(const float *__restrict__ logits, int vocab, int chunk_tokens
     const bool sampled = inv_t > 0.f;
     Best b{-INFINITY, vocab};
     Online o{-INFINITY, 0.f};
-    for (int t = begin + threadIdx.x; t < end; t += SAMPLE_THREADS) {
-        const float l = penalised(rl[t], mk, t, penalty);
-        b = better(b, Best{l, t});
-        if (sampled) o.add(l, inv_t);
+    // A thread's tokens in turns of SCAN_IN_FLIGHT, every load of a turn asked for before the first
+    // is used (a plain loop over a thread's four or eight tokens is a trip to memory each).
+    for (int base = begin + threadIdx.x; base < end; base += SCAN_IN_FLIGHT * SAMPLE_THREADS) {
+        float l[SCAN_IN_FLIGHT];
+        unsigned char marked[SCAN_IN_FLIGHT];
+#pragma unroll
+        for (int j = 0; j < SCAN_IN_FLIGHT; ++j) {
+            const int t = base + j * SAMPLE_THREADS;
+            l[j] = rl[t < end ? t : end - 1];
+            marked[j] = mk != nullptr ? mk[t < end ? t : end - 1] : (unsigned char)0;
+        }
+#pragma unroll
+        for (int j = 0; j < SCAN_IN_FLIGHT; ++j) {
+            const int t = base + j * SAMPLE_THREADS;
+            if (t >= end) break;
+            const float v = marked[j] != 0 ? (l[j] > 0.f ? l[j] / penalty : l[j] * penalty) : l[j];
+            b = better(b, Best{v, t});
+            if (sampled) o.add(v, inv_t);
+        }
     }
     b = wave_best(b);
     if (sampled) {
