@@ -25,21 +25,27 @@ from . import kernels as K
 #   rows the vendor GEMM wins everywhere because the few-rows kernel re-reads X once per 16 rows of W;
 # * the vocabulary-sized product (4 row tiles of W per wave share each X fragment, fp32 output
 #   without a cast) wins up to 48 rows.
+# Where "small" ends, whole decode steps of 17 / 24 / 32 requests at the 3B and 8B layer sizes: the
+# output projection by the few-rows kernel, 3,072 x 3,072: 2.80 / 2.94 / 3.04 -> 2.74 / 2.89 / 3.02
+# ms; 4,096 x 4,096: 4.55 / 4.75 / 4.91 -> 4.62 / 4.82 / 5.03.  The Q/K/V product with rotation and
+# cache write in its epilogue (it stands for the library's product and the rotation kernel) gains
+# at both: 3B 2.80 -> 2.77 (5,120 x 3,072), 8B 4.55 -> 4.52 (6,144 x 4,096).
 SKINNY_MAX_ROWS = 16            # every shape
-SKINNY_MID_ROWS = 32            # small or tall matrices
-SKINNY_MID_ELEMENTS = 1 << 23
+SKINNY_MID_ROWS = 32            # small or tall matrices, and the Q/K/V product with its epilogue
+SKINNY_MID_ELEMENTS = 3 << 22
 SKINNY_WIDE_ROWS = 64           # matrices whose waves share X through LDS
 SKINNY_WIDE_N = 32768
 
 
-def use_skinny(m: int, n: int, k: int, gated: bool = False) -> bool:
+def use_skinny(m: int, n: int, k: int, gated: bool = False, rotated: bool = False) -> bool:
     """``gated``: the weight is a joined [gate; up] matrix whose product is taken with the
-    activation fused."""
+    activation fused; ``rotated``: a joined [q; k; v] matrix whose product is taken with rotation
+    and cache write fused."""
     if not K.gemm_skinny_supported(m, n, k):
         return False
     if m <= SKINNY_MAX_ROWS:
         return True
-    if m <= SKINNY_MID_ROWS and (n * k <= SKINNY_MID_ELEMENTS or n >= 4 * k):
+    if m <= SKINNY_MID_ROWS and (rotated or n * k <= SKINNY_MID_ELEMENTS or n >= 4 * k):
         return True
     return m <= SKINNY_WIDE_ROWS and (n >= SKINNY_WIDE_N or (gated and n >= 4 * k))
 

@@ -39,7 +39,7 @@ class EncodedQKV:
         are the position-encoded queries; K (encoded) and V of the step's tokens are in the cache
         when ``kv`` allows writing."""
         tables, rows = None, x.shape[0]
-        kernel = self.linear.fused_kernel(rows, x.dtype)
+        kernel = self.linear.fused_kernel(rows, x.dtype, rotated=True)
         if kernel == Linear.GEMV and not K.gemv_qkv_rope_supported(rows, self.hidden_size, self.head_dim):
             kernel = Linear.FEW_ROWS if self.linear.tiled is not None else None
         if kernel == Linear.FEW_ROWS and not K.gemm_skinny_qkv_rope_supported(rows, self.hidden_size, self.head_dim):

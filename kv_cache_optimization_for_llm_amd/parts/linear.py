@@ -35,16 +35,18 @@ class Linear:
 
     GEMV, FEW_ROWS = "gemv", "few_rows"
 
-    def fused_kernel(self, rows: int, dtype) -> Optional[str]:
+    def fused_kernel(self, rows: int, dtype, rotated: bool = False) -> Optional[str]:
         """The hand-written product that takes ``rows`` rows of ``dtype`` with a norm on its input
         and/or the residual stream in its epilogue: ``GEMV`` (one token: a matrix-vector product
-        over the plain weight), ``FEW_ROWS`` (the matrix-core kernel over the tiled copy) or None."""
+        over the plain weight), ``FEW_ROWS`` (the matrix-core kernel over the tiled copy) or None.
+        ``rotated``: the product asked about is the joined Q/K/V product with rotation and cache
+        write in its epilogue."""
         from ..ops.gemm_bf16 import use_gemv, use_skinny
         if dtype != torch.bfloat16 or self.weight.dtype != torch.bfloat16 or not self.weight.is_cuda:
             return None
         if use_gemv(rows, self.out_features, self.in_features):
             return self.GEMV
-        if self.tiled is not None and use_skinny(rows, self.out_features, self.in_features, self.halves == 2):
+        if self.tiled is not None and use_skinny(rows, self.out_features, self.in_features, self.halves == 2, rotated):
             return self.FEW_ROWS
         return None
 
