@@ -107,14 +107,16 @@ def main():
     dev = engine.device
     gen = torch.Generator().manual_seed(0)
 
-    def decode_run(batch, steps, warmup, context):
+    def decode_run(batch, steps, warmup, context, decoded_before=0):
         """Times ``steps`` decode steps of ``batch`` requests through the serving loop (scheduler,
         step function, sampler; a step is launched while the host still waits for the previous
         step's tokens).  The prompts are prefilled first, in portions; their lengths are set so
-        that the longest context ENDS at ``context``.  Returns (seconds, mean context length
-        over the timed steps)."""
+        that the longest context ENDS at ``context``.  ``decoded_before``: the requests have been
+        decoding for that many steps when the warm-up steps begin.  Returns (seconds, mean
+        context length over the timed steps)."""
         budget = 32768
         runner = Runner(engine, ServeOptions(ignore_eos=True, run_ahead=True, max_batch_tokens=budget))
+        warmup += decoded_before
         lead = warmup + steps + 2
         first = context - lead
         first -= (batch * first + budget - 1) // budget + 1      # steps that other requests' prompts take
@@ -185,6 +187,17 @@ def main():
             k = max(16, args.steps // 2)
             d, c = decode_run(b, k, 8, ctx)
             add_point(f"decode_b{b}", b, k, d, c)
+        # The default run again, with the requests 320 steps into their decoding when the same warm-up
+        # and the same timed steps begin.  After a prefill (seconds of matrix products that ask
+        # little of the memory) the first third of a second of decode steps runs 6-7 % slower than
+        # all that follow: every kernel that streams weights takes 0.5-1 us longer, until the
+        # memory has been busy for that long (one run of 8 x 8,192, 40 steps at a time: 1.227 ms
+        # seven times, then 1.169, 1.150, 1.149 ..; kernel by kernel in a trace: down and output
+        # 8.9 -> 7.9 us, gate/up 14.1 -> 13.1, Q/K/V 7.9 -> 7.4, attention 25.4 -> 24.8).  A server
+        # that decodes is past that point; the default run, timed right after its prompts, is not.
+        if ctx >= 320 + args.warmup + args.steps + 64:
+            d, c = decode_run(args.batch, args.steps, args.warmup, ctx, decoded_before=320)
+            add_point(f"decode_b{args.batch}_sustained", args.batch, args.steps, d, c)
         # the serving workload of the comparison: 512-token prompts, 256 generated tokens
         for b in (1, 8, 64):
             d, c = decode_run(b, 240, 8, 512 + 256)
