@@ -38,6 +38,9 @@
 #include <math.h>
 
 // STREAM: keys and values are loaded with the non-temporal hint (see load_block).
+// a wavefront's key range from which a third block of keys is kept in flight (decoded tokens)
+#define LONG_RANGE_KEYS 1536
+
 template <int D, int RT, bool FAST, bool STREAM>
 __device__ __forceinline__ void
 attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
@@ -316,17 +319,35 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
         else compute_block_as(std::false_type{}, f, kstart);
     };
 
-    // Two blocks in flight (a third does not pay: the waits are for bandwidth, not latency).  The
+    // Two blocks in flight; three for a decoded token's wavefront that walks all of a long context
+    // alone (few wavefronts, each a long stream: decode steps of 48 requests at 8,192 keys 3.78 ->
+    // 3.56 ms, 64 requests 4.02 -> 3.88, 48 at 2,048 keys 1.86 -> 1.81; short ranges lose 1 % by it,
+    // wavefronts that share a context in splits 3 % - there are a thousand of them and the third set of
+    // registers costs them their place - and prompt items wait for the softmax's vector work, not
+    // for memory).  The
     // loads are issued unconditionally (a block past the end is
     // redirected or predicated off inside load_block and its values are never used): a load
     // under a branch would make the wait before the next product a wait for everything.
     BlockFrags fa, fb;
     load_block(fa, k_begin);
-    for (int kstart = k_begin; kstart < k_end; kstart += 64) {
-        load_block(fb, kstart + 32);
-        compute_block(fa, kstart);
-        load_block(fa, kstart + 64);
-        if (kstart + 32 < k_end) compute_block(fb, kstart + 32);
+    if (RT == 1 && STREAM && D <= 128 && splits == 1 && k_end - k_begin >= LONG_RANGE_KEYS) {   // (a third set of registers spills from 224 on)
+        BlockFrags fc;
+        load_block(fb, k_begin + 32);
+        for (int kstart = k_begin; kstart < k_end; kstart += 96) {
+            load_block(fc, kstart + 64);
+            compute_block(fa, kstart);
+            load_block(fa, kstart + 96);
+            if (kstart + 32 < k_end) compute_block(fb, kstart + 32);
+            load_block(fb, kstart + 128);
+            if (kstart + 64 < k_end) compute_block(fc, kstart + 64);
+        }
+    } else {
+        for (int kstart = k_begin; kstart < k_end; kstart += 64) {
+            load_block(fb, kstart + 32);
+            compute_block(fa, kstart);
+            load_block(fa, kstart + 64);
+            if (kstart + 32 < k_end) compute_block(fb, kstart + 32);
+        }
     }
 
     // lane (r, g) holds O[row r][dt * 16 + 4g + i]
