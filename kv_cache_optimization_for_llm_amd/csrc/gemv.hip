@@ -1,4 +1,7 @@
 // y = x W^T for one or two tokens: matrix-vector products that stream the row-major weight once.
+// Stands where the reference's decode step calls cublasGemmEx with one column per active row
+// (base/src/engine.cu:1040-1117, 1141-1159, 1166-1253) followed by its norm, rotation, activation
+// and residual kernels (base/src/kernels.cu:10-52, 227-275).
 //
 // For one or two tokens the matrix cores have nothing to reuse, and what bounds the product is how
 // soon a wavefront has asked for all of its bytes and how short the chain is from the last byte's
