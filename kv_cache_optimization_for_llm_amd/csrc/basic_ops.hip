@@ -172,16 +172,40 @@ extern "C" int kva_embed_gather_prep(void *hidden, void *scaled, float *sumsq, c
 }
 
 #define RMS_VEC_CACHE 4   // vectors of 8 a thread keeps between the passes
+// 8 elements of the branch output that is added to the stream: from the bf16 delta, or (parts > 0)
+// the sum of `parts` fp32 partial products [parts][rows][width], rounded to bf16 as the product
+// itself would have been
+__device__ inline void load_delta8(const bf16_t *dl, const float *parts_row, int parts, size_t part_stride, int i,
+                                   float (&d)[8]) {
+    if (parts > 0) {
+        float4 lo = make_float4(0.f, 0.f, 0.f, 0.f), hi = lo;
+        for (int s = 0; s < parts; ++s) {
+            const float4 a = *reinterpret_cast<const float4 *>(parts_row + (size_t)s * part_stride + i);
+            const float4 b = *reinterpret_cast<const float4 *>(parts_row + (size_t)s * part_stride + i + 4);
+            lo.x += a.x; lo.y += a.y; lo.z += a.z; lo.w += a.w;
+            hi.x += b.x; hi.y += b.y; hi.z += b.z; hi.w += b.w;
+        }
+        const float f[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) d[j] = bf16_bits_to_float(float_to_bf16_bits(f[j]));
+    } else {
+        unpack8(*reinterpret_cast<const uint4 *>(dl + i), d);
+    }
+}
+
 template <typename TW>
 __global__ void rmsnorm_vec_kernel(bf16_t *__restrict__ out, bf16_t *__restrict__ hidden,
-                                   const bf16_t *__restrict__ delta, const TW *__restrict__ weight,
+                                   const bf16_t *__restrict__ delta, const float *__restrict__ delta_parts,
+                                   int parts, size_t part_stride, const TW *__restrict__ weight,
                                    const int *__restrict__ row_idx, int width, float eps) {
     __shared__ float scratch[16];
     const int orow = blockIdx.x;
     const int irow = row_idx ? row_idx[orow] : orow;
     bf16_t *x = hidden + (size_t)irow * width;
     const bf16_t *dl = delta ? delta + (size_t)irow * width : nullptr;
-    const bool write_back = dl && !row_idx;
+    const float *pr = parts > 0 ? delta_parts + (size_t)irow * width : nullptr;
+    const bool adds = dl != nullptr || parts > 0;
+    const bool write_back = adds && !row_idx;
     bf16_t *y = out + (size_t)orow * width;
     float cache[RMS_VEC_CACHE][8];
     float ss = 0.f;
@@ -189,9 +213,9 @@ __global__ void rmsnorm_vec_kernel(bf16_t *__restrict__ out, bf16_t *__restrict_
     for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8, ++c) {
         float v[8];
         unpack8(*reinterpret_cast<const uint4 *>(x + i), v);
-        if (dl) {
+        if (adds) {
             float d[8];
-            unpack8(*reinterpret_cast<const uint4 *>(dl + i), d);
+            load_delta8(dl, pr, parts, part_stride, i, d);
 #pragma unroll
             for (int j = 0; j < 8; ++j) v[j] = bf16_bits_to_float(float_to_bf16_bits(v[j] + d[j]));
             if (write_back) *reinterpret_cast<uint4 *>(x + i) = pack8(v);
@@ -213,9 +237,9 @@ __global__ void rmsnorm_vec_kernel(bf16_t *__restrict__ out, bf16_t *__restrict_
             for (int j = 0; j < 8; ++j) v[j] = cache[c][j];
         } else {
             unpack8(*reinterpret_cast<const uint4 *>(x + i), v);
-            if (dl && !write_back) {
+            if (adds && !write_back) {
                 float d[8];
-                unpack8(*reinterpret_cast<const uint4 *>(dl + i), d);
+                load_delta8(dl, pr, parts, part_stride, i, d);
 #pragma unroll
                 for (int j = 0; j < 8; ++j) v[j] = bf16_bits_to_float(float_to_bf16_bits(v[j] + d[j]));
             }
@@ -227,22 +251,29 @@ __global__ void rmsnorm_vec_kernel(bf16_t *__restrict__ out, bf16_t *__restrict_
     }
 }
 
+// delta_parts (bf16 rows of a width that is a multiple of 8 only): instead of delta, `parts` fp32
+// partial products [parts][part_rows][width] whose sum, rounded to bf16, is what is added.
 extern "C" int kva_rmsnorm(void *out, void *hidden, const void *delta, const void *weight,
                            const int *row_idx, int out_rows, int width, float eps, int dtype,
-                           int weight_dtype, hipStream_t stream) {
+                           int weight_dtype, const float *delta_parts, int parts, int part_rows,
+                           hipStream_t stream) {
     KVA_REQUIRE(out_rows >= 0 && width > 0, "rmsnorm: bad sizes rows=%d width=%d", out_rows, width);
+    KVA_REQUIRE(parts == 0 || (delta_parts != nullptr && delta == nullptr && parts > 0 && part_rows > 0 &&
+                               dtype == KVA_BF16 && width % 8 == 0),
+                "rmsnorm: partial products stand in for a bf16 delta of a width that is a multiple of 8");
     if (out_rows == 0) return KVA_OK;
     if (dtype == KVA_BF16 && width % 8 == 0) {
         const int threads = width >= 8192 ? 1024 : (width >= 2048 ? 256 : (width >= 1024 ? 128 : 64));
         dim3 vgrid(out_rows), vblock(threads);
+        const size_t part_stride = (size_t)part_rows * width;
         if (weight_dtype == KVA_BF16)
             hipLaunchKernelGGL(rmsnorm_vec_kernel<bf16_t>, vgrid, vblock, 0, stream, (bf16_t *)out,
-                               (bf16_t *)hidden, (const bf16_t *)delta, (const bf16_t *)weight, row_idx,
-                               width, eps);
+                               (bf16_t *)hidden, (const bf16_t *)delta, delta_parts, parts, part_stride,
+                               (const bf16_t *)weight, row_idx, width, eps);
         else if (weight_dtype == KVA_F32)
             hipLaunchKernelGGL(rmsnorm_vec_kernel<float>, vgrid, vblock, 0, stream, (bf16_t *)out,
-                               (bf16_t *)hidden, (const bf16_t *)delta, (const float *)weight, row_idx,
-                               width, eps);
+                               (bf16_t *)hidden, (const bf16_t *)delta, delta_parts, parts, part_stride,
+                               (const float *)weight, row_idx, width, eps);
         else KVA_REQUIRE(false, "rmsnorm: unsupported weight dtype %d", weight_dtype);
         KVA_CHECK_LAUNCH("rmsnorm");
         return KVA_OK;

@@ -89,6 +89,10 @@ struct SkinnyArgs {
     // same 8 columns of four neighbouring rows, then take 64 contiguous bytes; row-major they take
     // four pieces 2 K bytes apart).  A private layout between two products of one part.
     int x_tiled, y_tiled;
+    // K cut into k_slices ranges, one per blockIdx.y, each leaving its own fp32 partial product
+    // [M, N] in Y (slice s at Y + s * M * ldy): for matrices with too few tiles to fill the chip
+    // with whole-K workgroups when the rows go through LDS (see kva_gemm_skinny_partials)
+    int k_slices;
 };
 
 // XL: the waves of a workgroup that work on the same K range (one per tile group) share X through
@@ -127,8 +131,9 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
         rope_rotated = rope_head < a.nq + a.nkv;
     }
     const int K = a.K;
-    const int kper = K / k_waves;
-    const int kbeg = kpart * kper, kend = kbeg + kper;
+    const int kslice = K / a.k_slices;
+    const int kper = kslice / k_waves;
+    const int kbeg = (int)blockIdx.y * kslice + kpart * kper, kend = kbeg + kper;
 
     // W is stored tiled: [n-tile][K / 32][g][r][8 of K], so the 1 KiB a wave needs per step is
     // contiguous, in the order of its lanes (lane r + 16 g takes bytes 16 (r + 16 g) ..), and a
@@ -666,7 +671,7 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
             }
             if (!m_ok || !lane_on) continue;
             if (a.out_f32) {
-                float *dst = reinterpret_cast<float *>(a.Y) + (size_t)m * a.ldy + n;
+                float *dst = reinterpret_cast<float *>(a.Y) + ((size_t)blockIdx.y * a.M + m) * a.ldy + n;
                 if (n + 3 < rows && (a.ldy % 4 == 0)) {
                     *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
                 } else {
@@ -776,7 +781,7 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
                 "gemm_skinny: the residual epilogue needs hidden, scaled_out and sumsq_out");
     SkinnyArgs a = {};
     a.X = (const bf16_t *)X; a.W = (const bf16_t *)W; a.Y = Y;
-    a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldy = ldy;
+    a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldy = ldy; a.k_slices = 1;
     a.inter = mode == 2 ? N / 2 : 0;
     a.out_f32 = mode == 1 ? 1 : 0;
     a.sumsq = sumsq; a.sumsq_parts = sumsq_parts; a.norm_width = norm_width; a.eps = eps;
@@ -858,7 +863,7 @@ extern "C" int kva_gemm_skinny_qkv_rope(void *q_out, int ldq, const void *X, con
                 "gemm_skinny_qkv_rope: row scaling needs a part count and the norm's width");
     SkinnyArgs a = {};
     a.X = (const bf16_t *)X; a.W = (const bf16_t *)W; a.Y = q_out;
-    a.M = M; a.N = (nq + 2 * nkv) * head_dim; a.K = K; a.ldx = ldx; a.ldy = ldq;
+    a.M = M; a.N = (nq + 2 * nkv) * head_dim; a.K = K; a.ldx = ldx; a.ldy = ldq; a.k_slices = 1;
     a.sumsq = sumsq; a.sumsq_parts = sumsq_parts; a.norm_width = norm_width; a.eps = eps;
     a.cos_t = cos_t; a.sin_t = sin_t; a.positions = positions; a.slots = slots;
     a.k_cache = (bf16_t *)k_cache; a.v_cache = (bf16_t *)v_cache;
@@ -888,5 +893,43 @@ extern "C" int kva_gemm_skinny_qkv_rope(void *q_out, int ldq, const void *X, con
     if (xl) launch_xl<2, EPI_ROPE>(a, grid, block, lds, stream);
     else launch_mt<2, EPI_ROPE>(a, grid, block, lds, stream);
     KVA_CHECK_LAUNCH("gemm_skinny_qkv_rope");
+    return KVA_OK;
+}
+
+// How many K ranges kva_gemm_skinny_partials cuts a product into (0: it does not take the shape).
+// Two tiles of W per wavefront, two wavefronts per K range and two K ranges per workgroup share
+// their rows of X through LDS; the ranges across workgroups are as many as fill the compute units
+// while a range keeps at least 256 columns.
+extern "C" int kva_gemm_skinny_partial_slices(int M, int N, int K) {
+    if (M <= 16 || M > 64 || N < 32 || K % 128 != 0) return 0;
+    const int n_tiles = (N + 15) / 16;
+    const int groups = (n_tiles + 1) / 2;
+    const int wgs = (groups + 1) / 2;
+    int slices = 1;
+    while (wgs * slices * 2 <= compute_units() && K % (slices * 2 * 128) == 0 && K / (slices * 2) >= 256) slices *= 2;
+    return slices;
+}
+
+// P[s][M][N] (fp32) = X[:, range s of K] W[:, range s]^T for s in [0, slices): partial products for a
+// kernel that adds them up and does what follows the product (residual and norm).  W: the tiled copy.
+extern "C" int kva_gemm_skinny_partials(float *P, const void *X, const void *W, int M, int N, int K, int ldx,
+                                        int slices, hipStream_t stream) {
+    KVA_REQUIRE(slices >= 1 && slices == kva_gemm_skinny_partial_slices(M, N, K),
+                "gemm_skinny_partials: M=%d N=%d K=%d is not taken in %d ranges", M, N, K, slices);
+    KVA_REQUIRE(ldx >= K && ldx % 8 == 0, "gemm_skinny_partials: X row stride %d must be a multiple of 8 and >= K", ldx);
+    SkinnyArgs a = {};
+    a.X = (const bf16_t *)X; a.W = (const bf16_t *)W; a.Y = P;
+    a.M = M; a.N = N; a.K = K; a.ldx = ldx; a.ldy = N; a.k_slices = slices;
+    a.out_f32 = 1;
+    const int n_tiles = (N + 15) / 16;
+    const int groups = (n_tiles + 1) / 2;
+    a.k_waves = 2;
+    const int groups_per_wg = 2, waves = 4;
+    const size_t stage = (size_t)a.k_waves * 2 * ((M + 15) / 16 * 16) * 128;
+    const size_t sums = (size_t)waves * 2 * 64 * 4 * sizeof(float);
+    const size_t lds = stage > sums ? stage : sums;
+    dim3 grid((groups + groups_per_wg - 1) / groups_per_wg, slices), block(64 * waves);
+    launch_xl<2, EPI_PLAIN>(a, grid, block, lds, stream);
+    KVA_CHECK_LAUNCH("gemm_skinny_partials");
     return KVA_OK;
 }

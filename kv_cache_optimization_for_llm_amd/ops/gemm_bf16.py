@@ -50,6 +50,13 @@ def use_skinny(m: int, n: int, k: int, gated: bool = False, rotated: bool = Fals
     return m <= SKINNY_WIDE_ROWS and (n >= SKINNY_WIDE_N or (gated and n >= 4 * k))
 
 
+def use_partial_sums(m: int, n: int, k: int) -> bool:
+    """17 to 64 rows of a product that goes into the residual stream and that the few-rows kernel
+    does not take whole: its shared-X form over ranges of K (``kernels.gemm_skinny_partials``)
+    instead of the vendor library, the norm kernel adding the ranges up."""
+    return SKINNY_MAX_ROWS < m <= SKINNY_WIDE_ROWS and K.gemm_skinny_partial_ranges(m, n, k) >= 1
+
+
 # One or two tokens go to the matrix-vector kernel over the plain weight (csrc/gemv.hip): measured
 # inside a graph at the 1B sizes with the epilogues the model uses, one token, it takes 5.5 / 4.2 /
 # 12.6 / 8.6 microseconds for Q/K/V, output, gate/up and down against the few-rows kernel's 7.3 /

@@ -104,10 +104,38 @@ def embed_gather_prep(table: torch.Tensor, ids: torch.Tensor, hidden: torch.Tens
     return hidden
 
 
+class PartialSums:
+    """A branch output that has not been added up yet: ``parts`` fp32 ``[ranges, rows, width]``, the
+    products of :func:`gemm_skinny_partials` over ranges of K.  It stands where a bf16 ``[rows,
+    width]`` delta stands; the norm kernel that adds the delta to the stream adds the ranges first
+    (and rounds their sum to bf16, as the whole product would have been).  ``materialize()`` gives
+    the plain delta."""
+
+    def __init__(self, parts: torch.Tensor):
+        if parts.dim() != 3 or parts.dtype != torch.float32:
+            raise KernelError("PartialSums: fp32 [ranges, rows, width] needed")
+        self.parts = parts
+
+    @property
+    def shape(self):
+        return self.parts.shape[1:]
+
+    @property
+    def dtype(self):
+        return torch.bfloat16
+
+    @property
+    def device(self):
+        return self.parts.device
+
+    def materialize(self) -> torch.Tensor:
+        return self.parts.sum(0).to(torch.bfloat16)
+
+
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
-            delta: Optional[torch.Tensor] = None, row_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out = rmsnorm(x) * weight.  With ``delta``: x += delta first (in place, fp32 add).  With
-    ``row_idx``: out[i] = rmsnorm(x[row_idx[i]])."""
+            delta=None, row_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = rmsnorm(x) * weight.  With ``delta`` (a tensor like x, or :class:`PartialSums`): x +=
+    delta first (in place, fp32 add).  With ``row_idx``: out[i] = rmsnorm(x[row_idx[i]])."""
     width = x.shape[-1]
     out_rows = out.shape[0]
     if x.dim() != 2 or out.dim() != 2 or out.shape[1] != width or weight.shape != (width,):
@@ -120,12 +148,19 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
             raise KernelError("rmsnorm: out needs as many rows as x")
     elif row_idx.shape != (out_rows,):
         raise KernelError("rmsnorm: one row index per output row")
+    parts = None
+    if isinstance(delta, PartialSums):
+        if tuple(delta.shape) != tuple(x.shape) or x.dtype != torch.bfloat16 or width % 8:
+            raise KernelError("rmsnorm: partial sums stand in for a bf16 delta of x's shape, width a multiple of 8")
+        parts, delta = delta.parts, None
     if delta is not None and (delta.shape != x.shape or delta.dtype != x.dtype):
         raise KernelError("rmsnorm: delta must match x")
     check(hip_lib().kva_rmsnorm(_dev(out, "out"), _dev(x, "x"), _opt(delta, "delta"),
                                 _dev(weight, "weight"), _opt(row_idx, "row_idx", torch.int32),
                                 out_rows, width, float(eps), dtype_code(x.dtype),
-                                dtype_code(weight.dtype), _stream()), "rmsnorm")
+                                dtype_code(weight.dtype), _opt(parts, "partial sums", torch.float32),
+                                parts.shape[0] if parts is not None else 0,
+                                parts.shape[1] if parts is not None else 0, _stream()), "rmsnorm")
     return out
 
 
@@ -620,6 +655,30 @@ def gemm_skinny(x: torch.Tensor, w: TiledWeight, out: Optional[torch.Tensor], sw
                               None, None, 0, None, None, 1 if x_tiled else 0, 1 if out_tiled else 0, _stream()),
           "gemm_skinny")
     return out
+
+
+def gemm_skinny_partial_ranges(m: int, n: int, k: int) -> int:
+    """Into how many ranges of K :func:`gemm_skinny_partials` cuts an [n, k] product of ``m`` rows;
+    0: it does not take the shape (it takes 17 to 64 rows, K a multiple of 128)."""
+    return int(hip_lib().kva_gemm_skinny_partial_slices(int(m), int(n), int(k)))
+
+
+def gemm_skinny_partials(x: torch.Tensor, w: "TiledWeight") -> PartialSums:
+    """x @ W^T for 17 to 64 rows as fp32 partial products over ranges of K, one per group of
+    workgroups, so that a matrix with few rows of tiles still fills the chip while the rows of x go
+    through LDS; whoever takes the :class:`PartialSums` adds them up."""
+    if not isinstance(w, TiledWeight) or w.halves != 1:
+        raise KernelError("gemm_skinny_partials: the weight must be a plain TiledWeight")
+    m, k = x.shape
+    if x.dtype != torch.bfloat16 or k != w.k:
+        raise KernelError(f"gemm_skinny_partials: bf16 x {tuple(x.shape)} does not fit weight [{w.n}, {w.k}]")
+    ranges = gemm_skinny_partial_ranges(m, w.n, k)
+    if ranges < 1:
+        raise KernelError(f"gemm_skinny_partials: {m} rows of a [{w.n}, {k}] product are not taken (17..64 rows, K % 128 == 0)")
+    parts = torch.empty((ranges, m, w.n), dtype=torch.float32, device=x.device)
+    check(hip_lib().kva_gemm_skinny_partials(_dev(parts, "parts"), _dev(x, "x"), _dev(w.data, "w"), m, w.n, k, k,
+                                             ranges, _stream()), "gemm_skinny_partials")
+    return PartialSums(parts)
 
 
 def gemm_skinny_qkv_rope_supported(m: int, k: int, head_dim: int) -> bool:

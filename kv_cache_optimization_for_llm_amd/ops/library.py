@@ -34,7 +34,7 @@ U = c_uint
 _HIP_SIGNATURES = {
     "kva_embed_gather": [P, P, P, P, I, I, I, I, P],
     "kva_embed_gather_prep": [P, P, P, P, P, P, P, I, I, I, P],
-    "kva_rmsnorm": [P, P, P, P, P, I, I, F, I, I, P],
+    "kva_rmsnorm": [P, P, P, P, P, I, I, F, I, I, P, I, I, P],
     "kva_residual_add": [P, P, LL, I, P],
     "kva_scale_softcap": [P, LL, F, F, I, P],
     "kva_stream_read": [P, LL, I, P, P],
@@ -50,6 +50,8 @@ _HIP_SIGNATURES = {
     "kva_attention_lds": [P, P, P, P, I, P, P, P, I, P, I, I, I, I, I, I, F, I, I, I, I, I, P],
     "kva_gemm_skinny": [P, P, P, I, I, I, I, I, I, P, I, I, F, P, P, I, P, P, I, I, P],
     "kva_gemm_skinny_sumsq_parts": [I],
+    "kva_gemm_skinny_partial_slices": [I, I, I],
+    "kva_gemm_skinny_partials": [P, P, P, I, I, I, I, I, P],
     "kva_normed_rows_finish": [P, P, P, I, I, P, I, F, P],
     "kva_gemm_skinny_supported": [I, I, I],
     "kva_gemm_skinny_qkv_rope_supported": [I, I, I],

@@ -115,7 +115,10 @@ class BranchTail:
     place) and the sum is handed to ``norm``, the norm that reads the stream next.  A mixer or
     feed-forward that is given a tail MAY do both inside its last product and return the
     :class:`NormedRows` prepared for ``norm``; returning its plain output instead is always
-    allowed (the block then adds and normalises itself)."""
+    allowed (the block then adds and normalises itself).  For a ``norm`` with
+    ``takes_partial_sums`` the output may also come back as ``ops.kernels.PartialSums`` (fp32
+    products over ranges of K, not yet added up): the block hands it to that norm as ``delta``
+    like a plain output."""
 
     hidden: torch.Tensor
     norm: object

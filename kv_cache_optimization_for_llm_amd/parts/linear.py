@@ -63,12 +63,15 @@ class Linear:
             return None
         return self.fused_kernel(rows, dtype)
 
-    def into_residual(self, x, tail: BranchTail) -> Optional[NormedRows]:
-        """hidden += x @ W^T in place and the sum prepared for ``tail.norm``; ``None`` when this
-        cannot be fused (the caller then takes the plain product)."""
+    def into_residual(self, x, tail: BranchTail):
+        """hidden += x @ W^T in place and the sum prepared for ``tail.norm`` (NormedRows); or, at
+        17 to 64 rows of a matrix that the few-rows kernel does not take whole, the product as
+        ``ops.kernels.PartialSums`` for a ``tail.norm`` that says it adds them up
+        (``takes_partial_sums``); ``None`` when neither is possible (the caller then takes the
+        plain product)."""
         kernel = self.residual_kernel(x.shape[0], x.dtype, tail)
         if kernel is None:
-            return None
+            return self._partial_sums(x, tail)
         next_w, width, eps = tail.norm.prepared_by_product()
         rows = x.shape[0]
         scaled = torch.empty((rows, self.out_features), dtype=torch.bfloat16, device=x.device)
@@ -89,6 +92,14 @@ class Linear:
             K.gemm_skinny(x, self.tiled, None, hidden=tail.hidden, next_weight=next_w, scaled_out=scaled,
                           sumsq_out=sumsq, x_tiled=isinstance(x, K.TiledRows), **norm)
         return NormedRows(scaled, sumsq, width, eps, tail.norm)
+
+    def _partial_sums(self, x, tail: Optional[BranchTail]):
+        from ..ops.gemm_bf16 import use_partial_sums
+        if tail is None or not getattr(tail.norm, "takes_partial_sums", False) or self.tiled is None \
+                or not isinstance(x, torch.Tensor) or x.dtype != torch.bfloat16 or tail.hidden.dtype != torch.bfloat16 \
+                or not use_partial_sums(x.shape[0], self.out_features, self.in_features):
+            return None
+        return K.gemm_skinny_partials(x, self.tiled)
 
     def gated(self, x, out) -> None:
         """``out`` = silu(x gate^T) * (x up^T) for a joined [gate; up] weight whose rows

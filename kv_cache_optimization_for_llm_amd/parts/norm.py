@@ -18,6 +18,7 @@ from .base import Norm
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
     graph_safe = True
+    takes_partial_sums = True       # ``delta`` may be ops.kernels.PartialSums (bf16 streams)
 
     def __init__(self, prefix: str, *, width: int, eps: float, weight_name: str = "weight"):
         super().__init__(prefix)
@@ -41,4 +42,6 @@ class RMSNorm(Norm):
         if out is None:
             rows = x.shape[0] if row_idx is None else row_idx.shape[0]
             out = torch.empty((rows, self.width), dtype=x.dtype, device=x.device)
+        if isinstance(delta, K.PartialSums) and (x.dtype != torch.bfloat16 or self.width % 8):
+            delta = delta.materialize()
         return K.rmsnorm(x, self.weight, self.eps, out, delta=delta, row_idx=row_idx)

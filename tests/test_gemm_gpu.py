@@ -227,6 +227,47 @@ def test_vendor_product_bf16_and_fp32_results(m, n, k, gpu):
             assert err <= tol, f"{dt}: {err:.3g}"
 
 
+@pytest.mark.parametrize("m", [17, 31, 48, 64])
+@pytest.mark.parametrize("n, k", [(2048, 8192), (2048, 2048), (100, 128), (389, 384), (48, 1024), (3072, 3072)])
+def test_partial_products_over_ranges_of_k_add_up_to_the_product(m, n, k, gpu):
+    """17 to 64 rows of a matrix with few rows of tiles: K is cut into ranges across workgroups
+    (as many as fill the chip; one for a small K), each range leaves an fp32 partial product, and
+    their sum is the product.  The norm kernel takes the ranges in place of a bf16 delta: the
+    stream and the normalised rows are bit for bit what the rounded sum gives.  Fewer rows, and
+    a K that 128 does not divide, are refused."""
+    ranges = K.gemm_skinny_partial_ranges(m, n, k)
+    assert ranges >= 1 and k % (ranges * 128) == 0
+    x, w = rnd(m, k), rnd(n, k, scale=0.05, seed=7)
+    want = x.double() @ w.double().t()
+    ps = K.gemm_skinny_partials(x.to(gpu), K.TiledWeight(w.to(gpu)))
+    assert ps.parts.shape == (ranges, m, n) and tuple(ps.shape) == (m, n)
+    total = ps.parts.double().sum(0).cpu()
+    assert (total - want).abs().max() <= 2e-5 * want.abs().max()
+    # as a delta of the norm kernel: the same as its sum (ranges added in order, in fp32) rounded to bf16
+    if n % 8 == 0:
+        seq = ps.parts[0].clone()
+        for r in range(1, ranges):
+            seq += ps.parts[r]
+        delta = seq.to(torch.bfloat16)
+        hidden = rnd(m, n, seed=8)
+        wn = (1 + 0.1 * rnd(n, seed=9).float()).to(torch.bfloat16).to(gpu)
+        h1, h2 = hidden.clone().to(gpu), hidden.clone().to(gpu)
+        o1, o2 = torch.empty_like(h1), torch.empty_like(h2)
+        K.rmsnorm(h1, wn, 1e-5, o1, delta=ps)
+        K.rmsnorm(h2, wn, 1e-5, o2, delta=delta)
+        assert torch.equal(h1, h2) and torch.equal(o1, o2)
+        rows = torch.tensor([m - 1, 0, 5, 5], dtype=torch.int32, device=gpu)
+        g1, g2 = torch.empty((4, n), dtype=torch.bfloat16, device=gpu), torch.empty((4, n), dtype=torch.bfloat16, device=gpu)
+        K.rmsnorm(h1, wn, 1e-5, g1, delta=ps, row_idx=rows)
+        K.rmsnorm(h2, wn, 1e-5, g2, delta=delta, row_idx=rows)
+        assert torch.equal(g1, g2) and torch.equal(h1, h2)
+        assert torch.equal(ps.materialize().float(), ps.parts.sum(0).to(torch.bfloat16).float())
+    assert K.gemm_skinny_partial_ranges(16, n, k) == 0 and K.gemm_skinny_partial_ranges(65, n, k) == 0
+    assert K.gemm_skinny_partial_ranges(m, n, 96) == 0
+    with pytest.raises(K.KernelError):
+        K.gemm_skinny_partials(x[:16].contiguous().to(gpu), K.TiledWeight(w.to(gpu)))
+
+
 @pytest.mark.parametrize("m", [1, 7, 16])
 @pytest.mark.parametrize("inter, hidden", [(8192, 2048), (256, 96), (96, 64)])
 def test_activations_pass_between_two_products_in_lane_order(m, inter, hidden, gpu):

@@ -193,6 +193,62 @@ def test_pre_norm_block_adds_both_branches_to_the_stream(dtype, gpu):
     assert err(hidden, want) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("T", [5, 20, 40, 64, 100])
+def test_two_blocks_hand_the_stream_on_at_every_row_count(T, gpu):
+    """bf16, widths that are multiples of 128.  At few rows every product that feeds the stream
+    prepares the next norm in its epilogue (NormedRows); from 17 to 64 rows the down projection
+    (and from 33 the output projection) leaves partial products over ranges of K that the next
+    norm's kernel adds up; above that the vendor library's product comes back as it is.  Two
+    blocks in a row, so that the second block's first norm is reached across the block boundary;
+    the last branch is added here, whatever form it has."""
+    from kv_cache_optimization_for_llm_amd.ops import kernels as K
+    from kv_cache_optimization_for_llm_amd.parts.base import NormedRows
+    H, nq, nkv, d, inter = 128, 4, 2, 32, 384
+    blocks, W = [], {}
+    for b in range(2):
+        mixer = GQAAttention(f"b{b}.m.", hidden_size=H, num_heads=nq, num_kv_heads=nkv, head_dim=d, scale=d ** -0.5,
+                             position=PartSpec("rotary", dict(head_dim=d, max_positions=128, theta=10000.0)))
+        ffn = SwiGLU(f"b{b}.f.", hidden_size=H, intermediate_size=inter)
+        norms = {"mixer": RMSNorm(f"b{b}.n1.", width=H, eps=1e-5), "feed_forward": RMSNorm(f"b{b}.n2.", width=H, eps=1e-5)}
+        block = PreNormBlock(mixer, ffn, norms)
+        for i, part in enumerate(block.parts()):
+            t = {k: (1 + 0.1 * rnd(*s.shape, seed=i + b)) if s.init == "norm" else rnd(*s.shape, scale=0.12, seed=i + b)
+                 for k, s in part.tensor_specs().items()}
+            W.update(load(part, t, "bfloat16", gpu))
+        blocks.append(block)
+    h0 = rnd(T, H).to(torch.bfloat16)
+    cfg = dict(num_attention_heads=nq, num_key_value_heads=nkv, head_dim=d, hidden_size=H, rope_theta=10000.0)
+    want = h0.float()
+    for b in range(2):
+        p = f"b{b}."
+        want = want + plain.attention_block(plain.rms_norm(want, W[p + "n1.weight"], 1e-5), W, p + "m.", cfg, list(range(T)))
+        want = want + plain.swiglu(plain.rms_norm(want, W[p + "n2.weight"], 1e-5), W[p + "f.gate_proj.weight"],
+                                   W[p + "f.up_proj.weight"], W[p + "f.down_proj.weight"])
+    cm, seat = one_request_context(nkv, d, 16, T, 0, "bfloat16", gpu, slots=(0, 1))
+    assert cm.grow(seat, T)
+    sm = cm.slot_mapping(seat, 0, T, 0)
+    cm.flush_tables()
+    batch = build_batch([seat], [0], [np.zeros(T, dtype=np.int32)], [[]], [[sm]], gpu)
+    g = cm.groups[0]
+    hidden, delta = h0.to(gpu).clone(), None
+    handed_on = []
+    for b, block in enumerate(blocks):
+        _, k, v = cm.kv_arrays(b)
+        ctx = MixerContext(batch=batch, kv=KVView(k, v, g.table_dev, batch.slot_mapping[0], g.page_size))
+        hidden, delta = block.forward(hidden, delta, ctx, blocks[1].first_norm() if b == 0 else None)
+        handed_on.append(delta)
+    first = handed_on[0]
+    if T <= 16:
+        assert isinstance(first, NormedRows)
+    elif T <= 64:
+        assert isinstance(first, (NormedRows, K.PartialSums)), type(first)
+    else:
+        assert isinstance(first, torch.Tensor)
+    assert not isinstance(delta, NormedRows), "without a next norm the last branch is not added by its product"
+    K.residual_add(hidden, delta.materialize() if isinstance(delta, K.PartialSums) else delta)
+    assert err(hidden, want) <= TOL["bfloat16"]
+
+
 def test_linear_chooses_its_kernel_by_rows_and_width(gpu):
     """One or two rows of a width that is a multiple of 512 take the matrix-vector kernel, up to
     16 rows (and other widths) the few-rows kernel, fp32 neither; every choice gives the product."""
