@@ -179,28 +179,7 @@ extern "C" int kva_embed_gather_prep(void *hidden, void *scaled, float *sumsq, c
 __device__ inline void load_delta8(const bf16_t *dl, const float *parts_row, int parts, size_t part_stride, int i,
                                    float (&d)[8]) {
     if (parts > 0) {
-        // four ranges at a time, all eight loads asked for before the first is added (a plain loop
-        // over the ranges is a trip to memory per range); added in the order of the ranges
-        float4 lo = make_float4(0.f, 0.f, 0.f, 0.f), hi = lo;
-        for (int s0 = 0; s0 < parts; s0 += 4) {
-            float4 a[4], b[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int s = s0 + j < parts ? s0 + j : parts - 1;
-                a[j] = *reinterpret_cast<const float4 *>(parts_row + (size_t)s * part_stride + i);
-                b[j] = *reinterpret_cast<const float4 *>(parts_row + (size_t)s * part_stride + i + 4);
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                if (s0 + j < parts) {
-                    lo.x += a[j].x; lo.y += a[j].y; lo.z += a[j].z; lo.w += a[j].w;
-                    hi.x += b[j].x; hi.y += b[j].y; hi.z += b[j].z; hi.w += b[j].w;
-                }
-            }
-        }
-        const float f[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-#pragma unroll
-        for (int j = 0; j < 8; ++j) d[j] = bf16_bits_to_float(float_to_bf16_bits(f[j]));
+        sum_ranges8(parts_row, parts, part_stride, i, d);
     } else {
         unpack8(*reinterpret_cast<const uint4 *>(dl + i), d);
     }

@@ -133,6 +133,34 @@ __device__ inline float row16_sum(float v) {
 // another order than wave_sum's.
 __device__ inline float wave_sum_valu(float v) { return quad_rows_sum(row16_sum(v)); }
 
+// 8 neighbouring elements of the sum of `parts` fp32 partial products laid out [parts][rows][width]
+// (row: the row's start in range 0, stride: rows * width), each rounded to bf16 as the whole product
+// would have been.  Four ranges at a time, all eight loads asked for before the first is added (a
+// plain loop over the ranges is a trip to memory per range); added in the order of the ranges.
+__device__ inline void sum_ranges8(const float *row, int parts, size_t stride, int i, float (&f)[8]) {
+    float4 lo = make_float4(0.f, 0.f, 0.f, 0.f), hi = lo;
+    for (int s0 = 0; s0 < parts; s0 += 4) {
+        float4 a[4], b[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int s = s0 + j < parts ? s0 + j : parts - 1;
+            a[j] = *reinterpret_cast<const float4 *>(row + (size_t)s * stride + i);
+            b[j] = *reinterpret_cast<const float4 *>(row + (size_t)s * stride + i + 4);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (s0 + j < parts) {
+                lo.x += a[j].x; lo.y += a[j].y; lo.z += a[j].z; lo.w += a[j].w;
+                hi.x += b[j].x; hi.y += b[j].y; hi.z += b[j].z; hi.w += b[j].w;
+            }
+        }
+    }
+    const float t[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f[j] = bf16_bits_to_float(float_to_bf16_bits(t[j]));
+}
+
+
 // Sum over a whole workgroup of `nwaves` wavefronts; `scratch` holds at least nwaves floats.
 // Every thread gets the result.  The order of the additions is fixed.
 __device__ inline float block_sum(float v, float *scratch, int nwaves) {
