@@ -97,7 +97,7 @@ class Linear:
         from ..ops.gemm_bf16 import use_partial_sums
         if tail is None or not getattr(tail.norm, "takes_partial_sums", False) or self.tiled is None \
                 or not isinstance(x, torch.Tensor) or x.dtype != torch.bfloat16 or tail.hidden.dtype != torch.bfloat16 \
-                or not use_partial_sums(x.shape[0], self.out_features, self.in_features):
+                or self.out_features % 8 or not use_partial_sums(x.shape[0], self.out_features, self.in_features):
             return None
         return K.gemm_skinny_partials(x, self.tiled)
 

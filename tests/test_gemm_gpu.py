@@ -261,7 +261,7 @@ def test_partial_products_over_ranges_of_k_add_up_to_the_product(m, n, k, gpu):
         K.rmsnorm(h1, wn, 1e-5, g1, delta=ps, row_idx=rows)
         K.rmsnorm(h2, wn, 1e-5, g2, delta=delta, row_idx=rows)
         assert torch.equal(g1, g2) and torch.equal(h1, h2)
-        assert torch.equal(ps.materialize().float(), ps.parts.sum(0).to(torch.bfloat16).float())
+        assert torch.equal(ps.materialize(), delta)
     assert K.gemm_skinny_partial_ranges(16, n, k) == 0 and K.gemm_skinny_partial_ranges(65, n, k) == 0
     assert K.gemm_skinny_partial_ranges(m, n, 96) == 0
     with pytest.raises(K.KernelError):
