@@ -80,7 +80,10 @@ class StepBatch:
                                                    self.h_entry_seat, group, row_tiles, which)
             n = ent.shape[0]
             parts = [ent, row0] + ([meta.reshape(-1)] if meta is not None else [])
-            dev = torch.from_numpy(np.concatenate(parts)).to(self.token_ids.device, non_blocking=True)
+            flat = np.concatenate(parts)
+            staging = torch.empty(flat.shape[0], dtype=torch.int32, pin_memory=True)      # (a pageable source makes the copy wait)
+            staging.numpy()[:] = flat
+            dev = staging.to(self.token_ids.device, non_blocking=True)
             self._items[key] = (dev[:n], dev[n:2 * n], dev[2 * n:].view(n, 8) if meta is not None else None)
         return self._items[key]
 

@@ -127,8 +127,10 @@ class DecodeGraphs:
             # No garbage collection while the stream captures: an unreachable engine of earlier
             # (its pinned tables, events, graphs) freed in the middle of a capture makes calls that
             # a capturing stream forbids, and the failure is raised inside a destructor, where it
-            # ends the process.  Collect first, then keep the collector off until the capture ends.
-            gc.collect()
+            # ends the process.  The collector stays off until the capture ends; what is garbage
+            # now is collected at some later allocation, outside a capture.  (A full collection
+            # here, before every capture, was 28 ms each: a third of a serving loop's host time
+            # while new step shapes kept coming.)
             gc_was_on = gc.isenabled()
             gc.disable()
             try:
@@ -277,8 +279,7 @@ class PortionGraphs:
         if slot.graph is None:
             torch.cuda.synchronize()
             g = torch.cuda.CUDAGraph()
-            gc.collect()                  # as for decode graphs: nothing is freed while the stream captures
-            gc_was_on = gc.isenabled()
+            gc_was_on = gc.isenabled()        # as for decode graphs: nothing is collected while the stream captures
             gc.disable()
             try:
                 with torch.cuda.graph(g):

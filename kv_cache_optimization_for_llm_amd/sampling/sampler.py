@@ -84,6 +84,28 @@ class Sampler:
         self._landing: List[torch.Tensor] = []
         self._kernel_writes_host = False
         self._landing_next = 0
+        # per-row arguments of a sampling (temperatures, random-stream keys and steps, seats)
+        self._args_dev: Optional[torch.Tensor] = None
+        self._args_host: List[tuple] = []
+        self._args_next = 0
+
+    def _row_arguments(self, n: int):
+        """A pinned staging array [5, capacity] int32 to fill (float rows as their bits) and the
+        device array it is copied to by :meth:`_send_row_arguments`."""
+        if self._args_dev is None or self._args_dev.shape[1] < n:
+            cap = max(64, n)
+            self._args_dev = torch.zeros((5, cap), dtype=torch.int32, device=self.device)
+            self._args_host = [(torch.zeros((5, cap), dtype=torch.int32, pin_memory=True), torch.cuda.Event())
+                               for _ in range(3)]
+        self._args_next = (self._args_next + 1) % len(self._args_host)
+        staging, copied = self._args_host[self._args_next]
+        copied.synchronize()             # its last copy has left it (three steps ago)
+        return staging.numpy(), self._args_dev
+
+    def _send_row_arguments(self) -> None:
+        staging, copied = self._args_host[self._args_next]
+        self._args_dev.copy_(staging, non_blocking=True)
+        copied.record()
 
     def reset_seat(self, seat: int, emitted: Sequence[int] = ()) -> None:
         """A request takes the seat: clear its mask and mark what it has emitted before (a
@@ -130,20 +152,26 @@ class Sampler:
             event.record()
             return PendingTokens(host, event, 0)
         any_sampled = any(r.temperature > 0 for r in rows)
-        inv_t = key = step = seat_t = None
-        if any_sampled:
-            inv_t = torch.tensor([1.0 / r.temperature if r.temperature > 0 else 0.0 for r in rows],
-                                 dtype=torch.float32).to(self.device)
-            key = torch.from_numpy(_as_i32([r.rng_key for r in rows])).to(self.device)
-            step = torch.from_numpy(_as_i32([r.rng_step for r in rows])).to(self.device)
         use_mask = self.mask is not None and any(r.apply_penalty for r in rows)
-        if use_mask:
-            seat_t = torch.tensor([r.seat if r.apply_penalty else -1 for r in rows],
-                                  dtype=torch.int32).to(self.device)
-        # every token a request emits is marked in its mask row, by the launch that chooses it
-        mark_seat = None
-        if self.mask is not None:
-            mark_seat = torch.from_numpy(np.asarray([r.seat for r in rows], dtype=np.int32)).to(self.device)
+        inv_t = key = step = seat_t = mark_seat = None
+        if any_sampled or self.mask is not None:
+            # the per-row arguments go up in one copy from pinned memory (five small pageable
+            # tensors, each copied by itself, were 0.4 ms of host time apiece in a serving loop)
+            host_args, dev_args = self._row_arguments(n)
+            if any_sampled:
+                host_args[0, :n] = np.asarray([1.0 / r.temperature if r.temperature > 0 else 0.0 for r in rows],
+                                              dtype=np.float32).view(np.int32)
+                host_args[1, :n] = _as_i32([r.rng_key for r in rows])
+                host_args[2, :n] = _as_i32([r.rng_step for r in rows])
+                inv_t, key, step = dev_args[0, :n].view(torch.float32), dev_args[1, :n], dev_args[2, :n]
+            if use_mask:
+                host_args[3, :n] = [r.seat if r.apply_penalty else -1 for r in rows]
+                seat_t = dev_args[3, :n]
+            if self.mask is not None:
+                # every token a request emits is marked in its mask row, by the launch that chooses it
+                host_args[4, :n] = [r.seat for r in rows]
+                mark_seat = dev_args[4, :n]
+            self._send_row_arguments()
         K.sample(logits, out, chunks=self.chunks, inv_temperature=inv_t, seed=self.seed, rng_key=key,
                  rng_step=step, penalty_mask=self.mask if use_mask else None, row_seat=seat_t,
                  penalty=self.penalty, mark_mask=self.mask if mark_seat is not None else None,

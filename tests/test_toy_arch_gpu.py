@@ -495,8 +495,8 @@ def test_garbage_of_an_earlier_engine_is_not_collected_inside_a_graph_capture(tm
     """An engine that has become unreachable (pinned block tables, events, captured graphs) is
     freed by Python's collector at some later allocation - also one made while the next engine
     captures a decode graph, where freeing such things is forbidden and fails inside a destructor.
-    The capture collects first and keeps the collector off: with a collector set to run at every
-    few allocations, a second engine captures and replays its graphs next to the garbage of a first."""
+    The capture keeps the collector off: with a collector set to run at every few allocations, a
+    second engine captures and replays its graphs next to the garbage of a first."""
     import gc
     from conftest import TINY
     cfg = TINY["A"][0]
