@@ -223,18 +223,25 @@ class PortionGraphs:
     A shape is (tokens per entry, wanted places, context bucket, whether the portions' rows visit
     enough keys for the workgroup attention kernel): everything the forward pass decides on the
     host.  Its first step runs eagerly and tells which sets of attention work items the pass asks
-    for; its second step is captured over static buffers; later ones upload their indices and
-    replay.  Logits come back in the shape's static buffer: they hold until its next step."""
+    for; the step at which it has come ``CAPTURE_AT`` times is captured over static buffers; later
+    ones upload their indices and replay.  Logits come back in the shape's static buffer: they hold
+    until its next step."""
 
     MAX_TOKENS = 4096          # tokens of one captured step
     MAX_LOGIT_ROWS = 64        # a graph keeps its logits: [rows, vocabulary] fp32
     MAX_SHAPES = 32            # captured shapes kept (least recently used goes first) ...
     MAX_KEPT_TOKENS = 16384    # ... and the tokens of all of them: a graph keeps its step's activations
     MAX_SEEN = 4096
+    # A capture costs some 6 ms of host time and a place among the shapes kept.  Under a load of random
+    # prompt lengths most shapes come twice at most: captured at their second step, 500 captures in
+    # 17 s pushed each other out of the 32 places before any was replayed much.  The shapes that
+    # carry such a load (so many decoded tokens beside a full portion) come again and again.
+    CAPTURE_AT = 3
 
     def __init__(self, model, cache, device, feedback=None):
         self.model, self.cache, self.device, self.feedback = model, cache, device, feedback
         self.seen: Dict[tuple, tuple] = {}
+        self.times: Dict[tuple, int] = {}            # steps a seen shape has come (while it has no graph)
         self.slots: "OrderedDict[tuple, _PortionSlot]" = OrderedDict()
         self.replays = 0
         self.captures = 0
@@ -256,7 +263,9 @@ class PortionGraphs:
         if key not in self.seen:
             if len(self.seen) >= self.MAX_SEEN:
                 self.seen.clear()
+                self.times.clear()
             self.seen[key] = tuple(batch._items.keys())
+            self.times[key] = 1
 
     def run(self, key: tuple, tokens: np.ndarray, seats: np.ndarray, starts: np.ndarray,
             slot_maps: Sequence[np.ndarray]) -> Optional[torch.Tensor]:
@@ -267,6 +276,9 @@ class PortionGraphs:
             return None
         slot = self.slots.get(key)
         if slot is None:
+            self.times[key] = self.times.get(key, 1) + 1
+            if self.times[key] < self.CAPTURE_AT:
+                return None
             lens, rows, bucket, _ = key
             while self.slots and (len(self.slots) >= self.MAX_SHAPES or
                                   sum(s.T for s in self.slots.values()) + sum(lens) > self.MAX_KEPT_TOKENS):
