@@ -57,6 +57,8 @@ class StepBatch:
     meta_provider: object = None         # callable(group, row_tiles) -> attention items, or None
     static_items: bool = False           # a captured step: every set of attention items is prepared ahead
     _items: Dict[tuple, tuple] = field(default_factory=dict, repr=False)
+    # the attention launches decided for this step, per geometry (ops.attention.paged_attention)
+    attention_plans: Dict[tuple, list] = field(default_factory=dict, repr=False)
 
     def attention_items(self, group: int, row_tiles: int = 1, which: str = "all"):
         """Work items of the matrix-core attention kernels for a query-head group size: (entry,

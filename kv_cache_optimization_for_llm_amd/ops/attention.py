@@ -91,7 +91,9 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
     one-wavefront kernel with their keys split over wavefronts; prompt portions take the
     workgroup kernel that shares key blocks through LDS when there is enough of them to fill the
     chip, else the one-wavefront kernel with two row tiles.  A step that holds both is two
-    launches, each over its own entries."""
+    launches, each over its own entries.  Which kernels, over which work items and key splits, is
+    decided once per step and geometry (every layer of a model asks the same) and kept with the
+    batch."""
     if kv is None:
         raise K.KernelError("paged_attention: the mixer has no cache view")
     if not (qkv.dtype == torch.bfloat16 and K.attention_mfma_supported(head_dim, kv.page_size)
@@ -99,15 +101,31 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
         return K.attention_rowwise(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table,
                                    batch.tok_seat, batch.positions, num_q_heads, num_kv_heads,
                                    head_dim, scale, window)
-    group = num_q_heads // num_kv_heads
+    plans = batch.attention_plans
+    key = (num_q_heads, num_kv_heads, head_dim, kv.page_size)
+    plan = plans.get(key)
+    if plan is None:
+        plan = plans[key] = _plan(batch, num_q_heads // num_kv_heads, num_kv_heads, head_dim, kv.page_size)
     stride = qkv.shape[1]
+    for launch in plan:
+        if launch[0] == "wave":
+            _, (item_entry, item_row0, meta), tiles, splits, per, pair, covers_all, keep_cached = launch
+            K.attention_mfma(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table, item_entry, item_row0,
+                             batch.entry_seat, batch.entry_q_start, batch.entry_start_pos, num_q_heads,
+                             num_kv_heads, head_dim, scale, window, splits, per, tiles, pair, meta,
+                             covers_all_rows=covers_all, keep_cached=keep_cached)
+        else:
+            _, meta, splits, per, covers_all = launch
+            K.attention_lds(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table, meta, num_q_heads,
+                            num_kv_heads, head_dim, scale, window, False, splits, per, covers_all_rows=covers_all)
+    return out
 
-    def wave_kernel(items, tiles, splits, per, pair, which, keep_cached=False):
-        item_entry, item_row0, meta = items
-        K.attention_mfma(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table, item_entry, item_row0,
-                         batch.entry_seat, batch.entry_q_start, batch.entry_start_pos, num_q_heads,
-                         num_kv_heads, head_dim, scale, window, splits, per, tiles, pair, meta,
-                         covers_all_rows=which == "all", keep_cached=keep_cached)
+
+def _plan(batch, group: int, num_kv_heads: int, head_dim: int, page_size: int) -> list:
+    """The launches of one attention call over ``batch``: ("wave", items, row tiles, splits, keys per
+    split, pair, covers all rows, keep cached) and ("lds", item records, splits, keys per split,
+    covers all rows)."""
+    plan = []
 
     def decoded(which):
         items = batch.attention_items(group, 1, which)
@@ -118,23 +136,21 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
         # of 768 keys, 12.6 MB a layer: 0.913 -> 0.902 ms; 8 of 8,192, 134 MB a layer: 1.27 -> 1.30,
         # so only the small ones)
         small = n * batch.max_context * num_kv_heads * head_dim * 4 <= _KEEP_CACHED_BYTES
-        wave_kernel(items, 1, splits, per, False, which, keep_cached=small)
+        plan.append(("wave", items, 1, splits, per, False, which == "all", small))
 
     if batch.max_q_len * group <= 16:
         decoded("all")
-        return out
+        return plan
     mixed = batch.min_q_len * group <= 16
     which = "long" if mixed else "all"
     done = False
-    if K.attention_lds_supported(head_dim, kv.page_size):
+    if K.attention_lds_supported(head_dim, page_size):
         items = batch.attention_items(group, 8, which)
         groups = items[0].shape[0] * num_kv_heads
         if items[2] is not None and groups >= _LDS_MIN_GROUPS and (
                 groups >= _LDS_MANY_GROUPS or batch.mean_keys_of_long_entries() >= _LDS_MIN_MEAN_KEYS):
             splits, per = choose_lds_splits(groups, batch.max_context)
-            K.attention_lds(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table, items[2], num_q_heads,
-                            num_kv_heads, head_dim, scale, window, False, splits, per,
-                            covers_all_rows=which == "all")
+            plan.append(("lds", items[2], splits, per, which == "all"))
             done = True
     if not done:
         # two row tiles per wave, so each key and value loaded serves 32 query rows; whole key
@@ -145,12 +161,12 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
         if waves >= _WIDE_MIN_WAVES:
             # items come ordered by work: a wavefront that takes the i-th and the i-th last does
             # about the average; worth it while every SIMD still gets a wavefront
-            wave_kernel(items, tiles, 1, 0, waves >= _PAIR_MIN_WAVES, which)
+            plan.append(("wave", items, tiles, 1, 0, waves >= _PAIR_MIN_WAVES, which == "all", False))
         else:
             # too few items to fill the chip: the keys are split over wavefronts as well (portions
             # of 256 tokens late in an 8,192-token prompt: 16 % faster than one row tile per wave)
             splits, per = choose_splits(items[0].shape[0], num_kv_heads, batch.max_context)
-            wave_kernel(items, tiles, splits, per, False, which)
+            plan.append(("wave", items, tiles, splits, per, False, which == "all", False))
     if mixed:
         decoded("short")
-    return out
+    return plan
