@@ -128,7 +128,10 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, float *__restrict__ part
     // chunk c of the V^T tile is 8 keys of value dimension (c % 2D) / 2 in page c / 2D.  A tile
     // outside the keys the workgroup needs is redirected to the nearest needed one (its page is
     // certainly mapped); its scores are masked away.
-    uint4 stage_k[Geo::SB][Geo::PER_THREAD], stage_v[Geo::SB][Geo::PER_THREAD];
+    // (named registers, not arrays: as arrays the compiler kept them in scratch memory for head sizes
+    // with two chunks per thread, a store and a load of 64 bytes per thread and block)
+    static_assert(Geo::SB == 1 && Geo::PER_THREAD <= 2, "the staging registers below are two chunks of one block");
+    uint4 stage_k0, stage_k1, stage_v0, stage_v1;
     // which of the block's two pages a thread's chunk lies in is the same for a whole wavefront
     // (said explicitly, so that the page's address stays scalar arithmetic); its place inside the
     // page never changes
@@ -151,28 +154,30 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, float *__restrict__ part
             tile0 = tile0 < lo_tile ? lo_tile : (tile0 > hi_tile ? hi_tile : tile0);
             pg[t] = bt[__builtin_amdgcn_readfirstlane(tile0 >> 4)];
         }
-#pragma unroll
-        for (int i = 0; i < Geo::PER_THREAD; ++i) {
+        auto chunk = [&](int i, uint4 &k, uint4 &v) {
             const int c = tid + i * 256;
             if (Geo::CHUNKS % 256 == 0 || c < Geo::CHUNKS) {
                 const size_t kpage = ((size_t)(k_sel[i] ? pg[1] : pg[0]) * num_kv_heads + kvh) * (size_t)(16 * D);
-                stage_k[b][i] = *reinterpret_cast<const uint4 *>(k_cache + kpage + k_off[i]);
+                k = *reinterpret_cast<const uint4 *>(k_cache + kpage + k_off[i]);
                 const size_t vpage = ((size_t)(v_sel[i] ? pg[1] : pg[0]) * num_kv_heads + kvh) * (size_t)(16 * D);
-                stage_v[b][i] = *reinterpret_cast<const uint4 *>(v_cache + vpage + v_off[i]);
+                v = *reinterpret_cast<const uint4 *>(v_cache + vpage + v_off[i]);
             }
-        }
+        };
+        chunk(0, stage_k0, stage_v0);
+        if (Geo::PER_THREAD > 1) chunk(1, stage_k1, stage_v1);
     };
     auto stash = [&](int b, char *buf) {
-#pragma unroll
-        for (int i = 0; i < Geo::PER_THREAD; ++i) {
+        auto chunk = [&](int i, const uint4 &k, const uint4 &v) {
             const int c = tid + i * 256;
             if (Geo::CHUNKS % 256 == 0 || c < Geo::CHUNKS) {
                 const int key = c / (D / 8), kc = c % (D / 8);
-                *reinterpret_cast<uint4 *>(buf + key * Geo::KROW + kc * 16) = stage_k[b][i];
+                *reinterpret_cast<uint4 *>(buf + key * Geo::KROW + kc * 16) = k;
                 const int t = c / (2 * D), rem = c % (2 * D);
-                *reinterpret_cast<uint4 *>(buf + Geo::KBYTES + (rem >> 1) * Geo::VROW + (t * 16 + (rem & 1) * 8) * 2) = stage_v[b][i];
+                *reinterpret_cast<uint4 *>(buf + Geo::KBYTES + (rem >> 1) * Geo::VROW + (t * 16 + (rem & 1) * 8) * 2) = v;
             }
-        }
+        };
+        chunk(0, stage_k0, stage_v0);
+        if (Geo::PER_THREAD > 1) chunk(1, stage_k1, stage_v1);
     };
 
     const float scale2 = scale * 1.44269504088896340736f;   // exp(x * scale) = exp2(x * scale * log2 e)
@@ -370,6 +375,14 @@ attention_lds_kernel_3(LDS_KERNEL_PARAMS) {
     attention_lds_body<D>(LDS_KERNEL_ARGS);
 }
 
+// Head sizes 96 and 128: left alone the compiler takes over 300 registers, which leaves one wavefront
+// per SIMD and nothing to overlap matrix-core, vector and LDS work with.
+template <int D>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+attention_lds_kernel_2(LDS_KERNEL_PARAMS) {
+    attention_lds_body<D>(LDS_KERNEL_ARGS);
+}
+
 extern "C" int kva_attention_lds_supported(int head_dim, int page_size) {
     return (page_size == 16 && (head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128)) ? 1 : 0;
 }
@@ -410,8 +423,8 @@ extern "C" int kva_attention_lds(void *out, float *part_o, float *part_ml, const
     switch (head_dim) {
     case 32: LAUNCH(attention_lds_kernel_3, 32); break;
     case 64: LAUNCH(attention_lds_kernel_3, 64); break;
-    case 96: LAUNCH(attention_lds_kernel, 96); break;
-    default: LAUNCH(attention_lds_kernel, 128); break;
+    case 96: LAUNCH(attention_lds_kernel_2, 96); break;
+    default: LAUNCH(attention_lds_kernel_2, 128); break;
     }
 #undef LAUNCH
     KVA_CHECK_LAUNCH("attention_lds");

@@ -248,7 +248,7 @@ class PortionGraphs:
 
     @staticmethod
     def shape_key(lens: Sequence[int], starts: Sequence[int], rows: Sequence[int]) -> Optional[tuple]:
-        from ..ops.attention import _LDS_MIN_MEAN_KEYS
+        from ..ops.attention import LDS_MEAN_KEYS_STEPS
         T = int(sum(lens))
         if T > PortionGraphs.MAX_TOKENS or len(rows) > PortionGraphs.MAX_LOGIT_ROWS:
             return None
@@ -256,7 +256,8 @@ class PortionGraphs:
         long = ln > 1
         mean_keys = float(((st[long] + (ln[long] + 1) / 2) * ln[long]).sum() / ln[long].sum())
         bucket = context_bucket(int(max(s + n for s, n in zip(starts, lens))))
-        return (tuple(int(n) for n in lens), tuple(int(r) for r in rows), bucket, mean_keys >= _LDS_MIN_MEAN_KEYS)
+        return (tuple(int(n) for n in lens), tuple(int(r) for r in rows), bucket,
+                tuple(mean_keys >= t for t in LDS_MEAN_KEYS_STEPS))
 
     def note(self, key: tuple, batch: StepBatch) -> None:
         """After the eager run of a shape: the sets of attention items its forward pass used."""

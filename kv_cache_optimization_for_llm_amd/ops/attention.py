@@ -39,6 +39,16 @@ _PAIR_MIN_WAVES = 2048      # two items per wavefront once that still leaves a w
 _LDS_MIN_GROUPS = 128
 _LDS_MANY_GROUPS = 768
 _LDS_MIN_MEAN_KEYS = 2048
+# Head sizes above 96 do twice the matrix-core work per key and row for the same vector work, and
+# one wavefront with two row tiles of them fills its SIMD's registers alone: there the workgroup kernel
+# (two workgroups per compute unit) is ahead from 1,024 keys a row on (head size 128, a 2,048-token
+# prompt from position 0: 93 us against 107; 4,096 tokens: 235 against 375; 1,024: 45 against 41).
+_LDS_MIN_MEAN_KEYS_WIDE_HEADS = 1024
+LDS_MEAN_KEYS_STEPS = (_LDS_MIN_MEAN_KEYS_WIDE_HEADS, _LDS_MIN_MEAN_KEYS)     # where the choice can change
+
+
+def lds_min_mean_keys(head_dim: int) -> int:
+    return _LDS_MIN_MEAN_KEYS_WIDE_HEADS if head_dim > 96 else _LDS_MIN_MEAN_KEYS
 # few workgroups that each walk thousands of keys: the keys are cut into ranges, one workgroup each
 _LDS_TARGET_GROUPS = 1024
 _LDS_MIN_KEYS_PER_SPLIT = 1024
@@ -148,7 +158,7 @@ def _plan(batch, group: int, num_kv_heads: int, head_dim: int, page_size: int) -
         items = batch.attention_items(group, 8, which)
         groups = items[0].shape[0] * num_kv_heads
         if items[2] is not None and groups >= _LDS_MIN_GROUPS and (
-                groups >= _LDS_MANY_GROUPS or batch.mean_keys_of_long_entries() >= _LDS_MIN_MEAN_KEYS):
+                groups >= _LDS_MANY_GROUPS or batch.mean_keys_of_long_entries() >= lds_min_mean_keys(head_dim)):
             splits, per = choose_lds_splits(groups, batch.max_context)
             plan.append(("lds", items[2], splits, per, which == "all"))
             done = True
