@@ -228,7 +228,7 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, float *__restrict__ part
                     sv[rt][t * 4 + i] = x;
                     mx = fmaxf(mx, x);
                 }
-            mloc[rt] = quad_rows_max(mx);
+            mloc[rt] = mx;            // this lane's part of the row: the whole row's only when the reference moves
         }
         // the reference of the exponentials follows the running maximum lazily (see attention_mfma.hip)
         bool rebase = false;
@@ -237,7 +237,7 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, float *__restrict__ part
         if (__builtin_amdgcn_ballot_w64(rebase) != 0) {
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
-                const float m_new = fmaxf(m[rt], mloc[rt]);
+                const float m_new = fmaxf(m[rt], quad_rows_max(mloc[rt]));
                 const float c = __builtin_amdgcn_exp2f((m[rt] - ((m_new == -INFINITY) ? 0.f : m_new)) * scale2);
                 ol[rt][0] *= c; ol[rt][1] *= c; ol[rt][2] *= c; ol[rt][3] *= c;
 #pragma unroll
@@ -257,6 +257,13 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, float *__restrict__ part
                 pf[rt].p2[j / 2] = pack_bf16(p0, p1);
             }
         }
+        // Head sizes above 64: the wavefront whose products are ready goes first (head size 128,
+        // 8,192-token prompt: 807 -> 772 us; head size 64 loses 1 % by it).  A SIMD issues either a
+        // matrix-core product or a vector instruction, from whichever wavefront: timed alone, 8 products
+        // and 24 multiply-adds in one wavefront take 126 ns, the products without the multiply-adds 67 and
+        // the multiply-adds without the products 56, and given to two wavefronts of one SIMD 109; so a key
+        // block costs its products plus its softmax, however the two are interleaved.
+        if (D > 64) __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
@@ -264,6 +271,7 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, float *__restrict__ part
                 o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf[rt].v, o[rt][dt], 0, 0, 0);
             ol[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pf[rt].v, ol[rt], 0, 0, 0);
         }
+        if (D > 64) __builtin_amdgcn_s_setprio(0);
     };
 
     // ---- the key loop: a stage is SB blocks of 32 keys; one barrier per stage, two LDS buffers.

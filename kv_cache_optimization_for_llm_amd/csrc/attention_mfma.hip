@@ -265,7 +265,7 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
                     sv[rt][t * 4 + i] = x;
                     mx = fmaxf(mx, x);
                 }
-            mloc[rt] = quad_rows_max(mx);
+            mloc[rt] = mx;            // this lane's part of the row: the whole row's only when the reference moves
         }
         // m[rt] is the reference the row's exponentials are taken against.  It follows the
         // running maximum lazily: only when a row's maximum has outgrown it by more than
@@ -281,7 +281,7 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
         if (__builtin_amdgcn_ballot_w64(rebase) != 0) {
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
-                const float m_new = fmaxf(m[rt], mloc[rt]);
+                const float m_new = fmaxf(m[rt], quad_rows_max(mloc[rt]));
                 // a row that has seen no key yet keeps m = -inf (exp2(-inf) = 0 clears nothing that counts)
                 const float c = __builtin_amdgcn_exp2f((m[rt] - ((m_new == -INFINITY) ? 0.f : m_new)) * scale2);
                 l[rt] *= c;
