@@ -69,8 +69,8 @@ def attention(args) -> None:
     nq, nkv, d, page = args.heads, args.kv_heads, args.head_dim, 16
     group = nq // nkv
     scale = d ** -0.5
-    if args.tokens:                                # one prompt of `tokens` tokens from position 0
-        entries = [(0, args.tokens)]
+    if args.tokens:                                # a prompt portion of `tokens` tokens from position `start`
+        entries = [(args.start, args.tokens)]
     else:                                          # `batch` decoded tokens at the end of `context`
         entries = [(args.context - 1, 1)] * args.batch
     ctx = max(s + n for s, n in entries)
@@ -98,12 +98,12 @@ def attention(args) -> None:
     qs = torch.from_numpy(q_start).to(dev)
     sp = torch.tensor([s for s, _ in entries], dtype=torch.int32, device=dev)
     splits, per = 1, 0
-    if not args.tokens:
-        splits = args.splits
+    if not args.tokens or args.portion_splits > 1:
+        splits = args.portion_splits if args.tokens else args.splits
         per = ((ctx + splits - 1) // splits + 31) // 32 * 32
     if args.kernel == "lds":
-        calls = [lambda c=c: K.attention_lds(qkv, nq * d, out, c[0], c[1], table, meta_d, nq, nkv, d, scale, 0, args.pair)
-                 for c in caches]
+        calls = [lambda c=c: K.attention_lds(qkv, nq * d, out, c[0], c[1], table, meta_d, nq, nkv, d, scale, 0, args.pair,
+                                             splits, per) for c in caches]
     else:
         pair = bool(args.tokens) and len(meta) * nkv >= 2048 and not args.no_pair
         calls = [lambda c=c: K.attention_mfma(qkv, nq * d, out, c[0], c[1], table, ent, row0, seat, qs, sp, nq, nkv,
@@ -111,7 +111,8 @@ def attention(args) -> None:
     us = _time_in_graph(calls, args.reps) if args.graph else _time(calls, args.reps)
     flops = sum(4.0 * nq * d * n * (2 * s + n + 1) / 2 for s, n in entries)
     kv_bytes = sum((s + n) * nkv * d * 4 for s, n in entries)
-    what = f"prompt of {args.tokens}" if args.tokens else f"batch {args.batch} at context {args.context}, {splits} splits"
+    what = (f"prompt of {args.tokens}" + (f" from position {args.start}" if args.start else "") +
+            (f", {splits} key ranges" if splits > 1 else "")) if args.tokens else f"batch {args.batch} at context {args.context}, {splits} splits"
     print(f"attention {args.kernel:4s} {what}: {us:9.1f} us  {flops / us / 1e6:8.1f} TFLOP/s  "
           f"{kv_bytes / us / 1e6:7.2f} TB/s of keys and values", flush=True)
 
@@ -227,6 +228,8 @@ def main(argv=None) -> int:
     a.add_argument("--kernel", choices=["wave", "lds"], default="wave",
                    help="one wavefront per work item, or a workgroup sharing key blocks through LDS")
     a.add_argument("--tokens", type=int, default=0, help="a prompt of this many tokens (else decoded tokens)")
+    a.add_argument("--start", type=int, default=0, help="with --tokens: the portion's first position (keys before it are in the cache)")
+    a.add_argument("--portion-splits", type=int, default=1, help="with --tokens: cut the keys into this many ranges")
     a.add_argument("--batch", type=int, default=8)
     a.add_argument("--context", type=int, default=8192)
     a.add_argument("--splits", type=int, default=32)

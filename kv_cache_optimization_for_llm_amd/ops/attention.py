@@ -42,16 +42,31 @@ _LDS_MIN_MEAN_KEYS = 2048
 # Head sizes above 96 do twice the matrix-core work per key and row for the same vector work, and
 # one wavefront with two row tiles of them fills its SIMD's registers alone: there the workgroup kernel
 # (two workgroups per compute unit) is ahead from 1,024 keys a row on (head size 128, a 2,048-token
-# prompt from position 0: 93 us against 107; 4,096 tokens: 235 against 375; 1,024: 45 against 41).
+# prompt from position 0: 93 us against 107; 4,096 tokens: 235 against 375; 1,024: 45 against 41), and
+# with the keys cut into shorter ranges also for short portions deep in a context (256 tokens at
+# position 4,096: 48 us in 8 ranges against 71 for the one-wavefront kernel at its best split; 128 at
+# 8,192: 47 against 64; 64 at 8,192: 35 against 41; 256 at 2,048: 38 against 50; 128 at 2,048 and
+# 256 at 1,024 are ties or losses, hence the 2,048 keys a row for fewer than 128 workgroups).
 _LDS_MIN_MEAN_KEYS_WIDE_HEADS = 1024
+_LDS_MIN_GROUPS_WIDE_HEADS = 16
+_LDS_TARGET_GROUPS_WIDE_HEADS = 512
+_LDS_MIN_KEYS_PER_SPLIT_WIDE_HEADS = 256
 LDS_MEAN_KEYS_STEPS = (_LDS_MIN_MEAN_KEYS_WIDE_HEADS, _LDS_MIN_MEAN_KEYS)     # where the choice can change
-
-
-def lds_min_mean_keys(head_dim: int) -> int:
-    return _LDS_MIN_MEAN_KEYS_WIDE_HEADS if head_dim > 96 else _LDS_MIN_MEAN_KEYS
 # few workgroups that each walk thousands of keys: the keys are cut into ranges, one workgroup each
 _LDS_TARGET_GROUPS = 1024
 _LDS_MIN_KEYS_PER_SPLIT = 1024
+
+
+def use_lds_kernel(groups: int, mean_keys: float, head_dim: int) -> bool:
+    """Whether prompt rows that make ``groups`` workgroups of 128 rows (over all kv heads) and visit
+    ``mean_keys`` keys each on average go to the workgroup kernel."""
+    if groups >= _LDS_MANY_GROUPS:
+        return True
+    if head_dim > 96:
+        if groups >= _LDS_MIN_GROUPS:
+            return mean_keys >= _LDS_MIN_MEAN_KEYS_WIDE_HEADS
+        return groups >= _LDS_MIN_GROUPS_WIDE_HEADS and mean_keys >= _LDS_MIN_MEAN_KEYS
+    return groups >= _LDS_MIN_GROUPS and mean_keys >= _LDS_MIN_MEAN_KEYS
 
 
 def _cut_keys(want: int, max_context: int, max_splits: int) -> tuple:
@@ -83,12 +98,14 @@ def choose_splits(num_items: int, num_kv_heads: int, max_context: int, max_split
     return _cut_keys(min(want, most), max_context, max_splits)
 
 
-def choose_lds_splits(groups: int, max_context: int, max_splits: int = None) -> tuple:
+def choose_lds_splits(groups: int, max_context: int, max_splits: int = None, head_dim: int = 64) -> tuple:
     """(splits, keys_per_split) for the workgroup kernel, under the same limit."""
     if max_splits is None:
         max_splits = K.attention_max_splits()
-    want = max(1, _LDS_TARGET_GROUPS // max(1, groups))
-    return _cut_keys(min(want, max(1, max_context // _LDS_MIN_KEYS_PER_SPLIT)), max_context, max_splits)
+    wide = head_dim > 96
+    want = max(1, (_LDS_TARGET_GROUPS_WIDE_HEADS if wide else _LDS_TARGET_GROUPS) // max(1, groups))
+    min_keys = _LDS_MIN_KEYS_PER_SPLIT_WIDE_HEADS if wide else _LDS_MIN_KEYS_PER_SPLIT
+    return _cut_keys(min(want, max(1, max_context // min_keys)), max_context, max_splits)
 
 
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads: int,
@@ -157,9 +174,8 @@ def _plan(batch, group: int, num_kv_heads: int, head_dim: int, page_size: int) -
     if K.attention_lds_supported(head_dim, page_size):
         items = batch.attention_items(group, 8, which)
         groups = items[0].shape[0] * num_kv_heads
-        if items[2] is not None and groups >= _LDS_MIN_GROUPS and (
-                groups >= _LDS_MANY_GROUPS or batch.mean_keys_of_long_entries() >= lds_min_mean_keys(head_dim)):
-            splits, per = choose_lds_splits(groups, batch.max_context)
+        if items[2] is not None and use_lds_kernel(groups, batch.mean_keys_of_long_entries(), head_dim):
+            splits, per = choose_lds_splits(groups, batch.max_context, head_dim=head_dim)
             plan.append(("lds", items[2], splits, per, which == "all"))
             done = True
     if not done:

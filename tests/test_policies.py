@@ -3,7 +3,7 @@ cache pool is made from leftover device memory."""
 import pytest
 
 from kv_cache_optimization_for_llm_amd.engine.engine import EngineError, pool_pages_from_memory
-from kv_cache_optimization_for_llm_amd.ops.attention import choose_lds_splits, choose_splits
+from kv_cache_optimization_for_llm_amd.ops.attention import choose_lds_splits, choose_splits, use_lds_kernel
 
 KERNEL_MAX_SPLITS = 256         # what the kernels and their merge take (kva_attention_max_splits)
 
@@ -16,7 +16,8 @@ def test_key_splits_never_exceed_what_the_kernels_take(nkv, items, context):
     policy must stop at the kernels' limit, and its ranges must still cover every key."""
     for splits, per in (choose_splits(items, nkv, context, KERNEL_MAX_SPLITS),
                         choose_splits(items, nkv, context, KERNEL_MAX_SPLITS, decoding=True),
-                        choose_lds_splits(items * nkv, context, KERNEL_MAX_SPLITS)):
+                        choose_lds_splits(items * nkv, context, KERNEL_MAX_SPLITS),
+                        choose_lds_splits(items * nkv, context, KERNEL_MAX_SPLITS, head_dim=128)):
         assert 1 <= splits <= KERNEL_MAX_SPLITS
         if splits > 1:
             assert per % 32 == 0 and splits * per >= context and (splits - 1) * per < context
@@ -29,6 +30,22 @@ def test_the_clamp_is_what_bites_for_few_kv_heads():
     assert choose_splits(1, 4, 65536, KERNEL_MAX_SPLITS) == (256, 256)
     assert choose_splits(4096, 8, 2048, KERNEL_MAX_SPLITS) == (1, 0)      # a big prompt fills the GPU by itself
     assert choose_splits(1, 8, 100, KERNEL_MAX_SPLITS) == (1, 0)          # too short to split
+
+
+def test_which_prompt_rows_go_to_the_workgroup_kernel():
+    """Workgroups (128 query rows x kv heads) and mean keys a row decide; head size 128 goes there
+    earlier, and with shorter key ranges."""
+    # a 2,048-token prompt from position 0 on 8 kv heads, 4 query heads each: 512 workgroups, 1,024 keys a row
+    assert not use_lds_kernel(512, 1024.5, 64) and use_lds_kernel(512, 1024.5, 128)
+    assert use_lds_kernel(1024, 2048.5, 64) and use_lds_kernel(1024, 2048.5, 96)
+    assert use_lds_kernel(768, 10, 64)                       # three workgroups per compute unit: whatever they visit
+    # a 256-token portion at position 4,096: 64 workgroups
+    assert not use_lds_kernel(64, 4224.5, 64) and use_lds_kernel(64, 4224.5, 128)
+    assert not use_lds_kernel(64, 1152.5, 128)               # the same portion at position 1,024
+    assert not use_lds_kernel(8, 8000, 128)                  # a 32-token portion: too few rows to share a key block
+    assert choose_lds_splits(64, 4352, KERNEL_MAX_SPLITS, head_dim=128) == (8, 544)
+    assert choose_lds_splits(128, 4608, KERNEL_MAX_SPLITS, head_dim=64) == (4, 1152)
+    assert choose_lds_splits(512, 2048, KERNEL_MAX_SPLITS, head_dim=128) == (1, 0)
 
 
 def test_pool_from_leftover_memory():
