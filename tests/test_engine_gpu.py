@@ -454,11 +454,13 @@ def test_preempted_requests_finish_with_the_tokens_of_an_unpreempted_run(model_d
     assert got_t == want_t
 
 
+@pytest.mark.parametrize("name", ["D", "F"])
 @pytest.mark.parametrize("split_keys", [False, True])
-def test_prompt_portions_through_the_workgroup_attention_kernel(split_keys, model_dirs, gpu, monkeypatch):
+def test_prompt_portions_through_the_workgroup_attention_kernel(split_keys, name, model_dirs, gpu, monkeypatch):
     """The attention kernel that shares key blocks through LDS is chosen for steps with many long
-    rows; with its thresholds lowered it runs on a tiny model: whole prompts, portions that start
-    deep in a request, and portions beside decoded tokens (two launches) all match the plain
+    rows; with its thresholds lowered it runs on a tiny model (head size 32) and on one with the
+    served models' head size of 128, which has thresholds of its own: whole prompts, portions that
+    start deep in a request, and portions beside decoded tokens (two launches) all match the plain
     implementation - also with the keys cut into ranges of 64, one workgroup each, and merged."""
     from kv_cache_optimization_for_llm_amd.ops import attention as policy
     from kv_cache_optimization_for_llm_amd.ops import kernels as K
@@ -473,10 +475,11 @@ def test_prompt_portions_through_the_workgroup_attention_kernel(split_keys, mode
     monkeypatch.setattr(policy, "_LDS_MANY_GROUPS", 1)
     if split_keys:
         monkeypatch.setattr(policy, "_LDS_MIN_KEYS_PER_SPLIT", 64)
+        monkeypatch.setattr(policy, "_LDS_MIN_KEYS_PER_SPLIT_WIDE_HEADS", 64)
     monkeypatch.setattr(K, "attention_lds", counted)
-    cfg, W = plain.load_model_dir(model_dirs["D"])
-    eng = Engine(model_dirs["D"], EngineOptions(dtype="bfloat16", max_seqs=3, max_seq_len=512))
-    pa, pb, pc = prompts_for("D", [300, 140, 77], seed=9)
+    cfg, W = plain.load_model_dir(model_dirs[name])
+    eng = Engine(model_dirs[name], EngineOptions(dtype="bfloat16", max_seqs=3, max_seq_len=512))
+    pa, pb, pc = prompts_for(name, [300, 140, 77], seed=9)
     ref = {k: plain.logits_all(cfg, W, p) for k, p in (("a", pa), ("b", pb), ("c", pc))}
 
     def worst(got, want):
