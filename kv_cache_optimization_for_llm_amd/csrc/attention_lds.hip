@@ -29,7 +29,7 @@
 template <int D>
 struct LdsGeom {
     static constexpr int KROW = D * 2 + 16;          // bytes per key row (D bf16 + pad)
-    static constexpr int VROW = 32 * 2 + 16;         // bytes per value-dimension row (32 keys + pad)
+    static constexpr int VROW = 32 * 2 + 8;          // bytes per value-dimension row (32 keys + pad)
     static constexpr int KBYTES = 32 * KROW;
     static constexpr int VBYTES = D * VROW;
     static constexpr int CHUNKS = 4 * D;             // 16-byte chunks of a K tile (and of a V^T tile)
@@ -173,7 +173,11 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, float *__restrict__ part
                 const int key = c / (D / 8), kc = c % (D / 8);
                 *reinterpret_cast<uint4 *>(buf + key * Geo::KROW + kc * 16) = k;
                 const int t = c / (2 * D), rem = c % (2 * D);
-                *reinterpret_cast<uint4 *>(buf + Geo::KBYTES + (rem >> 1) * Geo::VROW + (t * 16 + (rem & 1) * 8) * 2) = v;
+                // rows of 72 bytes: 18 banks apart, so that the 16 lanes of an 8-byte operand read (rows r = 0..15
+                // of one tile) meet 16 different pairs of the 32 banks; the price is two 8-byte writes here
+                char *vp = buf + Geo::KBYTES + (rem >> 1) * Geo::VROW + (t * 16 + (rem & 1) * 8) * 2;
+                *reinterpret_cast<uint2 *>(vp) = make_uint2(v.x, v.y);
+                *reinterpret_cast<uint2 *>(vp + 8) = make_uint2(v.z, v.w);
             }
         };
         chunk(0, stage_k0, stage_v0);
