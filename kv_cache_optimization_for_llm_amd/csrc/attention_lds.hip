@@ -7,7 +7,8 @@
 // of four wavefronts takes 128 consecutive query rows of one request and kv head (row =
 // token * G + head_in_group, as there), each wavefront 32 of them, and every 32-key block is
 // copied from the pages to LDS once for all four: 16 bytes per thread for K and for V^T, in the
-// pages' own layout, rows padded so that the operand reads do not collide on banks.  The copies of
+// pages' own layout, rows padded so that the operand reads do not collide on the 32 banks (K rows
+// 16 bytes longer, V^T rows 72 bytes apart).  The copies of
 // block i+1 travel (global -> registers) while block i is computed, are written to the other
 // half of LDS afterwards, and one barrier per block separates the two.
 //
