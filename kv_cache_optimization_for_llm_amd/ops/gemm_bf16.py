@@ -29,10 +29,13 @@ from . import kernels as K
 # output projection by the few-rows kernel, 3,072 x 3,072: 2.80 / 2.94 / 3.04 -> 2.74 / 2.89 / 3.02
 # ms; 4,096 x 4,096: 4.55 / 4.75 / 4.91 -> 4.62 / 4.82 / 5.03.  The Q/K/V product with rotation and
 # cache write in its epilogue (it stands for the library's product and the rotation kernel) gains
-# at both: 3B 2.80 -> 2.77 (5,120 x 3,072), 8B 4.55 -> 4.52 (6,144 x 4,096).
+# at both: 3B 2.80 -> 2.77 (5,120 x 3,072), 8B 4.55 -> 4.52 (6,144 x 4,096); for those larger
+# matrices up to 48 rows (decode steps of 40 / 48 requests: 3B 3.26 / 3.25 -> 3.20 / 3.20 ms, 8B 5.17 /
+# 5.16 -> 5.09 / 5.08; at 64 rows a tie at 8B and a loss at 3B; at the 1B sizes a tie at 48 already).
 SKINNY_MAX_ROWS = 16            # every shape
 SKINNY_MID_ROWS = 32            # small or tall matrices, and the Q/K/V product with its epilogue
 SKINNY_MID_ELEMENTS = 3 << 22
+SKINNY_ROTATED_ROWS = 48        # the Q/K/V product with its epilogue, matrices above SKINNY_MID_ELEMENTS
 SKINNY_WIDE_ROWS = 64           # matrices whose waves share X through LDS
 SKINNY_WIDE_N = 32768
 
@@ -46,6 +49,8 @@ def use_skinny(m: int, n: int, k: int, gated: bool = False, rotated: bool = Fals
     if m <= SKINNY_MAX_ROWS:
         return True
     if m <= SKINNY_MID_ROWS and (rotated or n * k <= SKINNY_MID_ELEMENTS or n >= 4 * k):
+        return True
+    if rotated and m <= SKINNY_ROTATED_ROWS and n * k > SKINNY_MID_ELEMENTS:
         return True
     return m <= SKINNY_WIDE_ROWS and (n >= SKINNY_WIDE_N or (gated and n >= 4 * k))
 
