@@ -812,6 +812,12 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
     if (xl) {
         kw = kw < 4 ? kw : 4;
         groups_per_wg = kw == 4 ? 2 : 4;
+        // A workgroup re-reads all of X for its tile groups: with two groups of a joined [gate; up]
+        // matrix that is as many bytes as its share of W.  Where four groups per workgroup still leave
+        // nearly a workgroup per compute unit, K goes over two ranges of waves instead of four and a
+        // workgroup takes four groups (8B sizes, 896 groups: decode steps of 48 / 64 requests
+        // 5.05 / 5.48 -> 4.96 / 5.30 ms; with 512 groups, 128 workgroups, 5 % slower).
+        if (kw == 4 && groups / 4 >= compute_units() * 7 / 8) { kw = 2; groups_per_wg = 4; }
     }
     a.k_waves = kw;
     const int waves = kw * groups_per_wg;

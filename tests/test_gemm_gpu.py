@@ -49,7 +49,7 @@ def test_skinny_product_of_vocabulary_sized_matrices(m, n, k, gpu):
 
 
 @pytest.mark.parametrize("m", [1, 5, 16, 40, 64])
-@pytest.mark.parametrize("inter, k", [(16, 64), (250, 96), (8192, 2048), (56, 160)])
+@pytest.mark.parametrize("inter, k", [(16, 64), (250, 96), (8192, 2048), (56, 160), (14336, 512)])
 def test_skinny_product_with_swiglu_epilogue(m, inter, k, gpu):
     x, w = rnd(m, k), rnd(2 * inter, k, scale=0.2, seed=2)
     g = x.double() @ w[:inter].double().t()
