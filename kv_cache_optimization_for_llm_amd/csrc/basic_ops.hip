@@ -28,10 +28,11 @@ void kva_set_error(const char *fmt, ...) {
 template <typename TW, typename TO>
 __global__ void embed_gather_kernel(TO *__restrict__ out, const TW *__restrict__ table,
                                     const int *__restrict__ ids, const int *__restrict__ feedback,
-                                    int width) {
+                                    int width, int table_rows) {
     const int row = blockIdx.x;
     int id = ids[row];
     if (id < 0) id = feedback[-1 - id];
+    id = id < 0 ? 0 : (id >= table_rows ? table_rows - 1 : id);      // whatever a kernel left there: inside the table
     const TW *src = table + (size_t)id * width;
     TO *dst = out + (size_t)row * width;
     for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = from_float<TO>(to_float(src[i]));
@@ -39,13 +40,15 @@ __global__ void embed_gather_kernel(TO *__restrict__ out, const TW *__restrict__
 
 // feedback may be null when no id is negative (the caller checks the ids it uploads).
 extern "C" int kva_embed_gather(void *out, const void *table, const int *ids, const int *feedback,
-                                int rows, int width, int table_dtype, int out_dtype, hipStream_t stream) {
-    KVA_REQUIRE(rows >= 0 && width > 0, "embed_gather: bad sizes rows=%d width=%d", rows, width);
+                                int rows, int width, int table_rows, int table_dtype, int out_dtype,
+                                hipStream_t stream) {
+    KVA_REQUIRE(rows >= 0 && width > 0 && table_rows > 0, "embed_gather: bad sizes rows=%d width=%d table rows=%d",
+                rows, width, table_rows);
     if (rows == 0) return KVA_OK;
     dim3 grid(rows), block(256);
 #define LAUNCH(TW, TO)                                                                    \
     hipLaunchKernelGGL((embed_gather_kernel<TW, TO>), grid, block, 0, stream, (TO *)out, \
-                       (const TW *)table, ids, feedback, width)
+                       (const TW *)table, ids, feedback, width, table_rows)
     if (table_dtype == KVA_F32 && out_dtype == KVA_F32) LAUNCH(float, float);
     else if (table_dtype == KVA_BF16 && out_dtype == KVA_BF16) LAUNCH(bf16_t, bf16_t);
     else if (table_dtype == KVA_F32 && out_dtype == KVA_BF16) LAUNCH(float, bf16_t);
@@ -129,11 +132,13 @@ template <typename TW>
 __global__ void __launch_bounds__(256)
 embed_gather_prep_kernel(bf16_t *__restrict__ hidden, bf16_t *__restrict__ scaled, float *__restrict__ sumsq,
                          const bf16_t *__restrict__ table, const int *__restrict__ ids,
-                         const int *__restrict__ feedback, const TW *__restrict__ norm_w, int width) {
+                         const int *__restrict__ feedback, const TW *__restrict__ norm_w, int width,
+                         int table_rows) {
     __shared__ float scratch[4];
     const int row = blockIdx.x;
     int id = ids[row];
     if (id < 0) id = feedback[-1 - id];
+    id = id < 0 ? 0 : (id >= table_rows ? table_rows - 1 : id);
     const bf16_t *src = table + (size_t)id * width;
     float ss = 0.f;
     for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8) {
@@ -156,18 +161,18 @@ embed_gather_prep_kernel(bf16_t *__restrict__ hidden, bf16_t *__restrict__ scale
 // bf16 table and outputs, width a multiple of 8; norm_w [width] bf16 or fp32.
 extern "C" int kva_embed_gather_prep(void *hidden, void *scaled, float *sumsq, const void *table, const int *ids,
                                      const int *feedback, const void *norm_w, int norm_w_f32, int rows, int width,
-                                     hipStream_t stream) {
-    KVA_REQUIRE(rows >= 0 && width > 0 && width % 8 == 0, "embed_gather_prep: bad sizes rows=%d width=%d (a multiple of 8)",
-                rows, width);
+                                     int table_rows, hipStream_t stream) {
+    KVA_REQUIRE(rows >= 0 && width > 0 && width % 8 == 0 && table_rows > 0,
+                "embed_gather_prep: bad sizes rows=%d width=%d (a multiple of 8) table rows=%d", rows, width, table_rows);
     KVA_REQUIRE(hidden && scaled && sumsq && table && ids && norm_w, "embed_gather_prep: a pointer is missing");
     if (rows == 0) return KVA_OK;
     dim3 grid(rows), block(256);
     if (norm_w_f32)
         hipLaunchKernelGGL(embed_gather_prep_kernel<float>, grid, block, 0, stream, (bf16_t *)hidden, (bf16_t *)scaled,
-                           sumsq, (const bf16_t *)table, ids, feedback, (const float *)norm_w, width);
+                           sumsq, (const bf16_t *)table, ids, feedback, (const float *)norm_w, width, table_rows);
     else
         hipLaunchKernelGGL(embed_gather_prep_kernel<bf16_t>, grid, block, 0, stream, (bf16_t *)hidden, (bf16_t *)scaled,
-                           sumsq, (const bf16_t *)table, ids, feedback, (const bf16_t *)norm_w, width);
+                           sumsq, (const bf16_t *)table, ids, feedback, (const bf16_t *)norm_w, width, table_rows);
     KVA_CHECK_LAUNCH("embed_gather_prep");
     return KVA_OK;
 }

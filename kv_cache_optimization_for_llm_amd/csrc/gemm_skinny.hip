@@ -819,6 +819,8 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
         // 5.05 / 5.48 -> 4.96 / 5.30 ms; with 512 groups, 128 workgroups, 5 % slower).
         if (kw == 4 && groups / 4 >= compute_units() * 7 / 8) { kw = 2; groups_per_wg = 4; }
     }
+    // the waves of a K range bring X to LDS together, 64 of a chunk's 128 units per row tile each
+    KVA_REQUIRE(!xl || groups_per_wg >= 2, "gemm_skinny: the shared-X form needs two tile groups per workgroup");
     a.k_waves = kw;
     const int waves = kw * groups_per_wg;
     size_t lds = kw > 1 ? (size_t)waves * ntw * 64 * 4 * sizeof(float) : 0;
@@ -887,6 +889,7 @@ extern "C" int kva_gemm_skinny_qkv_rope(void *q_out, int ldq, const void *X, con
         kw = kw < 4 ? kw : 4;
         groups_per_wg = kw == 4 ? 2 : 4;
     }
+    KVA_REQUIRE(!xl || groups_per_wg >= 2, "gemm_skinny_qkv_rope: the shared-X form needs two tile groups per workgroup");
     a.k_waves = kw;
     const int waves = kw * groups_per_wg;
     size_t lds = kw > 1 ? (size_t)waves * 2 * 64 * 4 * sizeof(float) : 0;

@@ -283,6 +283,10 @@ sample_pick_kernel(const float *__restrict__ logits, int vocab, int chunk_tokens
         }
         token = __shfl(found, owner < 0 ? 0 : owner, KVA_WAVE);
     }
+    // A row whose logits are all NaN (or all -inf) has no best token: nothing compares greater than
+    // the start value and the index stays at `vocab`.  Token 0 then: the next step looks its token
+    // up in the embedding table on the device, and a row past the table's end is a memory fault.
+    if (token < 0 || token >= vocab) token = 0;
     if (lane == 0) {
         out_tokens[row] = token;
         if (host_tokens != nullptr) host_tokens[row] = token;      // pinned host memory, mapped for the device

@@ -71,14 +71,16 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor,
                  feedback: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[t, :] = table[ids[t], :], converted to out's dtype.  A negative id ``-1 - r`` stands
     for ``feedback[r]`` (a token still on the device); the caller guarantees ``r`` is inside
-    ``feedback`` and that no id is negative when there is none."""
+    ``feedback`` and that no id is negative when there is none.  An id outside the table (only
+    what a kernel left in ``feedback`` can be: the host checks the ids it uploads) reads the
+    nearest row of it."""
     rows, width = out.shape
     if table.dim() != 2 or table.shape[1] != width or ids.shape != (rows,):
         raise KernelError(f"embed_gather: shapes table {tuple(table.shape)} ids {tuple(ids.shape)} "
                           f"out {tuple(out.shape)} do not fit")
     check(hip_lib().kva_embed_gather(_dev(out, "out"), _dev(table, "table"),
                                      _dev(ids, "ids", torch.int32),
-                                     _opt(feedback, "feedback", torch.int32), rows, width,
+                                     _opt(feedback, "feedback", torch.int32), rows, width, table.shape[0],
                                      dtype_code(table.dtype), dtype_code(out.dtype), _stream()),
           "embed_gather")
     return out
@@ -100,7 +102,7 @@ def embed_gather_prep(table: torch.Tensor, ids: torch.Tensor, hidden: torch.Tens
     check(hip_lib().kva_embed_gather_prep(
         _dev(hidden, "hidden"), _dev(scaled, "scaled"), _dev(sumsq, "sumsq", torch.float32), _dev(table, "table"),
         _dev(ids, "ids", torch.int32), _opt(feedback, "feedback", torch.int32), _dev(norm_weight, "norm_weight"),
-        1 if norm_weight.dtype == torch.float32 else 0, rows, width, _stream()), "embed_gather_prep")
+        1 if norm_weight.dtype == torch.float32 else 0, rows, width, table.shape[0], _stream()), "embed_gather_prep")
     return hidden
 
 

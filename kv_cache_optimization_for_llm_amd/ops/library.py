@@ -32,8 +32,8 @@ LL = c_longlong
 U = c_uint
 
 _HIP_SIGNATURES = {
-    "kva_embed_gather": [P, P, P, P, I, I, I, I, P],
-    "kva_embed_gather_prep": [P, P, P, P, P, P, P, I, I, I, P],
+    "kva_embed_gather": [P, P, P, P, I, I, I, I, I, P],
+    "kva_embed_gather_prep": [P, P, P, P, P, P, P, I, I, I, I, P],
     "kva_rmsnorm": [P, P, P, P, P, I, I, F, I, I, P, I, I, P],
     "kva_residual_add": [P, P, LL, I, P],
     "kva_scale_softcap": [P, LL, F, F, I, P],

@@ -36,6 +36,38 @@ def test_embed_gather(dtype, table_dtype, gpu):
     assert torch.equal(out.cpu(), want)
 
 
+def test_logits_without_a_best_token_still_name_a_token_of_the_table(gpu):
+    """A row of logits that are all NaN or all -inf has no best token.  The sampler names token 0
+    for it (greedy and sampled rows alike stay inside the vocabulary), and a lookup of whatever a
+    kernel left in the feedback buffer stays inside the table: the token of such a row is looked
+    up on the device by the next step, where a row past the table's end is a memory fault, not an
+    error message."""
+    vocab = 333
+    lg = torch.randn(4, vocab)
+    lg[0] = float("nan")
+    lg[1] = float("-inf")
+    lg[3] = float("nan")
+    lg = lg.to(gpu)
+    out = torch.full((4,), -7, dtype=torch.int32, device=gpu)
+    K.sample(lg, out, chunks=4)
+    assert out.cpu().tolist() == [0, 0, int(lg[2].argmax()), 0]
+    inv_t = torch.tensor([1.0, 1.25, 0.0, 2.0], device=gpu)
+    zeros = torch.zeros(4, dtype=torch.int32, device=gpu)
+    K.sample(lg, out, chunks=4, inv_temperature=inv_t, seed=5, rng_key=zeros, rng_step=zeros)
+    got = out.cpu().tolist()
+    assert all(0 <= t < vocab for t in got) and got[2] == int(lg[2].argmax())
+    table = rnd(vocab, 64, dtype=torch.bfloat16)
+    feedback = torch.tensor([vocab, -9, 1 << 30, 5], dtype=torch.int32)
+    ids = torch.tensor([-1, -2, -3, -4], dtype=torch.int32)
+    emb = torch.empty(4, 64, dtype=torch.bfloat16, device=gpu)
+    K.embed_gather(table.to(gpu), ids.to(gpu), emb, feedback.to(gpu))
+    assert torch.equal(emb.cpu(), table[[vocab - 1, 0, vocab - 1, 5]])
+    hidden, scaled = torch.empty_like(emb), torch.empty_like(emb)
+    sumsq = torch.empty((4, 1), device=gpu)
+    K.embed_gather_prep(table.to(gpu), ids.to(gpu), hidden, scaled, sumsq, torch.ones(64).to(gpu), feedback.to(gpu))
+    assert torch.equal(hidden.cpu(), table[[vocab - 1, 0, vocab - 1, 5]])
+
+
 @pytest.mark.parametrize("width", [8, 520, 2048, 4104])
 @pytest.mark.parametrize("weight_dtype", ["float32", "bfloat16"])
 def test_embed_gather_that_prepares_the_first_norm(width, weight_dtype, gpu):
