@@ -39,6 +39,8 @@ _PAIR_MIN_WAVES = 2048      # two items per wavefront once that still leaves a w
 _LDS_MIN_GROUPS = 128
 _LDS_MANY_GROUPS = 768
 _LDS_MIN_MEAN_KEYS = 2048
+_LDS_SOME_GROUPS = 576
+_LDS_SOME_GROUPS_MEAN_KEYS = 1024
 # Head sizes above 96 do twice the matrix-core work per key and row for the same vector work, and
 # one wavefront with two row tiles of them fills its SIMD's registers alone: there the workgroup kernel
 # (two workgroups per compute unit) is ahead from 1,024 keys a row on (head size 128, a 2,048-token
@@ -51,7 +53,8 @@ _LDS_MIN_MEAN_KEYS_WIDE_HEADS = 1024
 _LDS_MIN_GROUPS_WIDE_HEADS = 16
 _LDS_TARGET_GROUPS_WIDE_HEADS = 512
 _LDS_MIN_KEYS_PER_SPLIT_WIDE_HEADS = 256
-LDS_MEAN_KEYS_STEPS = (_LDS_MIN_MEAN_KEYS_WIDE_HEADS, _LDS_MIN_MEAN_KEYS)     # where the choice can change
+# where the choice can change (a step shape that has a graph is told apart by these too)
+LDS_MEAN_KEYS_STEPS = tuple(sorted({_LDS_MIN_MEAN_KEYS_WIDE_HEADS, _LDS_SOME_GROUPS_MEAN_KEYS, _LDS_MIN_MEAN_KEYS}))
 # few workgroups that each walk thousands of keys: the keys are cut into ranges, one workgroup each
 _LDS_TARGET_GROUPS = 1024
 _LDS_MIN_KEYS_PER_SPLIT = 1024
@@ -66,7 +69,12 @@ def use_lds_kernel(groups: int, mean_keys: float, head_dim: int) -> bool:
         if groups >= _LDS_MIN_GROUPS:
             return mean_keys >= _LDS_MIN_MEAN_KEYS_WIDE_HEADS
         return groups >= _LDS_MIN_GROUPS_WIDE_HEADS and mean_keys >= _LDS_MIN_MEAN_KEYS
-    return groups >= _LDS_MIN_GROUPS and mean_keys >= _LDS_MIN_MEAN_KEYS
+    if groups >= _LDS_MIN_GROUPS and mean_keys >= _LDS_MIN_MEAN_KEYS:
+        return True
+    # Between 512 and 768 workgroups, whole prefill passes at the 1B sizes (one prompt from position 0):
+    # 2,048 tokens (512 workgroups) 5.74 ms with the one-wavefront kernel against 6.03, but 2,304 tokens
+    # 7.15 against 6.90, 2,560 7.66 against 7.36, 2,816 8.58 against 8.08.
+    return groups >= _LDS_SOME_GROUPS and mean_keys >= _LDS_SOME_GROUPS_MEAN_KEYS
 
 
 def _cut_keys(want: int, max_context: int, max_splits: int) -> tuple:

@@ -39,6 +39,7 @@ def test_which_prompt_rows_go_to_the_workgroup_kernel():
     assert not use_lds_kernel(512, 1024.5, 64) and use_lds_kernel(512, 1024.5, 128)
     assert use_lds_kernel(1024, 2048.5, 64) and use_lds_kernel(1024, 2048.5, 96)
     assert use_lds_kernel(768, 10, 64)                       # three workgroups per compute unit: whatever they visit
+    assert use_lds_kernel(576, 1152.5, 64) and not use_lds_kernel(576, 500, 64)      # a 2,304-token prompt; many short ones
     # a 256-token portion at position 4,096: 64 workgroups
     assert not use_lds_kernel(64, 4224.5, 64) and use_lds_kernel(64, 4224.5, 128)
     assert not use_lds_kernel(64, 1152.5, 128)               # the same portion at position 1,024
