@@ -343,7 +343,9 @@ class Scheduler:
                                              head.max_new_tokens + head.resumed_tokens, cache.max_seq_len)
             seat = cache.admit(head.id, reserve)
             if seat is None:
-                if not paged and not self.running:
+                # given up only when nothing can still free room: a request that waits for its
+                # last token's value (``closing``) holds its run one more step and then leaves
+                if not paged and not self.running and not self.closing:
                     self.waiting.popleft()
                     events.append(Event("done", head.id, head.seq_index, tokens=head.resumed_tokens,
                                         reason="kv_cache_exhausted"))

@@ -330,12 +330,66 @@ def test_prompts_admitted_together_are_counted_with_the_pages_they_still_need():
         assert p.entries or p.events, "a plan with nothing to run and nothing to report"
 
 
+@pytest.mark.parametrize("policy", ["max", "pow2", "oracle"])
+def test_running_ahead_in_contiguous_mode_makes_the_head_wait_for_a_closing_request(policy):
+    """Three equal requests, a pool for two reservations of the longest sequence: the third has to
+    wait, also while the two before it only wait for their last token's value (they hold their
+    runs one step longer when the loop runs ahead).  The reference's queue head blocks until its
+    reservation can be placed and nothing that fits is refused (``base/src/engine.cu:432-437``)."""
+    def make():
+        s = Scheduler(cache(pages=16, seqs=4, mode="contiguous", max_len=128), reserve_policy=policy,
+                      max_batch_tokens=64, ignore_eos=True)
+        for i in range(3):
+            s.add(Request(i, [9] * 10, 3))
+        return s
+    want_out, want_reasons, _, _ = run(make())
+    assert all(r == "length" for r in want_reasons.values()) and len(want_reasons) == 3
+    s = make()
+    out, reasons, _, _ = run_ahead(s)
+    assert out == want_out and reasons == want_reasons
+    assert s.preemptions == 0 and s.cache.free_seats == 4
+
+
+@pytest.mark.parametrize("policy", ["max", "pow2", "oracle"])
+@pytest.mark.parametrize("seed", range(12))
+def test_running_ahead_gives_the_synchronous_loops_results_in_contiguous_mode(seed, policy):
+    """Random requests with end-of-sequence tokens on a pool that holds two or three reservations:
+    the same tokens and the same reasons from both loops, and a request is failed only if its
+    reservation cannot be placed in an empty pool."""
+    import numpy as np
+    rng = np.random.default_rng(1000 + seed)
+    eos = EOS + 8
+    lens = [int(x) for x in rng.integers(1, 60, int(rng.integers(3, 9)))]
+    news = [int(x) for x in rng.integers(1, 40, len(lens))]
+    max_len = 128
+    pages = int(rng.integers(8, 24))                    # pages of 16: 128 to 384 tokens
+
+    def make():
+        s = Scheduler(cache(pages=pages, seqs=4, mode="contiguous",
+                            max_len=max_len), reserve_policy=policy, max_batch_tokens=48,
+                      chunk_size=16, eos_token_ids=[eos])
+        for i, (n, k) in enumerate(zip(lens, news)):
+            s.add(Request(i, [20 + (j % 50) for j in range(n)], k))
+        return s
+
+    want_out, want_reasons, _, _ = run(make())
+    s = make()
+    out, reasons, _, _ = run_ahead(s)
+    assert out == want_out and reasons == want_reasons
+    assert set(want_reasons.values()) <= {"length", "eos", "sequence_too_long"}
+    assert s.preemptions == 0 and s.cache.free_seats == 4
+    s.cache.check()
+
+
+@pytest.mark.parametrize("mode", ["paged", "contiguous"])
 @pytest.mark.parametrize("ahead", [False, True])
 @pytest.mark.parametrize("seed", range(40))
-def test_random_tight_pools_always_finish(seed, ahead):
+def test_random_tight_pools_always_finish(seed, ahead, mode):
     """Random prompts, budgets, portion sizes, page sizes and pools barely larger than the longest
     request: every request ends, with its full budget of the right tokens unless the cache
-    could not hold it, and no page is lost."""
+    could not hold it, and no page is lost.  In contiguous mode a request reserves a power-of-two
+    run of pages; one whose run is larger than the largest the pool can ever place fails alone, in
+    both loops alike, and every other gets its full budget."""
     import numpy as np
     rng = np.random.default_rng(seed)
     page = int(rng.choice([16, 8, 4]))
@@ -345,12 +399,23 @@ def test_random_tight_pools_always_finish(seed, ahead):
     longest = max(lens) + new + 1
     pool = int(rng.integers(longest + page, seats * longest + 2 * page))
     chunk = int(rng.choice([0, 8, 24, 64])) or None
-    s = Scheduler(cache(pages=(pool + page - 1) // page, seqs=seats, page=page, max_len=longest),
-                  max_batch_tokens=int(rng.choice([32, 64, 256])), chunk_size=chunk, ignore_eos=True)
+    policy = str(rng.choice(["max", "pow2", "oracle"]))
+    s = Scheduler(cache(pages=(pool + page - 1) // page, seqs=seats, page=page, max_len=longest, mode=mode),
+                  max_batch_tokens=int(rng.choice([32, 64, 256])), chunk_size=chunk, ignore_eos=True,
+                  reserve_policy=policy)
     for i, n in enumerate(lens):
         s.add(Request(i, [8 + (j % 30) for j in range(n)], new))
     out, reasons, events, plans = (run_ahead if ahead else run)(s, max_steps=4000)
     for i, n in enumerate(lens):
+        if mode == "contiguous":
+            # what the request reserves, as a run of pages rounded up to a power of two, against
+            # the largest run an empty pool of this size holds
+            run_pages = -(-reservation_tokens(policy, n, new, longest) // page)
+            run_pages = 1 << (run_pages - 1).bit_length()
+            pool_pages = (pool + page - 1) // page
+            if run_pages > 1 << (pool_pages.bit_length() - 1):
+                assert reasons[(i, 0)] == "kv_cache_exhausted" and (i, 0) not in out, (i, reasons)
+                continue
         assert reasons[(i, 0)] == "length", (i, reasons)
         assert out[(i, 0)] == [fake_token(i, n + k) for k in range(new)]
     s.cache.check()
