@@ -11,7 +11,9 @@ time / HBM peak, and against what a plain read stream gets from this GPU); ``poi
 batch 64 at the same context and batches 1, 8 and 64 with 512-token prompts and 256 generated
 tokens, each with its step time, bytes and fraction of the HBM peak, and the serving loop at the
 3B and 8B layer sizes (mixed prompt lengths; paged against contiguous cache occupancy).
-``--kernel-classes`` adds device time per class of kernel.
+``points`` also holds the device time per class of kernel of one decode step and of the prefill
+(``kclass_...``; ``--no-kernel-classes`` leaves them out) and, for the serving runs, pages reused,
+preemptions and fragmentation failures.
 """
 import argparse
 import json
@@ -74,9 +76,9 @@ def main():
     ap.add_argument("--skip-points", action="store_true", help="only the default decode run and the prefill")
     ap.add_argument("--skip-large", action="store_true",
                     help="leave out the serving runs at the 3B and 8B layer sizes (about a minute together)")
-    ap.add_argument("--kernel-classes", action="store_true",
-                    help="also time one decode step and the prefill kernel class by kernel class (events around "
-                         "every launch, steps launched one by one instead of replayed from graphs)")
+    ap.add_argument("--no-kernel-classes", dest="kernel_classes", action="store_false",
+                    help="leave out the device time per class of kernel (one decode step and the prefill with events "
+                         "around every launch, launched one by one instead of replayed from graphs: a second or two)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")
@@ -144,9 +146,9 @@ def main():
         assert len(sched.running) == batch and max(s.computed for s in sched.running) <= context
         mean_ctx = ctx0 + steps / 2
         # drop the requests (their remaining budget is not part of the measurement)
-        runner._resolve_in_flight()
-        for s_ in list(sched.running) + list(sched.closing):
-            sched._finish(s_, "length", [])
+        for rid in runner.live_requests():
+            runner.cancel(rid)
+        assert runner.idle()
         return dt, mean_ctx
 
     dt, mean_ctx = decode_run(args.batch, args.steps, args.warmup, ctx)
@@ -265,7 +267,9 @@ def main():
         points.update({"serve_3b_mixed_b32_tok_s": round(r["tokens_emitted"] / r["wall_s"], 1),
                        "serve_3b_mixed_b32_wall_s": r["wall_s"], "serve_3b_mixed_b32_prefill_tok_s": r["prefill_tok_s"],
                        "serve_3b_mixed_b32_decode_tok_s": r["decode_tok_s"],
-                       "serve_3b_mixed_b32_decode_frac": r.get("decode_hbm_frac")})
+                       "serve_3b_mixed_b32_decode_frac": r.get("decode_hbm_frac"),
+                       "serve_3b_mixed_b32_pages_reused": r["pages_reused"],
+                       "serve_3b_mixed_b32_preemptions": r["preemptions"]})
         gc.collect()
         torch.cuda.empty_cache()
         long = sweep.build_parser().parse_args(
@@ -278,7 +282,9 @@ def main():
                            key + "_prefill_tok_s": r["prefill_tok_s"], key + "_wall_s": r["wall_s"],
                            key + "_kv_tokens_reserved": r["peak_kv_tokens_reserved"],
                            key + "_kv_tokens_live": r["peak_kv_tokens_live"],
-                           key + "_reserved_over_live": r["reserved_over_live"]})
+                           key + "_reserved_over_live": r["reserved_over_live"],
+                           key + "_pages_reused": r["pages_reused"], key + "_preemptions": r["preemptions"],
+                           key + "_fragmentation_failures": r["fragmentation_failures"]})
             gc.collect()
             torch.cuda.empty_cache()
 
@@ -302,6 +308,12 @@ def main():
     }
     if kernel_ms is not None:
         out["kernel_ms"] = kernel_ms
+        for run, classes in kernel_ms.items():          # and flat, beside the other points
+            for cls, ms in classes.items():
+                name = "".join(c if c.isalnum() else "_" for c in cls).strip("_")
+                while "__" in name:
+                    name = name.replace("__", "_")
+                points[f"kclass_{run}_{name}_ms"] = ms
     print(json.dumps(out))
     return 0
 

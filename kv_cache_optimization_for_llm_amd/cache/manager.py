@@ -1,13 +1,15 @@
 """The cache manager: paged keys and values with a block table per request, per-request state
 slots, and the contiguous (buddy) mode as a second way of handing out the same pages.
 
-Layout.  Mixer calls with the same needs (:class:`~..parts.base.KVCacheSpec`: heads, head size,
-all keys or a window) form a *group*.  A group owns a pool of ``num_pages`` pages and one block
-table ``[seats, max_blocks]``; a page holds ``page_size`` tokens of every cache slot of the group
-(slot = one mixer call's K array ``[pages, kv_heads, page_size, head_dim]`` and V array
-``[pages, kv_heads, head_dim, page_size]``), so one
-table row serves all layers of the group.  Groups with other needs have pools and tables of
-their own.
+Layout.  Mixer calls with the same needs (:class:`~..parts.base.KVCacheSpec`: the arrays kept per
+token - names, per-token shapes, layout inside a page - and whether all positions stay or a
+window of them) form a *group*.  A group owns a pool of ``num_pages`` pages and one block table
+``[seats, max_blocks]``; a page holds ``page_size`` tokens of every array of every cache slot of
+the group (slot = one mixer call's arrays, each ``[pages, *page_shape]``: for attention a K array
+``[pages, kv_heads, page_size, head_dim]`` and a V array ``[pages, kv_heads, head_dim,
+page_size]``), so one table row serves all layers of the group.  Groups with other needs have
+pools and tables of their own.  The manager allocates what the description says and hands the
+arrays over by name; it never looks inside them.
 
 Paged mode (reference: ``paged_attention/src/engine.cu:176-254, 376-454``): pages are taken one
 by one as a request grows, dropped when it ends or - in a window group - once every position
@@ -38,6 +40,11 @@ class CacheError(RuntimeError):
     pass
 
 
+def page_bytes(group_specs, page_size: int, dtype) -> int:
+    """Bytes of one page over all groups: every array of every cache slot, ``page_size`` tokens."""
+    return sum(len(slots) * spec.bytes_per_token(dtype) * int(page_size) for spec, slots in group_specs)
+
+
 @dataclass
 class _Seat:
     request_id: object
@@ -58,8 +65,7 @@ class CacheGroup:
         self.table_host = np.full((max_seqs, max_blocks), -1, dtype=np.int32)
         self.table_dev = None
         self._table_pinned = None
-        self.k = None          # [slots, pages, kv_heads, page_size, head_dim]
-        self.v = None
+        self.arrays: Dict[str, object] = {}     # name -> [slots, pages, *page_shape] on the device
         self.dirty: Dict[int, List[int]] = {}
 
     def free_pages(self) -> int:
@@ -117,10 +123,9 @@ class CacheManager:
     def _allocate_device(self) -> None:
         import torch
         for g in self.groups:
-            n, kvh, d = len(g.slot_ids), g.spec.num_kv_heads, g.spec.head_dim
-            g.k = torch.zeros((n, g.num_pages, kvh, g.page_size, d), dtype=self.dtype, device=self.device)
-            # V pages are stored transposed (see csrc/rope_cache.hip)
-            g.v = torch.zeros((n, g.num_pages, kvh, d, g.page_size), dtype=self.dtype, device=self.device)
+            for a in g.spec.arrays:
+                g.arrays[a.name] = torch.zeros((len(g.slot_ids), g.num_pages, *a.page_shape(g.page_size)),
+                                               dtype=a.dtype or self.dtype, device=self.device)
             pinned = torch.full((self.max_seqs, self.max_blocks), -1, dtype=torch.int32,
                                 pin_memory=True)
             g._table_pinned = pinned
@@ -153,11 +158,16 @@ class CacheManager:
             self._flush_event = None
 
     def kv_arrays(self, cache_slot: int):
+        """(group, {array name: the slot's ``[pages, *page_shape]`` tensor})."""
         for g in self.groups:
             if cache_slot in g.slot_ids:
                 i = g.slot_of(cache_slot)
-                return g, g.k[i], g.v[i]
+                return g, {name: t[i] for name, t in g.arrays.items()}
         raise CacheError(f"cache slot {cache_slot} belongs to no group")
+
+    def page_bytes(self) -> int:
+        """Bytes one page takes over all groups, slots and arrays."""
+        return page_bytes(((g.spec, g.slot_ids) for g in self.groups), self.page_size, self.dtype)
 
     def group_of(self, cache_slot: int) -> Optional[CacheGroup]:
         for g in self.groups:

@@ -35,7 +35,7 @@ import threading
 import time
 from typing import Dict, Optional, Tuple
 
-MAX_PARALLEL_SEQUENCES = 8        # reference: base/src/config.h:97
+from ..engine.runner import MAX_PARALLEL_SEQUENCES       # reference: base/src/config.h:97
 STEP_TELEMETRY_EVERY = 8          # reference: base/src/config.h:170
 
 
@@ -47,22 +47,21 @@ def parse_request_line(line: str) -> Optional[Tuple[int, int, int, list]]:
     try:
         rid = int(fields[0])
     except ValueError:
-        print(f"Malformed input line (no request id), ignoring: {line.strip()}", file=sys.stderr)
+        print(f"request line dropped, it does not start with an integer id: {line.strip()!r}", file=sys.stderr)
         return None
     try:
         max_tokens = int(fields[1])
         if max_tokens < 1:
             raise ValueError
     except (IndexError, ValueError):
-        print(f"Request {rid} has no usable output budget, ignoring", file=sys.stderr)
+        print(f"request {rid} dropped: max_tokens is missing or below 1", file=sys.stderr)
         return None
     try:
         n_seqs = int(fields[2])
         if not 1 <= n_seqs <= MAX_PARALLEL_SEQUENCES:
             raise ValueError
     except (IndexError, ValueError):
-        print(f"Request {rid}: n_seqs field is outside 1..{MAX_PARALLEL_SEQUENCES}, ignoring the request",
-              file=sys.stderr)
+        print(f"request {rid} dropped: n_seqs is missing or not in 1..{MAX_PARALLEL_SEQUENCES}", file=sys.stderr)
         return None
     tokens = []
     for f in fields[3:]:
@@ -71,9 +70,20 @@ def parse_request_line(line: str) -> Optional[Tuple[int, int, int, list]]:
         except ValueError:
             break
     if not tokens:
-        print(f"Request {rid} carries no tokens, ignoring", file=sys.stderr)
+        print(f"request {rid} dropped: no prompt token ids follow its three header fields", file=sys.stderr)
         return None
     return rid, max_tokens, n_seqs, tokens
+
+
+def serve_tune_rows(max_seqs: int, chunk_size: Optional[int], max_batch_tokens: int) -> list:
+    """Row counts a server has the vendor library's algorithms timed for: its decode batches and
+    the size of the prompt portions its steps are mostly made of."""
+    from ..ops.gemm_bf16 import decode_tune_rows
+    rows = decode_tune_rows(max_seqs)
+    portion = min(int(chunk_size or max_batch_tokens), int(max_batch_tokens))
+    if portion > max_seqs and portion not in rows:
+        rows.append(portion)
+    return rows
 
 
 def _reader(inbox: "queue.Queue") -> None:
@@ -105,7 +115,8 @@ def main(argv=None) -> int:
                     help="comma list of row counts (tokens per step) for which the vendor GEMM library's "
                          "algorithms are timed at start-up (a few seconds); smaller row counts down to half "
                          "share what is found.  'auto': the powers of two from 32 up to the number of seats, "
-                         "and that number; '' for none")
+                         "that number, and the size of a prompt portion (--chunk-size, else "
+                         "--max-batch-tokens); '' for none")
     args = ap.parse_args(argv)
     if not args.model_dir:
         print("no model folder: pass it as the first argument or set MODEL_DIR", file=sys.stderr)
@@ -131,14 +142,12 @@ def main(argv=None) -> int:
 
     from ..engine.engine import Engine, EngineOptions
     from ..engine.runner import Runner, ServeOptions
-    from ..ops.gemm_bf16 import decode_tune_rows
-
     engine = Engine(args.model_dir, EngineOptions(
         dtype=args.dtype, cache_mode=args.cache_mode, page_size=args.page_size, max_seqs=args.max_seqs,
         max_seq_len=args.max_seq_len, cache_tokens=args.cache_tokens, max_batch_tokens=args.max_batch_tokens,
         max_logit_rows=args.max_seqs,         # one sampled token per request and step
-        gemm_tune_rows=decode_tune_rows(args.max_seqs) if args.gemm_tune_rows == "auto"
-        else [int(r) for r in args.gemm_tune_rows.split(",") if r.strip()]))
+        gemm_tune_rows=serve_tune_rows(args.max_seqs, args.chunk_size, args.max_batch_tokens)
+        if args.gemm_tune_rows == "auto" else [int(r) for r in args.gemm_tune_rows.split(",") if r.strip()]))
     runner = Runner(engine, ServeOptions(
         temperature=temperature, sampling_seed=seed, ignore_eos=ignore_eos, repetition_penalty=penalty,
         max_batch_tokens=args.max_batch_tokens, chunk_size=args.chunk_size, reserve_policy=policy))

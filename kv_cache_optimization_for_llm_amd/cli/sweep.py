@@ -104,6 +104,8 @@ def run_one(args, shape: str, batch: int, mode: str) -> dict:
     peak_reserved = peak_live = 0
     decode_steps = decode_tokens = seen_decode_steps = 0
     decode_time = 0.0
+    decode_bytes = 0.0
+    wbytes, kvbytes = weight_bytes(cfg), kv_bytes_per_token(cfg)
     reasons: Dict[str, int] = {}
     torch.cuda.synchronize()
     t_start = time.perf_counter()
@@ -111,6 +113,9 @@ def run_one(args, shape: str, batch: int, mode: str) -> dict:
     last = t_start
     while not runner.idle():
         prefilling = bool(sched.waiting) or any(s.prefilling for s in sched.running)
+        # what this step has to read if it is a decode step: every weight once and the keys and
+        # values of the requests that are still decoding (early finishers have left)
+        step_bytes = wbytes + kvbytes * sum(s.computed + 1 for s in sched.running)
         events = runner.step()
         now = time.perf_counter()
         tokens = sum(1 for e in events if e.kind == "token")
@@ -129,6 +134,7 @@ def run_one(args, shape: str, batch: int, mode: str) -> dict:
                 decode_steps += 1
                 decode_tokens += tokens
                 decode_time += now - last
+                decode_bytes += step_bytes
         st = engine.cache.stats()
         peak_reserved = max(peak_reserved, st["kv_tokens_reserved"])
         peak_live = max(peak_live, st["kv_tokens_live"])
@@ -155,9 +161,7 @@ def run_one(args, shape: str, batch: int, mode: str) -> dict:
         "fragmentation_failures": st["fragmentation_failures"],
     }
     if decode_steps:
-        mean_ctx = sum(lens) / batch + args.new_tokens / 2
-        step_bytes = weight_bytes(cfg) + min(batch, seats) * mean_ctx * kv_bytes_per_token(cfg)
-        gbs = step_bytes / (decode_time / decode_steps) / 1e9
+        gbs = decode_bytes / decode_time / 1e9          # bytes of the steps that were timed, rows as they were
         out["decode_hbm_gbs"] = round(gbs, 1)
         out["decode_hbm_frac"] = round(gbs / HBM_PEAK_GBS, 4)
     return out

@@ -116,6 +116,9 @@ class LlamaConfig:
         if head_dim % 4 != 0:
             raise ConfigError(f"config.json: head_dim {head_dim} is not supported: the attention kernels "
                               f"take head sizes that are multiples of 4 (multiples of 16 run on the matrix cores)")
+        if head_dim > 256:
+            raise ConfigError(f"config.json: head_dim {head_dim} is not supported: no attention kernel here "
+                              f"takes a head size above 256")
         act = d.get("hidden_act", "silu")
         if act != "silu":
             raise ConfigError(f"config.json: hidden_act {act!r} is not supported (only 'silu')")

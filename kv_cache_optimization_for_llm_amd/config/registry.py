@@ -67,6 +67,7 @@ FEED_FORWARDS = Registry("feed-forward")
 NORMS = Registry("norm")
 POSITION_ENCODINGS = Registry("position encoding")
 BLOCKS = Registry("block arrangement")
+ROTARY_FREQUENCIES = Registry("rotary frequency rule")     # name -> f(rot_dim, theta, **params) -> fp32 [rot_dim / 2]
 
 
 def register_architecture(name: str, parse_config, build_spec, *, replace: bool = False) -> Architecture:

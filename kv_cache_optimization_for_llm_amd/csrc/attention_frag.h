@@ -29,6 +29,15 @@ __device__ inline b16x2 pack_bf16(float a, float b) {
     return __builtin_convertvector(f32x2{a, b}, b16x2);
 }
 
+// The values of a lane's four keys (4 bf16 = 8 bytes of a V^T operand), of which only the first
+// `n` hold something this request wrote: the others are set to zero.  A position past a request's
+// newest token belongs to the page but was written by the page's previous owner, or never; its
+// probability is exactly zero, and zero times whatever lies there must stay zero (0 x NaN is not).
+__device__ inline uint2 keep_first_keys(uint2 v, int n) {
+    const uint64_t mask = n >= 4 ? ~0ull : (n <= 0 ? 0ull : ((1ull << (16 * n)) - 1ull));
+    return make_uint2(v.x & (uint32_t)mask, v.y & (uint32_t)(mask >> 32));
+}
+
 // Most key splits the attention kernels and their merge take (the merge keeps one weight per
 // split in LDS).  The host's split policy asks kva_attention_max_splits() for it.
 #define MERGE_MAX_SPLITS 256

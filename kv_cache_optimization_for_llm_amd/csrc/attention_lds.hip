@@ -205,6 +205,18 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, float *__restrict__ part
             for (int t = 0; t < 2; ++t)
                 vf[dt].u2[t] = *reinterpret_cast<const uint2 *>(buf + Geo::KBYTES + (dt * 16 + r) * Geo::VROW + (t * 16 + 4 * g) * 2);
 
+        // Behind the workgroup's last key a block holds whatever the page held before (or the nearest
+        // needed tile, for a redirected one): P is zero there, and the values are made zero too, so
+        // that nothing non-finite left in a page can reach this request.
+        if (MASKED && kstart + 31 > g_hi) {
+            const int n0 = g_hi + 1 - (kstart + 4 * g), n1 = n0 - 16;
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) {
+                vf[dt].u2[0] = keep_first_keys(vf[dt].u2[0], n0);
+                vf[dt].u2[1] = keep_first_keys(vf[dt].u2[1], n1);
+            }
+        }
+
         f32x4 s[RT][2];
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)

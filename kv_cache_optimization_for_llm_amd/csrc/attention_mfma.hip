@@ -306,6 +306,22 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
             l[rt] += quad_rows_sum(lsum);
         }
         // ---- O^T += V^T * P^T
+        // A block that reaches past the item's last key holds, behind it, whatever the page held
+        // before (or the nearest needed tile, for a redirected one): P is zero there, and the
+        // values are made zero too, so that nothing non-finite left in a page can reach this request.
+        if (MASKED && kstart + 31 > item_hi) {
+            const int n0 = item_hi + 1 - (kstart + 4 * g), n1 = n0 - 16;
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) {
+                Frag8 vv;
+                vv.u2[0] = keep_first_keys(f.v[dt].u2[0], n0);
+                vv.u2[1] = keep_first_keys(f.v[dt].u2[1], n1);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+                    o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv.v, pf[rt].v, o[rt][dt], 0, 0, 0);
+            }
+            return;
+        }
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll

@@ -24,6 +24,7 @@
 #define SCAN_IN_FLIGHT 8
 #define SAMPLE_MAX_CHUNKS 1024
 #define PICK_CHUNKS_PER_LANE (SAMPLE_MAX_CHUNKS / KVA_WAVE)
+#define KVA_NO_TOKEN (-1)       // what a row gets whose logits name no token
 
 namespace {
 
@@ -77,11 +78,16 @@ __device__ inline const unsigned char *mask_row(const unsigned char *penalty_mas
     return seat < 0 ? nullptr : penalty_mask + (size_t)seat * vocab;
 }
 
+// exp((l - top) / T); a logit that is -inf or NaN weighs nothing (as in Online::add)
+__device__ inline float token_weight(float l, float top, float inv_t) {
+    return l > -INFINITY ? expf((l - top) * inv_t) : 0.f;
+}
+
 // Running softmax denominator: sum of exp((l - m) * inv_t) over what has been added, m their maximum.
 struct Online {
     float m, s;
     __device__ inline void add(float l, float inv_t) {
-        if (l == -INFINITY) return;          // weighs nothing
+        if (!(l > -INFINITY)) return;        // -inf and NaN weigh nothing
         if (l > m) {
             s = s * expf((m - l) * inv_t) + 1.f;
             m = l;
@@ -203,8 +209,9 @@ sample_pick_kernel(const float *__restrict__ logits, int vocab, int chunk_tokens
     for (int c = c0; c < c1; ++c) b = better(b, Best{rec[c].best_value, rec[c].best_index});
     b = wave_best(b);
     int token = b.index;                    // the greedy choice; the row maximum is b.value
+    bool bad_row = !(b.value > -INFINITY);  // NaN compares false too
     const float inv_t = inv_temperature != nullptr ? inv_temperature[row] : 0.f;
-    if (inv_t > 0.f) {
+    if (inv_t > 0.f && !bad_row) {
         const float top = b.value;
         // chunk sums brought to the row maximum, summed per lane, scanned over the lanes
         float weight[PICK_CHUNKS_PER_LANE];
@@ -217,6 +224,7 @@ sample_pick_kernel(const float *__restrict__ logits, int vocab, int chunk_tokens
         }
         const float upto = wave_prefix_sum(mine);
         const float total = __shfl(upto, KVA_WAVE - 1, KVA_WAVE);
+        bad_row = !(total > 0.f) || total == INFINITY;
         const float target = counter_uniform(seed, rng_key[row], rng_step[row]) * total;
         // the first lane whose chunks reach past the target holds the chunk
         int owner = first_lane(target < upto);
@@ -266,7 +274,7 @@ sample_pick_kernel(const float *__restrict__ logits, int vocab, int chunk_tokens
         const unsigned char *mk = mask_row(penalty_mask, row_seat, row, vocab);
         const float inner = target - before;
         float local = 0.f;
-        for (int t = t0; t < t1; ++t) local += expf((penalised(rl[t], mk, t, penalty) - top) * inv_t);
+        for (int t = t0; t < t1; ++t) local += token_weight(penalised(rl[t], mk, t, penalty), top, inv_t);
         const float reach = wave_prefix_sum(local);
         owner = first_lane(t0 < t1 && inner < reach);
         int found = end - 1;                 // past every span's reach (rounding): the chunk's last token
@@ -274,7 +282,7 @@ sample_pick_kernel(const float *__restrict__ logits, int vocab, int chunk_tokens
             float acc = reach - local;
             found = t1 - 1;
             for (int t = t0; t < t1; ++t) {
-                acc += expf((penalised(rl[t], mk, t, penalty) - top) * inv_t);
+                acc += token_weight(penalised(rl[t], mk, t, penalty), top, inv_t);
                 if (inner < acc) {
                     found = t;
                     break;
@@ -283,10 +291,12 @@ sample_pick_kernel(const float *__restrict__ logits, int vocab, int chunk_tokens
         }
         token = __shfl(found, owner < 0 ? 0 : owner, KVA_WAVE);
     }
-    // A row whose logits are all NaN (or all -inf) has no best token: nothing compares greater than
-    // the start value and the index stays at `vocab`.  Token 0 then: the next step looks its token
-    // up in the embedding table on the device, and a row past the table's end is a memory fault.
-    if (token < 0 || token >= vocab) token = 0;
+    // A row without a finite best logit (all NaN, all -inf) has no token to name, greedy or sampled,
+    // and neither has a temperature row whose weights do not add up to a positive finite total.
+    // Such a row gets KVA_NO_TOKEN (-1): the host sees it and ends the request with an error, and
+    // the next step's lookup of this buffer on the device, which may already be queued, takes
+    // token 0 for any negative value it finds (a row past the table's end would be a memory fault).
+    if (bad_row || token < 0 || token >= vocab) token = KVA_NO_TOKEN;
     if (lane == 0) {
         out_tokens[row] = token;
         if (host_tokens != nullptr) host_tokens[row] = token;      // pinned host memory, mapped for the device

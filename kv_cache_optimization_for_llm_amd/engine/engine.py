@@ -16,6 +16,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager
+from ..cache.manager import page_bytes as cache_page_bytes
 from ..config.model_config import read_config_json
 from ..models.builder import Model, spec_for_config
 from ..ops.library import KernelLibraryError, hip_lib
@@ -126,6 +127,7 @@ class Engine:
         self.vocab_size = self.spec.vocab_size
         max_seq_len = options.max_seq_len or self.spec.max_positions
         max_seq_len = min(max_seq_len, self.spec.max_positions)
+        self.model.limit_positions(max_seq_len)     # per-position tables no longer than the longest request
         if options.max_batch_tokens < 1:
             raise EngineError("max_batch_tokens must be at least 1")
         self.max_batch_tokens = int(options.max_batch_tokens)
@@ -136,9 +138,7 @@ class Engine:
         if options.cache_tokens:
             num_pages = (options.cache_tokens + options.page_size - 1) // options.page_size
         else:
-            elem = torch.empty((), dtype=self.dtype).element_size()
-            page_bytes = sum(2 * len(slots) * kv.num_kv_heads * kv.head_dim * options.page_size * elem
-                             for kv, slots in groups)
+            page_bytes = cache_page_bytes(groups, options.page_size, self.dtype)    # as the mixers' specs say
             if page_bytes == 0:
                 num_pages = 1           # no mixer keeps keys and values
             else:
@@ -191,6 +191,18 @@ class Engine:
         if seat is not None:
             self._seat_of[request_id] = seat
         return seat
+
+    def bind_request(self, request_id, seat: int) -> None:
+        """For a scheduler that takes seats from the cache manager itself: names the request that
+        sits in ``seat``, so that its entries are recognised by :meth:`step_planned`."""
+        if request_id in self._seat_of:
+            raise EngineError(f"request {request_id!r} is live already")
+        self.cache.seat(seat)               # raises unless the seat is taken
+        self._seat_of[request_id] = seat
+
+    def unbind_request(self, request_id) -> None:
+        """The scheduler has given the request's seat back itself."""
+        self._seat_of.pop(request_id, None)
 
     def release(self, request_id) -> None:
         """The request is finished: its pages, reservation and seat are given back."""

@@ -1,13 +1,24 @@
 """Scheduler + step function + sampler in one loop; the Python entry point ``LLM.generate``."""
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, replace
 from typing import Dict, Iterable, List, Optional, Sequence
 
 from ..sampling.sampler import SampleRow, Sampler
 from .batch import StepEntry
 from .engine import Engine, EngineOptions
 from .scheduler import Event, Request, Scheduler, StepPlan, UnresolvedTokens
+
+
+# A request may ask for up to this many sequences (reference: base/src/config.h:97); the random
+# stream of sequence i of request r is keyed r * MAX_PARALLEL_SEQUENCES + i (base/src/engine.cu:892-907).
+MAX_PARALLEL_SEQUENCES = 8
+
+
+def engine_key(request: Request):
+    """The name a scheduled sequence goes by in the engine (a preempted request that re-enters is
+    the same sequence again: same id, index and arrival)."""
+    return ("sched", request.id, request.seq_index, request.arrival)
 
 
 @dataclass
@@ -46,17 +57,19 @@ class Runner:
 
     # the scheduler owns seats; the engine only needs to know which request sits where
     def _on_admit(self, seq) -> None:
-        self.engine._seat_of[("sched", seq.request.id, seq.request.seq_index, seq.request.arrival)] = seq.seat
+        self.engine.bind_request(engine_key(seq.request), seq.seat)
         emitted = seq.prompt[len(seq.prompt) - seq.request.resumed_tokens:] if seq.request.resumed_tokens else ()
         self.sampler.reset_seat(seq.seat, emitted)
 
     def _on_release(self, seq) -> None:
-        self.engine._seat_of.pop(("sched", seq.request.id, seq.request.seq_index, seq.request.arrival), None)
+        self.engine.unbind_request(engine_key(seq.request))
 
     def submit(self, tokens: Sequence[int], max_new_tokens: int, *, request_id: Optional[int] = None,
                n_seqs: int = 1, temperature: Optional[float] = None) -> int:
         """Queues ``n_seqs`` copies of a request (reference wire format:
         ``<id> <max_tokens> <n_seqs> <tok> ...``, ``base/src/request_queue.cpp:11-61``)."""
+        if not 1 <= n_seqs <= MAX_PARALLEL_SEQUENCES:
+            raise ValueError(f"n_seqs {n_seqs} is not in 1..{MAX_PARALLEL_SEQUENCES}")
         if request_id is None:
             request_id = self._next_id
         self._next_id = max(self._next_id, request_id + 1)
@@ -69,16 +82,30 @@ class Runner:
     def idle(self) -> bool:
         return self.scheduler.idle() and self._in_flight is None
 
+    def cancel(self, request_id: int) -> List[Event]:
+        """Ends a request now, whatever it was doing: the tokens of the step in flight are taken
+        first (they are returned as events, before the ``done`` events with reason ``cancelled``),
+        then its sequences leave the queue or give back their seats and pages."""
+        events = self._resolve_in_flight()
+        events.extend(self.scheduler.cancel(request_id))
+        return events
+
+    def live_requests(self) -> List[int]:
+        """Ids of the requests that are waiting or hold a seat."""
+        sched = self.scheduler
+        ids = [r.id for r in sched.waiting] + [s.request.id for s in sched.running + sched.closing]
+        return sorted(set(ids))
+
     def _launch(self, plan: StepPlan):
         """Queues the forward pass and the sampling of a planned step; nothing is waited for."""
         entries, rows = [], []
         for e in plan.entries:
-            rid = ("sched", e.seq.request.id, e.seq.request.seq_index, e.seq.request.arrival)
+            rid = engine_key(e.seq.request)
             entries.append(StepEntry(rid, e.tokens, [len(e.tokens) - 1] if e.sample else []))
             if e.sample:
                 req = e.seq.request
                 emitted_before = req.resumed_tokens + len(e.seq.generated)
-                rows.append(SampleRow(e.seq.seat, req.temperature, req.id * 8 + req.seq_index,
+                rows.append(SampleRow(e.seq.seat, req.temperature, req.id * MAX_PARALLEL_SEQUENCES + req.seq_index,
                                       e.start + len(e.tokens), apply_penalty=emitted_before > 0))
         logits = self.engine.step_planned(entries, [e.seq.seat for e in plan.entries],
                                           [e.start for e in plan.entries])
@@ -126,7 +153,12 @@ class LLM:
 
     def __init__(self, model_dir: str, engine_options: Optional[EngineOptions] = None,
                  serve_options: Optional[ServeOptions] = None):
-        self.engine = Engine(model_dir, engine_options)
+        options = engine_options or EngineOptions()
+        if options.max_logit_rows is None:
+            # generation samples one token per request and step: logits for that many rows, not for
+            # every token a step may bring (at a vocabulary of 128,256 that is 4 GB of a step's memory)
+            options = replace(options, max_logit_rows=max(1, options.max_seqs))
+        self.engine = Engine(model_dir, options)
         self.serve_options = serve_options or ServeOptions()
 
     def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: int = 16, *,

@@ -7,7 +7,9 @@ Each call to :meth:`Scheduler.plan` makes one step's batch under a token budget:
    part-way through their prompt, then new admissions; a prompt may be cut at any token and a
    single request's portion is capped by ``chunk_size``;
 3. a request finishes on an end-of-sequence token (not emitted, not counted), when its budget
-   of new tokens is used up, or when it reaches the longest sequence the cache can hold.
+   of new tokens is used up, when it reaches the longest sequence the cache can hold, or - with
+   the error ``invalid_logits`` - when the sampler reports that its logits named no token
+   (a negative token id: no logit of the row was finite).
 
 The reference has no chunked prefill (its prefill attention cannot read the cache,
 ``base/src/engine.cu:730-737``); what it does have is kept: FCFS queue with preempted requests
@@ -167,6 +169,28 @@ class Scheduler:
 
     def idle(self) -> bool:
         return not self.waiting and not self.running and not self.closing
+
+    def cancel(self, request_id: int) -> List[Event]:
+        """Drops every sequence of a request, wherever it is: waiting ones leave the queue, seated
+        ones give back their seat and pages at once.  Each ends with reason ``cancelled`` and the
+        number of tokens it had emitted.  Tokens of a booked step that are still to be resolved
+        are dropped when they arrive.  The caller resolves the step in flight first if it wants
+        the tokens that step produced."""
+        events: List[Event] = []
+        kept: Deque[Request] = deque()
+        for r in self.waiting:
+            if r.id != request_id:
+                kept.append(r)
+                continue
+            events.append(Event("done", r.id, r.seq_index, tokens=r.resumed_tokens, reason="cancelled"))
+            if r.preempted:
+                self._preempted_gone()
+        self.waiting = kept
+        for seq in [s for s in self.running + self.closing if s.request.id == request_id]:
+            del seq.generated[len(seq.generated) - seq.unresolved:]      # placeholders of tokens never seen
+            seq.unresolved = 0
+            self._finish(seq, "cancelled", events)
+        return events
 
     # ------------------------------------------------------------------ helpers
     def _release(self, seq: Sequence_) -> None:
@@ -414,6 +438,13 @@ class Scheduler:
                 continue            # ended by an earlier token while this step was in flight
             tok = int(tok)
             seq.unresolved -= 1
+            if tok < 0:
+                # the sampler found no token in this row's logits (none of them finite): the request
+                # ends with an error instead of going on from a token nobody chose
+                del seq.generated[idx:]
+                seq.unresolved = 0
+                self._finish(seq, "invalid_logits", events)
+                continue
             if tok in self.eos and not self.ignore_eos:
                 del seq.generated[idx:]
                 seq.unresolved = 0

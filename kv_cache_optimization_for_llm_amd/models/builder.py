@@ -129,6 +129,16 @@ class Model:
                 parts.append(pos)
         return all(getattr(p, "graph_safe", False) for p in parts)
 
+    def limit_positions(self, positions: int) -> None:
+        """Tells every part that keeps something per position (tables of a position encoding) that
+        no position at or past ``positions`` will be asked for."""
+        for b in self.blocks:
+            for part in (*b.parts(), getattr(b.mixer, "position", None)):
+                limit = getattr(part, "limit_positions", None)
+                if limit is not None:
+                    limit(positions)
+                    part.tables(self.device)        # made now: they count when the cache pool is sized from what is left
+
     # ---- weights
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         return model_tensor_specs(self.spec, self.blocks, self.final_norm)
@@ -215,8 +225,8 @@ class Model:
             ctx = MixerContext(batch=batch)
             group = cache.group_of(slot)
             if group is not None:
-                _, k, v = cache.kv_arrays(slot)
-                ctx.kv = KVView(k, v, group.table_dev, batch.slot_mapping[group.index],
+                _, arrays = cache.kv_arrays(slot)
+                ctx.kv = KVView(arrays, group.table_dev, batch.slot_mapping[group.index],
                                 group.page_size, writes=call.writes_cache)
             if slot in cache.state:
                 ctx.state = cache.state[slot]

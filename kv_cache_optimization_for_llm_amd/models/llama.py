@@ -16,9 +16,12 @@ from .spec import LayerSpec, ModelSpec, PartSpec, default_order
 
 
 def llama_spec(cfg: LlamaConfig) -> ModelSpec:
-    scaling = asdict(cfg.rope_scaling) if cfg.rope_scaling is not None else None
+    rule, params = "plain", None
+    if cfg.rope_scaling is not None:
+        params = asdict(cfg.rope_scaling)
+        rule = params.pop("rope_type")
     position = PartSpec("rotary", dict(head_dim=cfg.head_dim, max_positions=cfg.max_position_embeddings,
-                                       theta=cfg.rope_theta, scaling=scaling))
+                                       theta=cfg.rope_theta, frequencies=rule, frequency_params=params))
     layers = []
     for i in range(cfg.num_hidden_layers):
         p = f"model.layers.{i}."

@@ -18,7 +18,7 @@ from ..config.registry import MIXERS, POSITION_ENCODINGS
 from ..models.spec import PartSpec, TensorSpec
 from ..ops import attention as attn_ops
 from ..ops import kernels as K
-from .base import BranchTail, KVCacheSpec, Mixer, MixerContext, NormedRows
+from .base import BranchTail, KVCacheSpec, Mixer, MixerContext, NormedRows, attention_cache_spec
 from .linear import Linear
 
 
@@ -100,8 +100,8 @@ class GQAAttention(Mixer):
         self.o = Linear(tensors[p + "o_proj.weight"])
 
     def kv_cache_spec(self) -> KVCacheSpec:
-        return KVCacheSpec(self.num_kv_heads, self.head_dim,
-                           kind="window" if self.window > 0 else "full", window=self.window)
+        return attention_cache_spec(self.num_kv_heads, self.head_dim,
+                                    kind="window" if self.window > 0 else "full", window=self.window)
 
     fuses_tail = True
 

@@ -6,7 +6,7 @@ checkpoint and how to run on a batch.  It never knows which model it is in.
 * :class:`Norm`             ``forward(x, out=None, delta=None, row_idx=None)``
 * :class:`PositionEncoding` ``apply_and_cache(qkv, positions, geometry, kv)``
 * :class:`Mixer`            ``forward(x, ctx)`` with a :class:`MixerContext`; declares the cache it
-  needs (:class:`KVCacheSpec`: all keys or a window of them) and/or a fixed-size per-request
+  needs (:class:`KVCacheSpec`: named arrays per token, all positions or a window of them) and/or a fixed-size per-request
   state (:class:`StateSpec`)
 * :class:`FeedForward`      ``forward(x, ctx)``
 * :class:`Block`            ``forward(hidden, delta, ctx, next_norm=None)`` -> ``(hidden, delta)``:
@@ -31,15 +31,70 @@ from ..models.spec import TensorSpec
 
 
 @dataclass(frozen=True)
-class KVCacheSpec:
-    """Paged key/value storage one mixer call needs, per token: ``num_kv_heads * head_dim`` keys
-    and as many values.  ``kind`` is ``"full"`` (every position stays) or ``"window"`` (only the
-    last ``window`` positions are ever read, pages behind them are given back)."""
+class CacheArray:
+    """One array of a paged cache entry: what a mixer call keeps per token under ``name``.
 
-    num_kv_heads: int
-    head_dim: int
+    ``token_shape`` is the shape of one token's entry; ``token_axis`` says where the page's token
+    axis lies inside a page: a page of the array has ``token_shape`` with ``page_size`` inserted at
+    that index, and the whole array is ``[pages, *page_shape]``.  Keys of attention heads
+    ``(kv_heads, head_dim)`` with ``token_axis=1`` give pages ``[kv_heads, page_size, head_dim]``;
+    values with ``token_axis=2`` give the transposed ``[kv_heads, head_dim, page_size]``; one
+    latent vector ``(width,)`` with ``token_axis=0`` gives ``[page_size, width]``.  ``dtype``
+    ``None`` is the engine's storage type."""
+
+    name: str
+    token_shape: Tuple[int, ...]
+    token_axis: int = 0
+    dtype: Optional[torch.dtype] = None
+
+    def __post_init__(self):
+        if not self.token_shape or any(int(n) <= 0 for n in self.token_shape):
+            raise ValueError(f"cache array {self.name!r}: token shape {self.token_shape} must be positive")
+        if not 0 <= self.token_axis <= len(self.token_shape):
+            raise ValueError(f"cache array {self.name!r}: token axis {self.token_axis} lies outside its page")
+
+    def page_shape(self, page_size: int) -> Tuple[int, ...]:
+        shape = list(self.token_shape)
+        shape.insert(self.token_axis, int(page_size))
+        return tuple(shape)
+
+    def elements_per_token(self) -> int:
+        n = 1
+        for d in self.token_shape:
+            n *= int(d)
+        return n
+
+
+@dataclass(frozen=True)
+class KVCacheSpec:
+    """Paged storage one mixer call needs: the arrays it keeps per token (names, per-token
+    shapes, layout inside a page) and which positions stay.  ``kind`` is ``"full"`` (every
+    position stays) or ``"window"`` (only the last ``window`` positions are ever read, pages
+    behind them are given back).  The cache manager allocates from this description and the
+    engine sizes the pool from it; neither knows what the arrays mean."""
+
+    arrays: Tuple[CacheArray, ...]
     kind: str = "full"
     window: int = 0
+
+    def __post_init__(self):
+        names = [a.name for a in self.arrays]
+        if not names or len(set(names)) != len(names):
+            raise ValueError(f"a cache entry needs arrays with distinct names, got {names}")
+        if self.kind not in ("full", "window"):
+            raise ValueError(f"cache kind {self.kind!r} is not one of 'full', 'window'")
+
+    def bytes_per_token(self, default_dtype: torch.dtype) -> int:
+        return sum(a.elements_per_token() * torch.empty((), dtype=a.dtype or default_dtype).element_size()
+                   for a in self.arrays)
+
+
+def attention_cache_spec(num_kv_heads: int, head_dim: int, kind: str = "full", window: int = 0) -> KVCacheSpec:
+    """Keys and values of ``num_kv_heads`` heads of ``head_dim``, as the attention kernels here
+    read them: K pages ``[kv_heads, page_size, head_dim]``, V pages transposed
+    ``[kv_heads, head_dim, page_size]``."""
+    heads = (int(num_kv_heads), int(head_dim))
+    return KVCacheSpec((CacheArray("k", heads, token_axis=1), CacheArray("v", heads, token_axis=2)), kind, window)
 
 
 @dataclass(frozen=True)
@@ -52,17 +107,24 @@ class StateSpec:
 
 @dataclass
 class KVView:
-    """What a mixer call sees of the paged cache: its own K array
-    ``[pages, kv_heads, page_size, head_dim]`` and V array (transposed inside a page)
-    ``[pages, kv_heads, head_dim, page_size]``, the block table ``[seats, max_blocks]`` of its
-    group, and for each token of the step the slot (page * page_size + row) to write to."""
+    """What a mixer call sees of the paged cache: its own arrays by name (each
+    ``[pages, *page_shape]`` as its :class:`CacheArray` says), the block table
+    ``[seats, max_blocks]`` of its group, and for each token of the step the slot
+    (page * page_size + row) to write to."""
 
-    k_cache: torch.Tensor
-    v_cache: torch.Tensor
+    arrays: Dict[str, torch.Tensor]
     block_table: torch.Tensor
     slot_mapping: torch.Tensor
     page_size: int
     writes: bool = True
+
+    @property
+    def k_cache(self) -> torch.Tensor:      # the two arrays of attention_cache_spec
+        return self.arrays["k"]
+
+    @property
+    def v_cache(self) -> torch.Tensor:
+        return self.arrays["v"]
 
 
 @dataclass

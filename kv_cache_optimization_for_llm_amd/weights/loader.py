@@ -48,6 +48,8 @@ def _weight_files(model_dir: str) -> List[str]:
 
 def _read_header(path: str) -> Dict[str, dict]:
     """The JSON header of a safetensors file: 8-byte little-endian length, then JSON."""
+    if not os.path.isfile(path):
+        raise WeightError(f"{path}: named by model.safetensors.index.json but not in the model folder")
     size = os.path.getsize(path)
     with open(path, "rb") as f:
         raw = f.read(8)

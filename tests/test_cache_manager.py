@@ -7,10 +7,10 @@ import pytest
 from kv_cache_optimization_for_llm_amd.cache.allocators import (BuddyAllocator, CacheAccountingError,
                                                                 PagePool)
 from kv_cache_optimization_for_llm_amd.cache.manager import CacheManager
-from kv_cache_optimization_for_llm_amd.parts.base import KVCacheSpec, StateSpec
+from kv_cache_optimization_for_llm_amd.parts.base import StateSpec, attention_cache_spec
 
-FULL = KVCacheSpec(2, 16)
-WIN = KVCacheSpec(1, 32, kind="window", window=40)
+FULL = attention_cache_spec(2, 16)
+WIN = attention_cache_spec(1, 32, kind="window", window=40)
 
 
 def test_pool_is_lifo_and_counts_references():
@@ -208,7 +208,7 @@ def test_random_orders_keep_the_books(mode, seed):
 def test_a_sequence_cannot_grow_past_the_longest_length_inside_its_last_page():
     """The longest sequence need not be a multiple of the page size: the last page then has rows
     that must never be used, also on the quick path that skips the books when a page is there."""
-    m = CacheManager([(KVCacheSpec(2, 16), [0])], {}, page_size=16, num_pages=8, max_seqs=2, max_seq_len=53)
+    m = CacheManager([(attention_cache_spec(2, 16), [0])], {}, page_size=16, num_pages=8, max_seqs=2, max_seq_len=53)
     seat = m.admit("r")
     assert m.grow(seat, 50) and m.capacity_tokens(seat) == 53
     m.commit(seat, 50)

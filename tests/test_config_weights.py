@@ -37,6 +37,7 @@ def test_config_defaults_follow_the_keys():
     ({"num_key_value_heads": 3}, "multiple"),
     ({"head_dim": 15}, "even"),
     ({"head_dim": 18}, "multiples of 4"),
+    ({"head_dim": 260}, "above 256"),
     ({"hidden_act": "gelu"}, "hidden_act"),
     ({"attention_bias": True}, "attention_bias"),
     ({"mlp_bias": True}, "mlp_bias"),
@@ -77,6 +78,11 @@ def test_spec_is_data_layer_by_layer():
     m = spec.layers[1].mixer
     assert m.kind == "gqa_attention" and m.params["num_kv_heads"] == 1 and m.params["head_dim"] == 24
     assert m.params["position"].kind == "rotary" and m.params["position"].params["theta"] == 500000.0
+    # the frequency rule is a named parameter of the part, its constants beside it
+    assert m.params["position"].params["frequencies"] == "llama3"
+    assert m.params["position"].params["frequency_params"] == dict(
+        factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=64)
+    assert spec_for_config(TINY_A)[1].layers[0].mixer.params["position"].params["frequencies"] == "plain"
     assert spec.layers[2].feed_forward.params["intermediate_size"] == 256
     assert spec.head_name == "lm_head.weight"
     assert spec_for_config(TINY_A)[1].head_name is None
@@ -135,6 +141,46 @@ def test_tied_model_may_carry_an_unused_head(tmp_path):
     save_file(w, path)
     _, spec = spec_for_config(TINY_A)
     validate(checkpoint_index(d), tensor_specs_for_config(TINY_A), spec.ignorable_tensors)
+
+
+def test_a_checkpoint_in_shards_is_read_through_its_index(tmp_path):
+    """Larger checkpoints come as several files and ``model.safetensors.index.json`` naming, per
+    tensor, the file that holds it (the reference reads the one-file form only,
+    ``base/src/model.cu:15-84``): the same tensors come out of the shards as out of one file, a
+    tensor that no shard holds is reported by name, and so is a shard the index names that is
+    not there."""
+    from safetensors.torch import load_file, save_file
+    from kv_cache_optimization_for_llm_amd.weights.loader import load_tensors
+    whole = write_random_model(str(tmp_path / "whole"), TINY_B, seed=9)
+    w = load_file(os.path.join(whole, "model.safetensors"))
+    names = sorted(w)
+    shards = {"model-00001-of-00002.safetensors": names[: len(names) // 3],
+              "model-00002-of-00002.safetensors": names[len(names) // 3:]}
+    d = tmp_path / "sharded"
+    d.mkdir()
+    (d / "config.json").write_text(json.dumps(TINY_B))
+    for fname, part in shards.items():
+        save_file({n: w[n] for n in part}, str(d / fname))
+    index = {"metadata": {"total_size": 0}, "weight_map": {n: f for f, part in shards.items() for n in part}}
+    (d / "model.safetensors.index.json").write_text(json.dumps(index))
+    specs = tensor_specs_for_config(TINY_B)
+    got = load_tensors(str(d), specs, torch.bfloat16, "cpu")
+    want = load_tensors(whole, specs, torch.bfloat16, "cpu")
+    assert sorted(got) == sorted(want) == sorted(specs)
+    assert all(torch.equal(got[n], want[n]) and got[n].dtype == want[n].dtype for n in want)
+    assert {os.path.basename(f) for f, _ in checkpoint_index(str(d)).values()} == set(shards)
+    # a tensor that is in no shard
+    lost = names[-1]
+    save_file({n: w[n] for n in shards["model-00002-of-00002.safetensors"] if n != lost},
+              str(d / "model-00002-of-00002.safetensors"))
+    with pytest.raises(WeightError) as e:
+        load_tensors(str(d), specs, torch.bfloat16, "cpu")
+    assert "missing tensors (1)" in str(e.value) and lost in str(e.value)
+    # a shard that the index names and the folder does not hold
+    os.remove(d / "model-00001-of-00002.safetensors")
+    with pytest.raises(WeightError) as e:
+        checkpoint_index(str(d))
+    assert "model-00001-of-00002.safetensors" in str(e.value)
 
 
 def test_broken_files_are_refused(tmp_path):

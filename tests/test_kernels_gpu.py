@@ -36,26 +36,32 @@ def test_embed_gather(dtype, table_dtype, gpu):
     assert torch.equal(out.cpu(), want)
 
 
-def test_logits_without_a_best_token_still_name_a_token_of_the_table(gpu):
-    """A row of logits that are all NaN or all -inf has no best token.  The sampler names token 0
-    for it (greedy and sampled rows alike stay inside the vocabulary), and a lookup of whatever a
-    kernel left in the feedback buffer stays inside the table: the token of such a row is looked
-    up on the device by the next step, where a row past the table's end is a memory fault, not an
-    error message."""
+def test_logits_without_a_finite_value_are_reported_and_lookups_stay_inside_the_table(gpu):
+    """A row of logits that are all NaN or all -inf names no token.  The sampler says so with -1,
+    greedy and sampled rows alike (the host ends the request with an error), and a lookup of
+    whatever a kernel left in the feedback buffer stays inside the table: the token of such a row
+    is looked up on the device by the next step, which may be queued before the host has seen
+    the -1, and a row past the table's end is a memory fault, not an error message."""
     vocab = 333
-    lg = torch.randn(4, vocab)
+    lg = torch.randn(5, vocab)
     lg[0] = float("nan")
     lg[1] = float("-inf")
     lg[3] = float("nan")
+    lg[4, 7:] = float("nan")                               # some finite logits: a token can be named
     lg = lg.to(gpu)
-    out = torch.full((4,), -7, dtype=torch.int32, device=gpu)
+    out = torch.full((5,), -7, dtype=torch.int32, device=gpu)
     K.sample(lg, out, chunks=4)
-    assert out.cpu().tolist() == [0, 0, int(lg[2].argmax()), 0]
-    inv_t = torch.tensor([1.0, 1.25, 0.0, 2.0], device=gpu)
-    zeros = torch.zeros(4, dtype=torch.int32, device=gpu)
-    K.sample(lg, out, chunks=4, inv_temperature=inv_t, seed=5, rng_key=zeros, rng_step=zeros)
+    assert out.cpu().tolist() == [-1, -1, int(lg[2].argmax()), -1, int(lg[4, :7].argmax())]
+    inv_t = torch.tensor([1.0, 1.25, 0.0, 2.0, 1.0], device=gpu)
+    zeros = torch.zeros(5, dtype=torch.int32, device=gpu)
+    host = torch.full((5,), -7, dtype=torch.int32).pin_memory()
+    K.sample(lg, out, chunks=4, inv_temperature=inv_t, seed=5, rng_key=zeros, rng_step=zeros, host_tokens=host)
+    torch.cuda.synchronize()
     got = out.cpu().tolist()
-    assert all(0 <= t < vocab for t in got) and got[2] == int(lg[2].argmax())
+    assert got[:4] == [-1, -1, int(lg[2].argmax()), -1] and 0 <= got[4] < 7 and host.tolist() == got
+    # more chunks than the vocabulary fills (the last ones are empty): the same answers
+    K.sample(lg, out, chunks=128, inv_temperature=inv_t, seed=5, rng_key=zeros, rng_step=zeros)
+    assert out.cpu().tolist()[:4] == got[:4]
     table = rnd(vocab, 64, dtype=torch.bfloat16)
     feedback = torch.tensor([vocab, -9, 1 << 30, 5], dtype=torch.int32)
     ids = torch.tensor([-1, -2, -3, -4], dtype=torch.int32)
@@ -216,8 +222,10 @@ def test_rope_and_cache_write(dtype, nq, nkv, d, rot, page, gpu):
             assert kc[s // page, :, s % page, :].abs().max() == 0 and vc[s // page, :, :, s % page].abs().max() == 0
 
 
-def attention_case(dtype, nq, nkv, d, page, window, entries, seed, gpu):
-    """entries: [(start_pos, q_len)].  Builds a cache with random pages, runs both kernels."""
+def attention_case(dtype, nq, nkv, d, page, window, entries, seed, gpu, stale=0.0):
+    """entries: [(start_pos, q_len)].  Builds a cache with random pages, runs both kernels.
+    ``stale``: what every position holds that no entry has written (the rest of a request's last
+    page, pages nobody owns)."""
     dt = DT[dtype]
     g = torch.Generator().manual_seed(seed)
     E = len(entries)
@@ -226,8 +234,11 @@ def attention_case(dtype, nq, nkv, d, page, window, entries, seed, gpu):
     perm = torch.randperm(n_pages, generator=g)
     table = torch.full((E + 2, max_blocks), -1, dtype=torch.int32)
     seats = [E + 1 - i for i in range(E)]                    # seats differ from entry numbers
-    kc = torch.zeros(n_pages, nkv, page, d)
-    vc = torch.zeros(n_pages, nkv, d, page)
+    kc = torch.full((n_pages, nkv, page, d), stale)
+    vc = torch.full((n_pages, nkv, d, page), stale)
+    if stale != 0.0:
+        vc[..., 1::2] = float("inf")        # NaN and infinities side by side
+        kc[:, :, 1::2, :] = float("-inf")
     keys, vals, qs = [], [], []
     used = 0
     for e, (s, n) in enumerate(entries):
@@ -340,6 +351,47 @@ def test_attention_mfma(nq, nkv, d, page, window, splits, wide, pair, gpu):
             assert torch.equal(out3[rows], out[rows])
         else:
             assert (out3[rows] == 7.0).all()
+
+
+@pytest.mark.parametrize("nq, nkv, d, page, window", [(4, 2, 16, 16, 0), (32, 8, 64, 16, 0), (8, 2, 64, 16, 45),
+                                                      (6, 2, 48, 8, 0), (4, 4, 96, 32, 33), (24, 8, 128, 16, 0)])
+def test_attention_never_sees_what_a_page_held_before(nq, nkv, d, page, window, gpu):
+    """A page handed to a request still holds its previous owner's keys and values behind the
+    request's newest token, and pages it does not own hold anything at all: here NaN and
+    infinities.  Those positions have probability zero, and zero times a non-finite value must not
+    reach the output (the matrix-core kernels multiply whole 32-key blocks, masked keys included)."""
+    dev, want, T, stride, scale, lens = attention_case("bfloat16", nq, nkv, d, page, window, ENTRIES, 13, gpu,
+                                                       stale=float("nan"))
+    assert not torch.isfinite(dev["kc"].float()).all() and not torch.isfinite(dev["vc"].float()).all()
+    out = torch.full((T, nq * d), float("nan"), dtype=torch.bfloat16, device=gpu)
+    K.attention_rowwise(dev["qkv"], stride, out, dev["kc"], dev["vc"], dev["table"], dev["tok_seat"],
+                        dev["tok_pos"], nq, nkv, d, scale, window)
+    close(out, want, torch.bfloat16, "attention_rowwise over stale pages", tol16=8e-3)
+    for splits, wide, pair in ((1, False, False), (3, False, False), (1, True, True), (2, True, False)):
+        tiles = K.attention_mfma_row_tiles(d, wide)
+        ent, row0 = items_for(lens, nq // nkv, gpu, tiles)
+        per = ((max(s + n for s, n in ENTRIES) + splits - 1) // splits + 31) // 32 * 32 if splits > 1 else 0
+        out = torch.full((T, nq * d), float("nan"), dtype=torch.bfloat16, device=gpu)
+        K.attention_mfma(dev["qkv"], stride, out, dev["kc"], dev["vc"], dev["table"], ent, row0,
+                         dev["entry_seat"], dev["q_start"], dev["start_pos"], nq, nkv, d, scale, window,
+                         splits, per, tiles, pair)
+        assert torch.isfinite(out.float()).all(), f"splits={splits} tiles={tiles}: a stale value reached the output"
+        close(out, want, torch.bfloat16, f"attention_mfma over stale pages splits={splits} tiles={tiles}", tol16=8e-3)
+    if K.attention_lds_supported(d, page):
+        dev, want, T, stride, scale, lens = attention_case("bfloat16", nq, nkv, d, page, window, LONG_ENTRIES, 17, gpu,
+                                                           stale=float("nan"))
+        group = nq // nkv
+        qs, sp, seat = dev["q_start"].cpu(), dev["start_pos"].cpu(), dev["entry_seat"].cpu()
+        rows = [(int(qs[e]), n, int(sp[e]), int(seat[e]), r0, 0, 0, 0)
+                for e, n in enumerate(lens) for r0 in range(0, n * group, 128)]
+        meta = torch.tensor(rows, dtype=torch.int32, device=gpu)
+        for splits in (1, 3):
+            per = ((max(s + n for s, n in LONG_ENTRIES) + splits - 1) // splits + 31) // 32 * 32 if splits > 1 else 0
+            out = torch.full((T, nq * d), float("nan"), dtype=torch.bfloat16, device=gpu)
+            K.attention_lds(dev["qkv"], stride, out, dev["kc"], dev["vc"], dev["table"], meta, nq, nkv, d, scale,
+                            window, False, splits, per)
+            assert torch.isfinite(out.float()).all(), f"workgroup kernel, splits={splits}: a stale value reached the output"
+            close(out, want, torch.bfloat16, f"attention_lds over stale pages splits={splits}", tol16=8e-3)
 
 
 LONG_ENTRIES = [(0, 300), (40, 1), (200, 131), (5, 64), (0, 33)]

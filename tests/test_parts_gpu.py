@@ -11,7 +11,7 @@ from kv_cache_optimization_for_llm_amd.cache.manager import CacheManager
 from kv_cache_optimization_for_llm_amd.engine.batch import build_batch
 from kv_cache_optimization_for_llm_amd.models.spec import PartSpec
 from kv_cache_optimization_for_llm_amd.parts.attention import GQAAttention
-from kv_cache_optimization_for_llm_amd.parts.base import KVCacheSpec, KVView, MixerContext
+from kv_cache_optimization_for_llm_amd.parts.base import KVView, MixerContext, attention_cache_spec
 from kv_cache_optimization_for_llm_amd.parts.block import PreNormBlock
 from kv_cache_optimization_for_llm_amd.parts.linear import Linear
 from kv_cache_optimization_for_llm_amd.parts.mlp import SwiGLU
@@ -23,6 +23,7 @@ DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 TOL = {"float32": 1e-5, "bfloat16": 1.5e-2}
 SCALING = dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
                original_max_position_embeddings=32)
+LLAMA3 = dict(frequencies="llama3", frequency_params={k: v for k, v in SCALING.items() if k != "rope_type"})
 
 
 def rnd(*shape, scale=1.0, seed=0, dtype=torch.float32):
@@ -62,7 +63,8 @@ def test_rmsnorm_part(dtype, gpu):
 def test_rotary_frequencies_and_tables_match_the_plain_formulas(gpu):
     for d, theta, sc in ((16, 10000.0, None), (48, 500000.0, SCALING), (64, 500000.0, dict(SCALING, factor=32.0))):
         assert np.array_equal(rotary_inv_freq(d, theta, sc), plain.rope_inv_freq(d, theta, sc))
-        enc = RotaryEncoding(head_dim=d, max_positions=300, theta=theta, scaling=sc)
+        rule = dict(frequencies="llama3", frequency_params={k: v for k, v in sc.items() if k != "rope_type"}) if sc else {}
+        enc = RotaryEncoding(head_dim=d, max_positions=300, theta=theta, **rule)
         cos, sin = enc.tables(gpu)
         pc, ps = plain.rope_cos_sin(range(300), plain.rope_inv_freq(d, theta, sc))
         assert np.array_equal(cos.cpu().numpy(), pc) and np.array_equal(sin.cpu().numpy(), ps)
@@ -70,10 +72,26 @@ def test_rotary_frequencies_and_tables_match_the_plain_formulas(gpu):
     assert part.tables(gpu)[0].shape == (64, 8)
     with pytest.raises(ValueError):
         RotaryEncoding(head_dim=32, max_positions=64, theta=10000.0, rotary_dim=40)
+    # the frequency rule is chosen by name: an unknown one is refused by name, another one is
+    # registered from outside and used without a change to the part
+    from kv_cache_optimization_for_llm_amd.config.registry import ROTARY_FREQUENCIES, RegistryError
+    with pytest.raises(RegistryError) as e:
+        RotaryEncoding(head_dim=32, max_positions=64, theta=10000.0, frequencies="yarn")
+    assert "yarn" in str(e.value) and "llama3" in str(e.value)
+    ROTARY_FREQUENCIES.register("toy_halved", lambda rot, theta, by: rotary_inv_freq(rot, theta, None) / np.float32(by))
+    try:
+        toy = RotaryEncoding(head_dim=16, max_positions=40, theta=10000.0, frequencies="toy_halved",
+                             frequency_params=dict(by=2.0))
+        pc, _ = plain.rope_cos_sin(range(40), plain.rope_inv_freq(16, 10000.0, None) / np.float32(2.0))
+        assert np.array_equal(toy.tables(gpu)[0].cpu().numpy(), pc)
+        toy.limit_positions(24)                      # an engine whose longest request is shorter
+        assert toy.tables(gpu)[0].shape == (24, 8) and np.array_equal(toy.tables(gpu)[0].cpu().numpy(), pc[:24])
+    finally:
+        ROTARY_FREQUENCIES.unregister("toy_halved")
 
 
 def one_request_context(nkv, d, page, T, start, dtype, gpu, slots=(0,)):
-    cm = CacheManager([(KVCacheSpec(nkv, d), list(slots))], {}, page_size=page, num_pages=40, max_seqs=3,
+    cm = CacheManager([(attention_cache_spec(nkv, d), list(slots))], {}, page_size=page, num_pages=40, max_seqs=3,
                       max_seq_len=512, device=gpu, dtype=DT[dtype])
     cm.admit("other")
     seat = cm.admit("x")
@@ -84,13 +102,13 @@ def run_mixer_in_portions(mixer, cm, seat, x, cuts, gpu):
     """Feeds the rows of x to the mixer in portions; returns the concatenated output."""
     outs, pos = [], 0
     g = cm.groups[0]
-    _, k, v = cm.kv_arrays(0)
+    _, arrays = cm.kv_arrays(0)
     for n in cuts:
         assert cm.grow(seat, pos + n)
         sm = cm.slot_mapping(seat, pos, n, 0)
         cm.flush_tables()
         batch = build_batch([seat], [pos], [np.zeros(n, dtype=np.int32)], [[]], [[sm]], gpu)
-        ctx = MixerContext(batch=batch, kv=KVView(k, v, g.table_dev, batch.slot_mapping[0], g.page_size))
+        ctx = MixerContext(batch=batch, kv=KVView(arrays, g.table_dev, batch.slot_mapping[0], g.page_size))
         outs.append(mixer.forward(x[pos:pos + n].contiguous(), ctx))
         cm.commit(seat, pos + n)
         pos += n
@@ -101,10 +119,10 @@ def run_mixer_in_portions(mixer, cm, seat, x, cuts, gpu):
 @pytest.mark.parametrize("nq, nkv, d, page", [(6, 2, 32, 16), (5, 1, 24, 8), (4, 4, 48, 4)])
 def test_attention_part_whole_and_in_portions(dtype, nq, nkv, d, page, gpu):
     H, T = 56, 75
-    pos = PartSpec("rotary", dict(head_dim=d, max_positions=128, theta=50000.0, scaling=SCALING))
+    pos = PartSpec("rotary", dict(head_dim=d, max_positions=128, theta=50000.0, **LLAMA3))
     part = GQAAttention("a.", hidden_size=H, num_heads=nq, num_kv_heads=nkv, head_dim=d,
                         scale=1 / math.sqrt(d), position=pos)
-    assert part.kv_cache_spec().num_kv_heads == nkv and part.state_spec() is None
+    assert part.kv_cache_spec().arrays[0].token_shape == (nkv, d) and part.state_spec() is None
     specs = part.tensor_specs()
     assert specs["a.q_proj.weight"].shape == (nq * d, H) and specs["a.o_proj.weight"].shape == (H, nq * d)
     W = load(part, {k: rnd(*s.shape, scale=0.2, seed=i) for i, (k, s) in enumerate(specs.items())}, dtype, gpu)
@@ -185,8 +203,8 @@ def test_pre_norm_block_adds_both_branches_to_the_stream(dtype, gpu):
     cm.flush_tables()
     batch = build_batch([seat], [0], [np.zeros(T, dtype=np.int32)], [[]], [[sm]], gpu)
     g = cm.groups[0]
-    _, k, v = cm.kv_arrays(0)
-    ctx = MixerContext(batch=batch, kv=KVView(k, v, g.table_dev, batch.slot_mapping[0], g.page_size))
+    _, arrays = cm.kv_arrays(0)
+    ctx = MixerContext(batch=batch, kv=KVView(arrays, g.table_dev, batch.slot_mapping[0], g.page_size))
     hidden, delta = block.forward(h0.to(gpu).clone(), None, ctx)
     from kv_cache_optimization_for_llm_amd.ops import kernels as K
     K.residual_add(hidden, delta)
@@ -233,8 +251,8 @@ def test_two_blocks_hand_the_stream_on_at_every_row_count(T, gpu):
     hidden, delta = h0.to(gpu).clone(), None
     handed_on = []
     for b, block in enumerate(blocks):
-        _, k, v = cm.kv_arrays(b)
-        ctx = MixerContext(batch=batch, kv=KVView(k, v, g.table_dev, batch.slot_mapping[0], g.page_size))
+        _, arrays = cm.kv_arrays(b)
+        ctx = MixerContext(batch=batch, kv=KVView(arrays, g.table_dev, batch.slot_mapping[0], g.page_size))
         hidden, delta = block.forward(hidden, delta, ctx, blocks[1].first_norm() if b == 0 else None)
         handed_on.append(delta)
     first = handed_on[0]

@@ -3,9 +3,9 @@ import pytest
 
 from kv_cache_optimization_for_llm_amd.cache.manager import CacheManager
 from kv_cache_optimization_for_llm_amd.engine.scheduler import (Request, Scheduler, reservation_tokens)
-from kv_cache_optimization_for_llm_amd.parts.base import KVCacheSpec
+from kv_cache_optimization_for_llm_amd.parts.base import attention_cache_spec
 
-SPEC = KVCacheSpec(2, 16)
+SPEC = attention_cache_spec(2, 16)
 EOS = 7
 
 
@@ -91,6 +91,69 @@ def test_eos_ends_a_request_and_is_not_emitted():
     assert out[(3, 0)] == [fake_token(3, 10), fake_token(3, 11)] and reasons[(3, 0)] == "eos"
     done = [e for e in events if e.kind == "done"][0]
     assert done.tokens == 2
+
+
+def test_a_row_without_a_token_ends_its_request_with_an_error():
+    """The sampler reports a row whose logits named no token (none finite) as a negative id: that
+    request ends with ``invalid_logits``, nothing is emitted for the row, the others go on, and
+    with the loop one step ahead the step already booked for the request is dropped."""
+    for ahead in (False, True):
+        s = Scheduler(cache(), max_batch_tokens=64, ignore_eos=True)
+        s.add(Request(0, list(range(10, 20)), 6))
+        s.add(Request(1, list(range(10, 25)), 6))
+        out, reasons, in_flight = {0: [], 1: []}, {}, None
+        for step in range(40):
+            if s.idle() and in_flight is None:
+                break
+            plan = s.plan()
+            for e in plan.entries:
+                assert s.cache.grow(e.seq.seat, e.start + len(e.tokens))
+            sampled = [-1 if (e.seq.request.id == 0 and e.start + len(e.tokens) == 12) else
+                       fake_token(e.seq.request.id, e.start + len(e.tokens)) for e in plan.entries if e.sample]
+            evs = []
+            if ahead:
+                launched = (s.book(plan), sampled) if plan.entries else None
+                if in_flight:
+                    evs = s.resolve(*in_flight)
+                in_flight = launched
+            else:
+                evs = s.complete(plan, sampled)
+            for ev in evs + plan.events:
+                if ev.kind == "token":
+                    out[ev.request_id].append(ev.token)
+                elif ev.kind == "done":
+                    reasons[ev.request_id] = (ev.reason, ev.tokens)
+            s.cache.check()
+        assert reasons == {0: ("invalid_logits", 2), 1: ("length", 6)}
+        assert out[0] == [fake_token(0, 10), fake_token(0, 11)] and len(out[1]) == 6
+        assert s.idle() and s.cache.free_seats == 8 and s.cache.groups[0].free_pages() == 64
+
+
+def test_cancelling_a_request_gives_back_what_it_holds_wherever_it_is():
+    s = Scheduler(cache(pages=8, seqs=2), max_batch_tokens=64, chunk_size=16, ignore_eos=True)
+    s.add(Request(0, list(range(10, 50)), 9))          # will be part-way through its prompt
+    s.add(Request(1, list(range(10, 20)), 9))          # will be decoding
+    s.add(Request(2, list(range(10, 20)), 9))          # waits for a seat
+    for _ in range(2):
+        plan = s.plan()
+        for e in plan.entries:
+            assert s.cache.grow(e.seq.seat, e.start + len(e.tokens))
+        s.complete(plan, [fake_token(e.seq.request.id, e.start + len(e.tokens)) for e in plan.entries if e.sample])
+    assert [q.request.id for q in s.running] == [0, 1] and s.running[0].prefilling and not s.running[1].prefilling
+    # a step booked but not resolved: the token it will bring for request 1 is dropped
+    plan = s.plan()
+    for e in plan.entries:
+        assert s.cache.grow(e.seq.seat, e.start + len(e.tokens))
+    ticket = s.book(plan)
+    evs = s.cancel(1) + s.cancel(2) + s.cancel(7)       # decoding, waiting, unknown
+    assert [(e.kind, e.request_id, e.reason, e.tokens) for e in evs] == [("done", 1, "cancelled", 2), ("done", 2, "cancelled", 0)]
+    sampled = [fake_token(e.seq.request.id, e.start + len(e.tokens)) for e in plan.entries if e.sample]
+    assert all(ev.request_id == 0 for ev in s.resolve(ticket, sampled))
+    s.cache.check()
+    assert s.cache.free_seats == 1 and not s.waiting
+    out, reasons, _, _ = run(s)
+    assert reasons == {(0, 0): "length"} and len(out[(0, 0)]) in (8, 9)
+    assert s.cache.free_seats == 2 and s.cache.groups[0].free_pages() == 8
 
 
 def test_n_seqs_share_an_id_and_differ_by_seq_index():
@@ -427,7 +490,7 @@ def test_admission_asks_each_group_what_a_prompt_needs():
     prompt is; a model without keys needs none.  Admission by ceil(prompt / page) for every
     group would refuse (or make wait) requests that fit."""
     from kv_cache_optimization_for_llm_amd.parts.base import StateSpec
-    win = KVCacheSpec(1, 16, kind="window", window=20)
+    win = attention_cache_spec(1, 16, kind="window", window=20)
     # 6 pages of 16: a prompt of 300 tokens is 19 pages of keys, but 20 - 1 + 16 positions at a time
     m = CacheManager([(win, [0])], {}, page_size=16, num_pages=6, max_seqs=2, max_seq_len=512)
     g = m.groups[0]

@@ -4,6 +4,9 @@
   model folder and stepped - whole, in portions, token by token, beside another request, and
   after its seat was used by someone else - without a change to the framework's files;
 * one model has different mixers in different layers;
+* a mixer whose cache entry is not keys and values of heads - one latent vector and one fp32 number
+  per token - declares its arrays by name and shape and gets pages, a block table and a pool of
+  its own from the same cache manager, beside an attention layer's;
 * the run order is data: a layer is run twice (with a cache of its own each time) and a layer
   reads another call's cache without writing;
 * another position encoding (rotation of neighbouring pairs instead of half-apart pairs) and a
@@ -24,8 +27,8 @@ from kv_cache_optimization_for_llm_amd.engine.engine import Engine, EngineOption
 from kv_cache_optimization_for_llm_amd.models.spec import (LayerCall, LayerSpec, ModelSpec, PartSpec,
                                                            TensorSpec)
 from kv_cache_optimization_for_llm_amd.ops import kernels as K
-from kv_cache_optimization_for_llm_amd.parts.base import (Block, FeedForward, Mixer, MixerContext,
-                                                          PositionEncoding, StateSpec)
+from kv_cache_optimization_for_llm_amd.parts.base import (Block, CacheArray, FeedForward, KVCacheSpec, Mixer,
+                                                          MixerContext, PositionEncoding, StateSpec)
 from kv_cache_optimization_for_llm_amd.weights.random_init import write_random_model
 
 pytestmark = pytest.mark.gpu
@@ -62,6 +65,55 @@ class ToyDecayMixer(Mixer):
                 y[t] = s
             ctx.state[seat] = s
         return (y @ self.w_out.t()).to(x.dtype)
+
+
+class ToyLatentMixer(Mixer):
+    """Attention over one latent vector per token: c_t = W_c x_t, g_t = 1 + tanh(w_g . x_t) (kept in
+    32-bit), q_t = W_q x_t; y_t = W_o sum_{s<=t} softmax_s(q_t . c_s / sqrt(w)) g_s c_s.  What it
+    keeps per token is not keys and values of heads but two arrays of its own, of different widths
+    and types; it reads them back through the block table it is handed."""
+
+    def __init__(self, prefix, *, hidden_size, latent_size):
+        super().__init__(prefix)
+        self.h, self.w = hidden_size, latent_size
+
+    def tensor_specs(self):
+        p = self.prefix
+        return {p + "c.weight": TensorSpec((self.w, self.h)), p + "q.weight": TensorSpec((self.w, self.h)),
+                p + "g.weight": TensorSpec((1, self.h)), p + "o.weight": TensorSpec((self.h, self.w))}
+
+    def load(self, tensors):
+        p = self.prefix
+        self.wc, self.wq, self.wg, self.wo = (tensors[p + n + ".weight"].float() for n in "cqgo")
+
+    def kv_cache_spec(self):
+        return KVCacheSpec((CacheArray("latent", (self.w,), token_axis=0),
+                            CacheArray("gain", (1,), token_axis=0, dtype=torch.float32)))
+
+    def forward(self, x, ctx: MixerContext):
+        b, kv = ctx.batch, ctx.kv
+        xf = x.float()
+        c, q, g = xf @ self.wc.t(), xf @ self.wq.t(), 1 + torch.tanh(xf @ self.wg.t())
+        latent, gain = kv.arrays["latent"], kv.arrays["gain"]           # [pages, page, w], [pages, page, 1]
+        assert latent.shape[1:] == (kv.page_size, self.w) and gain.dtype == torch.float32
+        if kv.writes:
+            slots = kv.slot_mapping.long()
+            latent.view(-1, self.w)[slots] = c.to(latent.dtype)
+            gain.view(-1)[slots] = g[:, 0]
+        y = torch.empty_like(c)
+        for e in range(b.num_entries):
+            seat, lo, hi = int(b.h_entry_seat[e]), int(b.h_entry_q_start[e]), int(b.h_entry_q_start[e + 1])
+            start = int(b.h_entry_start_pos[e])
+            ctx_len = start + hi - lo
+            pages = kv.block_table[seat, :(ctx_len + kv.page_size - 1) // kv.page_size].long()
+            cs = latent[pages].reshape(-1, self.w)[:ctx_len].float()      # what the cache holds (rounded to its type)
+            gs = gain[pages].reshape(-1)[:ctx_len]
+            scores = q[lo:hi] @ cs.t() / math.sqrt(self.w)
+            keys = torch.arange(ctx_len, device=x.device)[None, :]
+            mine = (start + torch.arange(hi - lo, device=x.device))[:, None]
+            prob = torch.softmax(scores.masked_fill(keys > mine, float("-inf")), dim=-1)
+            y[lo:hi] = (prob * gs[None, :]) @ cs
+        return (y @ self.wo.t()).to(x.dtype)
 
 
 class ToyNeighbourRotary(PositionEncoding):
@@ -119,7 +171,7 @@ ROUTER_GAIN = 40.0
 
 def toy_config(kind, dtype="float32"):
     return dict(architectures=[kind], vocab_size=97, hidden_size=40, state_size=24, intermediate_size=56,
-                num_heads=4, num_kv_heads=2, head_dim=16, eps=1e-5, theta=10000.0,
+                num_heads=4, num_kv_heads=2, head_dim=16, eps=1e-5, theta=10000.0, latent_size=12,
                 max_position_embeddings=256, torch_dtype=dtype)
 
 
@@ -127,6 +179,8 @@ def toy_layer(c, i, mixer):
     p = f"blocks.{i}."
     if mixer == "toy_decay":
         mx = PartSpec("toy_decay", dict(prefix=p + "mix.", hidden_size=c["hidden_size"], state_size=c["state_size"]))
+    elif mixer == "toy_latent":
+        mx = PartSpec("toy_latent", dict(prefix=p + "lat.", hidden_size=c["hidden_size"], latent_size=c["latent_size"]))
     else:
         pos = PartSpec("rotary", dict(head_dim=c["head_dim"], max_positions=c["max_position_embeddings"],
                                       theta=c["theta"]))
@@ -210,6 +264,10 @@ def registered():
     BLOCKS.register("toy_sandwich", ToySandwichBlock, replace=True)
     register_architecture("ToySandwichLM", dict, sandwich_spec, replace=True)
     MIXERS.register("toy_decay", ToyDecayMixer, replace=True)
+    MIXERS.register("toy_latent", ToyLatentMixer, replace=True)
+    register_architecture("ToyLatentLM", dict, toy_spec(
+        "ToyLatentLM", ["toy_latent", "gqa_attention", "toy_latent"],
+        [LayerCall(0, 0), LayerCall(1, 1), LayerCall(2, 2)]), replace=True)
     POSITION_ENCODINGS.register("toy_neighbour_rotary", ToyNeighbourRotary, replace=True)
     FEED_FORWARDS.register("toy_routed", ToyRoutedFFN, replace=True)
     register_architecture("ToyRoutedLM", dict, routed_spec, replace=True)
@@ -222,6 +280,7 @@ def registered():
         [LayerCall(0, 0), LayerCall(1, 1), LayerCall(0, 2), LayerCall(1, 1, writes_cache=False)]), replace=True)
     yield
     MIXERS.unregister("toy_decay")
+    MIXERS.unregister("toy_latent")
     BLOCKS.unregister("toy_sandwich")
     POSITION_ENCODINGS.unregister("toy_neighbour_rotary")
     FEED_FORWARDS.unregister("toy_routed")
@@ -318,6 +377,70 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(dtype, tol, tmp_pa
     eng.release("a")
     eng.release("b")
     assert err(eng.step([StepEntry("c", b, list(range(23)))]), rb) <= tol
+    eng.cache.check()
+
+
+def ref_latent_layer(c, W, i, h, cache_dtype):
+    p, w = f"blocks.{i}.", c["latent_size"]
+    x = plain.rms_norm(h, W[p + "n1.weight"], c["eps"])
+    cs = (x @ W[p + "lat.c.weight"].t()).to(cache_dtype).float()         # the cache stores the latent in its type
+    q, g = x @ W[p + "lat.q.weight"].t(), 1 + torch.tanh(x @ W[p + "lat.g.weight"].t())[:, 0]
+    T = h.shape[0]
+    scores = (q @ cs.t() / math.sqrt(w)).masked_fill(torch.triu(torch.ones(T, T, dtype=torch.bool), 1), float("-inf"))
+    y = (torch.softmax(scores, dim=-1) * g[None, :]) @ cs
+    return ref_ffn(c, W, p, h + y @ W[p + "lat.o.weight"].t())
+
+
+@pytest.mark.parametrize("dtype, tol", [("float32", 3e-5), ("bfloat16", 2e-2)])
+def test_a_mixer_whose_cache_entry_is_one_vector_per_token(dtype, tol, tmp_path, gpu):
+    """The cache manager allocates what a mixer's description says - here a latent vector of 12
+    elements and one 32-bit number per token, pages ``[page, 12]`` and ``[page, 1]`` - beside an
+    attention layer's keys and values, which form a group of their own with its own pool and block
+    table; the engine sizes the pool from the same description (no pool size is given).  Whole,
+    in portions beside another request's decoded tokens, and on pages that were used before."""
+    c = toy_config("ToyLatentLM", "bfloat16")
+    d = write_random_model(str(tmp_path / "toy"), c, seed=31, gain=1.0)
+    W = load_plain(d)
+    page = 8
+    eng = Engine(d, EngineOptions(dtype=dtype, max_seqs=2, max_seq_len=96, page_size=page))
+    assert eng.graphs is None
+    elem = 4 if dtype == "float32" else 2
+    groups = {tuple(a.name for a in g.spec.arrays): g for g in eng.cache.groups}
+    assert sorted(groups) == [("k", "v"), ("latent", "gain")]
+    lat, att = groups[("latent", "gain")], groups[("k", "v")]
+    assert lat.slot_ids == [0, 2] and att.slot_ids == [1]
+    assert lat.arrays["latent"].shape == (2, lat.num_pages, page, 12) and lat.arrays["gain"].dtype == torch.float32
+    assert att.arrays["v"].shape == (1, att.num_pages, 2, 16, page)
+    assert eng.cache.page_bytes() == page * (2 * (12 * elem + 4) + 2 * 2 * 16 * elem)
+    assert lat.num_pages == 2 * 96 // page            # every seat at its longest: nothing more is worth having
+
+    def ref(toks):
+        h = W["embed.weight"][torch.tensor(toks)]
+        h = ref_latent_layer(c, W, 0, h, eng.dtype)
+        h, _ = ref_attn_layer(c, W, 1, h)
+        h = ref_latent_layer(c, W, 2, h, eng.dtype)
+        return plain.rms_norm(h, W["final.weight"], c["eps"]) @ W["head.weight"].t()
+
+    rng = np.random.default_rng(6)
+    a = [int(t) for t in rng.integers(0, 97, 61)]
+    b = [int(t) for t in rng.integers(0, 97, 30)]
+    ra, rb = ref(a), ref(b)
+    assert err(eng.step([StepEntry("w", a, list(range(61)))]), ra) <= tol
+    eng.release("w")
+    reused_before = sum(g.pool.reuses for g in eng.cache.groups)
+    rows_a, rows_b, ia, ib = [], [], 0, 0
+    for n in (7, 2, 16, 1, 1, 5, 29):
+        step = [StepEntry("a", a[ia:ia + n], list(range(n)))]
+        if ib < len(b):
+            step.append(StepEntry("b", [b[ib]], [0]))
+        out = eng.step(step).cpu()
+        rows_a.append(out[:n])
+        if ib < len(b):
+            rows_b.append(out[n:])
+            ib += 1
+        ia += n
+    assert ia == 61 and err(torch.cat(rows_a), ra) <= tol and err(torch.cat(rows_b), rb[:ib]) <= tol
+    assert sum(g.pool.reuses for g in eng.cache.groups) > reused_before       # on pages the first request gave back
     eng.cache.check()
 
 
