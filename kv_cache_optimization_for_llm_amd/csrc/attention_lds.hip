@@ -78,15 +78,17 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, float *__restrict__ part
         my_lo[rt] = (window > 0 && my_pos[rt] - window + 1 > 0) ? my_pos[rt] - window + 1 : 0;
     }
     const int w_last = (wrow0 + 31 < M - 1) ? wrow0 + 31 : M - 1;
-    const int w_hi = start_pos + w_last / G;                              // last key the wave sees
-    const int w_first_pos = start_pos + wrow0 / G;
+    // (uniform over the wavefront: said explicitly, since the division by G is done in the vector
+    // ALU and the compiler then takes every test on these for a per-lane one)
+    const int w_hi = __builtin_amdgcn_readfirstlane(start_pos + w_last / G);      // last key the wave sees
+    const int w_first_pos = __builtin_amdgcn_readfirstlane(start_pos + wrow0 / G);
     const int w_lo = (window > 0 && w_first_pos - window + 1 > 0) ? w_first_pos - window + 1 : 0;
     const bool all_rows = wrow0 + 32 <= M;
 
     // ---- keys the workgroup visits
     const int g_last = (row0 + 127 < M - 1) ? row0 + 127 : M - 1;
-    const int g_hi = start_pos + g_last / G;
-    const int g_first_pos = start_pos + row0 / G;
+    const int g_hi = __builtin_amdgcn_readfirstlane(start_pos + g_last / G);
+    const int g_first_pos = __builtin_amdgcn_readfirstlane(start_pos + row0 / G);
     const int g_lo = (window > 0 && g_first_pos - window + 1 > 0) ? g_first_pos - window + 1 : 0;
     int k_begin = g_lo & ~31;
     int k_end = g_hi + 1;

@@ -97,8 +97,10 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
 
     // keys any row of this item may see
     const int last_row = (row0 + 16 * RT - 1 < M - 1) ? row0 + 16 * RT - 1 : M - 1;
-    const int item_hi = start_pos + last_row / G;                       // inclusive
-    const int item_pos_lo = start_pos + row0 / G;
+    // (uniform over the wavefront like everything above: said explicitly, because the division by G
+    // is done in the vector ALU and the compiler then takes every test on these for a per-lane one)
+    const int item_hi = __builtin_amdgcn_readfirstlane(start_pos + last_row / G);                       // inclusive
+    const int item_pos_lo = __builtin_amdgcn_readfirstlane(start_pos + row0 / G);
     const int item_lo = (window > 0 && item_pos_lo - window + 1 > 0) ? item_pos_lo - window + 1 : 0;
     int k_begin = item_lo & ~31;
     int k_end = item_hi + 1;                                            // exclusive
@@ -221,7 +223,7 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
 
     // exponentials are taken in base 2: exp(x * scale) = exp2(x * scale * log2(e))
     const float scale2 = scale * 1.44269504088896340736f;
-    const int first_pos = start_pos + row0 / G;          // smallest position among the item's rows
+    const int first_pos = item_pos_lo;                   // smallest position among the item's rows
     const bool all_rows = row0 + 16 * RT <= M;
 
     // One 32-key block for all row tiles of the item, as straight-line code: first every S^T
@@ -306,27 +308,27 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
             l[rt] += quad_rows_sum(lsum);
         }
         // ---- O^T += V^T * P^T
-        // A block that reaches past the item's last key holds, behind it, whatever the page held
-        // before (or the nearest needed tile, for a redirected one): P is zero there, and the
-        // values are made zero too, so that nothing non-finite left in a page can reach this request.
-        if (MASKED && kstart + 31 > item_hi) {
-            const int n0 = item_hi + 1 - (kstart + 4 * g), n1 = n0 - 16;
-#pragma unroll
-            for (int dt = 0; dt < NDT; ++dt) {
-                Frag8 vv;
-                vv.u2[0] = keep_first_keys(f.v[dt].u2[0], n0);
-                vv.u2[1] = keep_first_keys(f.v[dt].u2[1], n1);
-#pragma unroll
-                for (int rt = 0; rt < RT; ++rt)
-                    o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv.v, pf[rt].v, o[rt][dt], 0, 0, 0);
-            }
-            return;
+        // Behind the item's last key a block holds whatever the page held before (or the nearest
+        // needed tile, for a redirected one): P is zero there, and the values are made zero too, so
+        // that nothing non-finite left in a page can reach this request.  Straight-line code for
+        // every masked block (the masks are all ones where the block ends before the item's last key).
+        uint2 keep[2];
+        if (MASKED) {
+            const int n0 = item_hi + 1 - (kstart + 4 * g);
+            keep[0] = keep_first_keys(make_uint2(~0u, ~0u), n0);
+            keep[1] = keep_first_keys(make_uint2(~0u, ~0u), n0 - 16);
         }
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-            for (int dt = 0; dt < NDT; ++dt)
-                o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.v[dt].v, pf[rt].v, o[rt][dt], 0, 0, 0);
+            for (int dt = 0; dt < NDT; ++dt) {
+                Frag8 vv = f.v[dt];
+                if (MASKED) {
+                    vv.u2[0].x &= keep[0].x; vv.u2[0].y &= keep[0].y;
+                    vv.u2[1].x &= keep[1].x; vv.u2[1].y &= keep[1].y;
+                }
+                o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv.v, pf[rt].v, o[rt][dt], 0, 0, 0);
+            }
     };
     auto compute_block = [&](const BlockFrags &f, int kstart) {
         // incl. redirected tiles and items whose last row tile is cut short

@@ -391,7 +391,10 @@ def ref_latent_layer(c, W, i, h, cache_dtype):
     return ref_ffn(c, W, p, h + y @ W[p + "lat.o.weight"].t())
 
 
-@pytest.mark.parametrize("dtype, tol", [("float32", 3e-5), ("bfloat16", 2e-2)])
+# (bfloat16: three layers of N(0, 1 / sqrt(in)) matrices; rounding every op's output to bfloat16 moves
+# the plain two-layer models' logits by 1.0-1.5 % of their scale, so 3 % here; the 32-bit run is the
+# one that would show a wrong page or a wrong array)
+@pytest.mark.parametrize("dtype, tol", [("float32", 3e-5), ("bfloat16", 3e-2)])
 def test_a_mixer_whose_cache_entry_is_one_vector_per_token(dtype, tol, tmp_path, gpu):
     """The cache manager allocates what a mixer's description says - here a latent vector of 12
     elements and one 32-bit number per token, pages ``[page, 12]`` and ``[page, 1]`` - beside an
