@@ -141,7 +141,11 @@ def gemm(args) -> None:
                  for w in tiled]
     elif mode == "swiglu":
         out = torch.empty(m, n // 2, device=dev).bfloat16()
-        calls = [lambda w=w: product(x, w, out, swiglu=True) for w in tiled]
+        if args.x_tiled:
+            xt = K.TiledRows.from_rows(x)
+            calls = [lambda w=w: product(xt, w, out, swiglu=True, x_tiled=True) for w in tiled]
+        else:
+            calls = [lambda w=w: product(x, w, out, swiglu=True) for w in tiled]
     else:
         out = torch.empty(m, n, device=dev, dtype=torch.float32 if mode == "f32" else torch.bfloat16)
         calls = [lambda w=w: product(x, w, out) for w in tiled]
@@ -248,6 +252,7 @@ def main(argv=None) -> int:
     g.add_argument("--kernel", choices=["few-rows", "gemv"], default="few-rows",
                    help="the matrix-core kernel over the tiled weight, or the matrix-vector kernel (one or two rows)")
     g.add_argument("--graph", action="store_true", help="time the launches inside a captured graph")
+    g.add_argument("--x-tiled", action="store_true", help="gated product: the rows of X laid out [K / 8][rows][8]")
     g.add_argument("--reps", type=int, default=48)
     pr = sub.add_parser("prompt")
     pr.add_argument("--tokens", type=int, default=8192)

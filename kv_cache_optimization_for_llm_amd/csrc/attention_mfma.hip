@@ -41,7 +41,38 @@
 // a wavefront's key range from which a third block of keys is kept in flight (decoded tokens)
 #define LONG_RANGE_KEYS 1536
 
-template <int D, int RT, bool FAST, bool STREAM>
+// ROPE: the item is one decoded token whose Q, K and V lie in `q` as the joined projection left them
+// ([.., q heads | k heads | v heads] per row, not yet rotated, nothing cached).  The wavefront
+// rotates Q as it loads it, rotates the token's new K, puts K and V into the block of keys that
+// holds the token's position (in registers: the page is not read back) and - one wavefront per
+// (token, kv head) - stores them to the token's cache slot.  What the reference does in three
+// launches before its attention kernel (ropePackedKernel twice, scatterKVPackedKernel;
+// base/src/kernels.cu:289-319, paged_attention/src/kernels.cu:335-363) costs a decode step of
+// many requests one launch per layer less.  Head sizes that are multiples of 64 (a lane holds both
+// elements of a rotate-half pair), pages of 16.
+struct RopeArgs {
+    const float *cos_t, *sin_t;     // [positions, D / 2] fp32; both null: no rotation
+    const int *slots;               // [tokens] cache slot of each token (negative: no write); null: nothing is cached
+};
+
+__device__ __forceinline__ void unpack8(const Frag8 &f, float (&x)[8]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = bf16_bits_to_float(f.h[i]);
+}
+
+// (a, b) <- (a c - b s, a s + b c) element by element, rounded to bf16 as the rotation kernel rounds
+__device__ __forceinline__ void rotate_pair(Frag8 &fa, Frag8 &fb, const float (&c)[8], const float (&s)[8]) {
+    float a[8], b[8];
+    unpack8(fa, a);
+    unpack8(fb, b);
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) {
+        fa.p2[i / 2] = pack_bf16(a[i] * c[i] - b[i] * s[i], a[i + 1] * c[i + 1] - b[i + 1] * s[i + 1]);
+        fb.p2[i / 2] = pack_bf16(a[i] * s[i] + b[i] * c[i], a[i + 1] * s[i + 1] + b[i + 1] * c[i + 1]);
+    }
+}
+
+template <int D, int RT, bool FAST, bool STREAM, bool ROPE = false>
 __device__ __forceinline__ void
 attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
                       const bf16_t *__restrict__ q, int q_row_stride,
@@ -51,8 +82,10 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
                       const int *__restrict__ item_entry, const int *__restrict__ item_row0,
                       const int *__restrict__ entry_seat, const int *__restrict__ entry_q_start,
                       const int *__restrict__ entry_start_pos, int num_q_heads, int num_kv_heads,
-                      int page_size, float scale, int window, int splits, int keys_per_split, const int item, const int kvh, const int split) {
+                      int page_size, float scale, int window, int splits, int keys_per_split, const int item, const int kvh, const int split,
+                      const RopeArgs rope = RopeArgs{nullptr, nullptr, nullptr}) {
     constexpr int KSTEP = (D % 32 == 0) ? 32 : 16;   // head-dim slice per S^T product
+    static_assert(!ROPE || (RT == 1 && FAST && D % 64 == 0), "rotation inside the kernel: one row tile, pages of 16, head sizes that are multiples of 64");
     constexpr int NKS = D / KSTEP;
     constexpr int NDT = D / 16;                      // 16-wide tiles of the value dimension
 
@@ -125,6 +158,77 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
             else qf4[rt][ks].u2 = *reinterpret_cast<const uint2 *>(qrow + ks * 16 + g * 4);
         }
     }
+
+    // ---- ROPE: rotate Q; make the token's K (rotated) and V ready for the cache and for the
+    // block of keys that holds its position
+    constexpr int HK = NKS / 2;                       // a rotate-half pair lies HK slices apart
+    Frag8 k_new[ROPE ? NKS : 1];
+    uint16_t v_new[ROPE ? NDT : 1];
+    const bool caches = ROPE && rope.slots != nullptr;
+    int rope_slot = -1;
+    float cs[ROPE ? HK : 1][8], sn[ROPE ? HK : 1][8];
+    if constexpr (ROPE) {
+#pragma unroll
+        for (int h = 0; h < HK; ++h)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) { cs[h][i] = 1.f; sn[h][i] = 0.f; }
+        if (caches) rope_slot = rope.slots[q_start];
+        if (rope.cos_t != nullptr) {
+            const size_t at = (size_t)start_pos * (D / 2) + g * 8;
+#pragma unroll
+            for (int h = 0; h < HK; ++h) {
+                const float4 c0 = *reinterpret_cast<const float4 *>(rope.cos_t + at + h * 32);
+                const float4 c1 = *reinterpret_cast<const float4 *>(rope.cos_t + at + h * 32 + 4);
+                const float4 s0 = *reinterpret_cast<const float4 *>(rope.sin_t + at + h * 32);
+                const float4 s1 = *reinterpret_cast<const float4 *>(rope.sin_t + at + h * 32 + 4);
+                cs[h][0] = c0.x; cs[h][1] = c0.y; cs[h][2] = c0.z; cs[h][3] = c0.w;
+                cs[h][4] = c1.x; cs[h][5] = c1.y; cs[h][6] = c1.z; cs[h][7] = c1.w;
+                sn[h][0] = s0.x; sn[h][1] = s0.y; sn[h][2] = s0.z; sn[h][3] = s0.w;
+                sn[h][4] = s1.x; sn[h][5] = s1.y; sn[h][6] = s1.z; sn[h][7] = s1.w;
+            }
+        }
+        const bf16_t *tok_row = q + (size_t)q_start * q_row_stride;
+        if (caches) {
+            // every lane takes the slice of its lane group g (the same for all 16 rows r) and its
+            // row's value dimensions: no branch around loads
+            const bf16_t *krow = tok_row + (size_t)(num_q_heads + kvh) * D;
+            const bf16_t *vrow = tok_row + (size_t)(num_q_heads + num_kv_heads + kvh) * D;
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) k_new[ks].u4 = *reinterpret_cast<const uint4 *>(krow + ks * 32 + g * 8);
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) v_new[dt] = vrow[dt * 16 + r].bits;
+        }
+    }
+    // The arithmetic on what was asked for above waits for it, so it runs after the first blocks of
+    // keys have been asked for as well (one trip to memory for all of it, not two).
+    auto rotate_and_store = [&]() {
+        if constexpr (ROPE) {
+            if (rope.cos_t != nullptr) {
+    #pragma unroll
+                for (int h = 0; h < HK; ++h) {
+                    rotate_pair(qf8[0][h], qf8[0][h + HK], cs[h], sn[h]);
+                    if (caches) rotate_pair(k_new[h], k_new[h + HK], cs[h], sn[h]);
+                }
+            }
+            // one wavefront per (token, kv head) stores them: the one whose key range holds the position
+            const int off = start_pos & 15;
+            const bool owner = caches && row0 == 0 && (splits == 1 || split == start_pos / keys_per_split);
+            const int slot = rope_slot;
+            if (owner && slot >= 0) {
+                const size_t page_elems = ((size_t)(slot >> 4) * num_kv_heads + kvh) * (size_t)(16 * D);
+                if (r == off) {
+    #pragma unroll
+                    for (int ks = 0; ks < NKS; ++ks)
+                        *reinterpret_cast<uint4 *>(const_cast<bf16_t *>(k_cache) + page_elems + (size_t)(slot & 15) * D + ks * 32 + g * 8) = k_new[ks].u4;
+                }
+                if (g == 0) {
+    #pragma unroll
+                    for (int dt = 0; dt < NDT; ++dt)
+                        const_cast<bf16_t *>(v_cache)[page_elems + (size_t)(dt * 16 + r) * 16 + (slot & 15)].bits = v_new[dt];
+                }
+            }
+        }
+    };
 
     float m[RT], l[RT];
     f32x4 o[RT][NDT];
@@ -330,7 +434,34 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
                 o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv.v, pf[rt].v, o[rt][dt], 0, 0, 0);
             }
     };
-    auto compute_block = [&](const BlockFrags &f, int kstart) {
+    auto compute_block = [&](BlockFrags &f, int kstart) {
+        if constexpr (ROPE) {
+            // the block that holds the token's own position gets its key and value from registers
+            if (caches && kstart <= start_pos && start_pos < kstart + 32) {
+                // (selects between values: a store through a pointer chosen at run time, or under a
+                // branch per tile, makes the compiler keep the fragments in memory)
+                const int off = start_pos & 15, i = start_pos & 3;
+                const bool second = start_pos - kstart >= 16;           // uniform
+                const bool k0 = r == off && !second, k1 = r == off && second;
+#pragma unroll
+                for (int ks = 0; ks < NKS; ++ks) {
+                    const uint4 n = k_new[ks].u4, a = f.k8[0][ks].u4, b = f.k8[1][ks].u4;
+                    f.k8[0][ks].u4 = make_uint4(k0 ? n.x : a.x, k0 ? n.y : a.y, k0 ? n.z : a.z, k0 ? n.w : a.w);
+                    f.k8[1][ks].u4 = make_uint4(k1 ? n.x : b.x, k1 ? n.y : b.y, k1 ? n.z : b.z, k1 ? n.w : b.w);
+                }
+                const bool mine = g == (off >> 2);
+                const uint32_t sh = (i & 1) * 16, keep = ~(0xffffu << sh);
+                const bool x0 = mine && !second && i < 2, y0 = mine && !second && i >= 2;
+                const bool x1 = mine && second && i < 2, y1 = mine && second && i >= 2;
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt) {
+                    const uint32_t put = (uint32_t)v_new[dt] << sh;
+                    const uint2 a = f.v[dt].u2[0], b = f.v[dt].u2[1];
+                    f.v[dt].u2[0] = make_uint2(x0 ? (a.x & keep) | put : a.x, y0 ? (a.y & keep) | put : a.y);
+                    f.v[dt].u2[1] = make_uint2(x1 ? (b.x & keep) | put : b.x, y1 ? (b.y & keep) | put : b.y);
+                }
+            }
+        }
         // incl. redirected tiles and items whose last row tile is cut short
         const bool masked = window > 0 || kstart + 31 > first_pos || !all_rows;
         if (masked) compute_block_as(std::true_type{}, f, kstart);
@@ -351,6 +482,7 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
     if (RT == 1 && STREAM && D <= 128 && splits == 1 && k_end - k_begin >= LONG_RANGE_KEYS) {   // (a third set of registers spills from 224 on)
         BlockFrags fc;
         load_block(fb, k_begin + 32);
+        rotate_and_store();
         for (int kstart = k_begin; kstart < k_end; kstart += 96) {
             load_block(fc, kstart + 64);
             compute_block(fa, kstart);
@@ -360,6 +492,17 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
             if (kstart + 64 < k_end) compute_block(fc, kstart + 64);
         }
     } else {
+        if constexpr (ROPE) {
+            // the first turn written out, so that the second block is asked for before the rotation waits
+            load_block(fb, k_begin + 32);
+            rotate_and_store();
+            if (k_begin < k_end) {
+                compute_block(fa, k_begin);
+                load_block(fa, k_begin + 64);
+                if (k_begin + 32 < k_end) compute_block(fb, k_begin + 32);
+            }
+            k_begin += 64;
+        }
         for (int kstart = k_begin; kstart < k_end; kstart += 64) {
             load_block(fb, kstart + 32);
             compute_block(fa, kstart);
@@ -423,6 +566,22 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
         attention_item<D, RT, FAST, STREAM>(out, part_o, part_ml, q, q_row_stride, k_cache, v_cache, block_table, max_blocks,
                                     item_meta, item_entry, item_row0, entry_seat, entry_q_start, entry_start_pos, num_q_heads,
                                     num_kv_heads, page_size, scale, window, splits, keys_per_split, other, kvh, split);
+}
+
+// One wavefront per (decoded token, kv head, key split), with rotation and cache write inside.
+template <int D, bool STREAM>
+__global__ void __launch_bounds__(KVA_WAVE)
+attention_mfma_rope_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
+                           const bf16_t *__restrict__ qkv, int row_stride,
+                           bf16_t *k_cache, bf16_t *v_cache,
+                           const int *__restrict__ block_table, int max_blocks,
+                           const int *__restrict__ item_meta, int num_q_heads, int num_kv_heads,
+                           float scale, int window, int splits, int keys_per_split, const RopeArgs rope) {
+    const int kvh = blockIdx.x % num_kv_heads, split = blockIdx.z;
+    const int w = blockIdx.x / num_kv_heads;
+    attention_item<D, 1, true, STREAM, true>(out, part_o, part_ml, qkv, row_stride, k_cache, v_cache, block_table, max_blocks,
+                                             item_meta, nullptr, nullptr, nullptr, nullptr, nullptr, num_q_heads,
+                                             num_kv_heads, 16, scale, window, splits, keys_per_split, w, kvh, split, rope);
 }
 
 // out[row, :] = sum_s o_s * exp(m_s - M) / sum_s l_s * exp(m_s - M),  M = max_s m_s.
@@ -600,6 +759,56 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
         return kva_attention_merge_launch(out, part_o, part_ml, head_dim, splits, item_meta, item_entry, item_row0,
                                           entry_q_start, num_items, 16 * row_tiles, total_rows, num_q_heads,
                                           num_kv_heads, all_rows, stream);
+    return KVA_OK;
+}
+
+extern "C" int kva_attention_mfma_rope_supported(int head_dim, int page_size, int group) {
+    return ((head_dim == 64 || head_dim == 128) && page_size == 16 && group >= 1 && group <= 16) ? 1 : 0;
+}
+
+// Attention of decoded tokens (one token per item: item_meta [items, 8] = (token row, 1, position,
+// seat, 0, 0, 0, 0)) straight from the joined Q/K/V projection `qkv` [tokens, (nq + 2 nkv) d] bf16,
+// not yet rotated: the kernel rotates Q and K by the token's position (cos_t / sin_t [positions, d / 2]
+// fp32, both null: no rotation), stores the rotated K and the V at the token's cache slot
+// (slots [tokens], a negative slot or slots == null: nothing is stored and the token's key is taken
+// from the cache like every other) and attends.  At most 16 query heads per kv head.
+extern "C" int kva_attention_mfma_rope(void *out, float *part_o, float *part_ml, const void *qkv, int row_stride,
+                                       void *k_cache, void *v_cache, const int *block_table, int max_blocks,
+                                       const int *item_meta, int num_items, int total_rows, int num_q_heads,
+                                       int num_kv_heads, int head_dim, int page_size, float scale, int window,
+                                       int splits, int keys_per_split, int keep_cached, const float *cos_t,
+                                       const float *sin_t, const int *slots, hipStream_t stream) {
+    KVA_REQUIRE(num_items >= 0 && num_q_heads > 0 && num_kv_heads > 0 && max_blocks > 0 && item_meta != nullptr,
+                "attention_mfma_rope: bad sizes");
+    KVA_REQUIRE(num_q_heads % num_kv_heads == 0, "attention_mfma_rope: %d query heads is not a multiple of %d kv heads",
+                num_q_heads, num_kv_heads);
+    KVA_REQUIRE(kva_attention_mfma_rope_supported(head_dim, page_size, num_q_heads / num_kv_heads),
+                "attention_mfma_rope: head_dim %d / page_size %d / %d heads per kv head not supported (64 or 128, 16, "
+                "at most 16)", head_dim, page_size, num_q_heads / num_kv_heads);
+    KVA_REQUIRE(row_stride % 8 == 0 && row_stride >= (num_q_heads + 2 * num_kv_heads) * head_dim,
+                "attention_mfma_rope: row stride %d does not hold the joined projection", row_stride);
+    KVA_REQUIRE(splits >= 1 && splits <= MERGE_MAX_SPLITS && num_kv_heads <= 65535,
+                "attention_mfma_rope: at most %d splits and 65535 kv heads", MERGE_MAX_SPLITS);
+    KVA_REQUIRE(splits == 1 || (keys_per_split > 0 && keys_per_split % 32 == 0 && part_o && part_ml),
+                "attention_mfma_rope: splits need a key count that is a multiple of 32 and a workspace");
+    KVA_REQUIRE(window >= 0 && scale > 0.f, "attention_mfma_rope: window must not be negative and the scale positive");
+    KVA_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "attention_mfma_rope: one table missing");
+    if (num_items == 0) return KVA_OK;
+    KVA_REQUIRE((long)num_items * num_kv_heads < (1L << 31), "attention_mfma_rope: too many work items");
+    dim3 grid(num_items * num_kv_heads, 1, splits), block(KVA_WAVE);
+    const RopeArgs rope{cos_t, sin_t, slots};
+#define LAUNCH(DD, SS)                                                                               \
+    hipLaunchKernelGGL((attention_mfma_rope_kernel<DD, SS>), grid, block, 0, stream, (bf16_t *)out, part_o, \
+                       part_ml, (const bf16_t *)qkv, row_stride, (bf16_t *)k_cache, (bf16_t *)v_cache,     \
+                       block_table, max_blocks, item_meta, num_q_heads, num_kv_heads, scale, window,  \
+                       splits, keys_per_split, rope)
+    if (head_dim == 64) { if (keep_cached) LAUNCH(64, false); else LAUNCH(64, true); }
+    else { if (keep_cached) LAUNCH(128, false); else LAUNCH(128, true); }
+#undef LAUNCH
+    KVA_CHECK_LAUNCH("attention_mfma_rope");
+    if (splits > 1)
+        return kva_attention_merge_launch(out, part_o, part_ml, head_dim, splits, item_meta, nullptr, nullptr,
+                                          nullptr, num_items, 16, total_rows, num_q_heads, num_kv_heads, 1, stream);
     return KVA_OK;
 }
 

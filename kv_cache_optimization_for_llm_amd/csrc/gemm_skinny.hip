@@ -155,7 +155,7 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = mt * 16 + r;
-        xr[mt] = a.x_tiled ? a.X + (16 * g + r) * 8 : a.X + (size_t)(m < a.M ? m : 0) * a.ldx + 8 * g;
+        xr[mt] = a.x_tiled ? a.X + ((size_t)g * (MT * 16) + m) * 8 : a.X + (size_t)(m < a.M ? m : 0) * a.ldx + 8 * g;
     }
 
     gf32x4 acc[NTW][MT];
@@ -389,7 +389,7 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
         // trip to memory per step, 0.43 us each.)  What is left after the whole chunks goes in
         // chunks of S/2, S/4, .. 1 steps, each with its loads up front.
         constexpr int S = NTW + MT <= 2 ? 8 : ((MT == 1 && NTW == 2) ? 4 : (NTW * MT >= 12 ? 1 : 2));   // by registers
-        const size_t xstep = a.x_tiled ? 16 : 1;               // a step of 32 columns is 4 chunks of 16 rows x 8
+        const size_t xstep = a.x_tiled ? MT * 16 : 1;          // a step of 32 columns is 4 chunks of (16 MT) rows x 8
         const int kb = __builtin_amdgcn_readfirstlane(kbeg), ke = __builtin_amdgcn_readfirstlane(kend);
         const int steps = (ke - kb) / 32, full = steps / S;
         GFrag8 w[S][NTW], x[S][MT];
@@ -680,7 +680,7 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
                 }
             } else {
                 bf16_t *dst = reinterpret_cast<bf16_t *>(a.Y) + (size_t)m * a.ldy + n;
-                if (a.y_tiled) dst = reinterpret_cast<bf16_t *>(a.Y) + ((size_t)(n >> 3) * 16 + m) * 8 + (n & 7);
+                if (a.y_tiled) dst = reinterpret_cast<bf16_t *>(a.Y) + ((size_t)(n >> 3) * (MT * 16) + m) * 8 + (n & 7);
                 if (n + 3 < rows && (a.y_tiled || a.ldy % 4 == 0)) {
                     uint2 w;
                     w.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
@@ -787,7 +787,7 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
     a.sumsq = sumsq; a.sumsq_parts = sumsq_parts; a.norm_width = norm_width; a.eps = eps;
     a.hidden = (bf16_t *)hidden; a.next_w = next_w; a.next_w_f32 = next_w_f32;
     a.scaled_out = (bf16_t *)scaled_out; a.sumsq_out = sumsq_out;
-    KVA_REQUIRE(!(x_tiled || y_tiled) || M <= 16, "gemm_skinny: the tiled layouts of X and Y are for at most 16 rows");
+    // (tiled X or Y: [columns / 8][rows rounded up to 16][8])
     KVA_REQUIRE(!y_tiled || (mode == 2 && (N / 2) % 8 == 0), "gemm_skinny: a tiled result is for the gated product with a multiple of 8 columns");
     KVA_REQUIRE(!x_tiled || K % 8 == 0, "gemm_skinny: tiled X");
     a.x_tiled = x_tiled ? 1 : 0; a.y_tiled = y_tiled ? 1 : 0;
@@ -808,7 +808,7 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
     int groups_per_wg = kw >= 4 ? 1 : 4 / kw;
     // More than 16 tokens and several tiles per wave: workgroups of several tile groups that
     // share X through LDS (at most 4 K ranges of 2 x 64 tokens x 128 bytes: 64 KiB).
-    const bool xl = M > 16 && ntw >= 2 && groups >= 2;
+    const bool xl = M > 16 && ntw >= 2 && groups >= 2 && !x_tiled;      // tiled rows are read in whole cache lines as they are
     if (xl) {
         kw = kw < 4 ? kw : 4;
         groups_per_wg = kw == 4 ? 2 : 4;

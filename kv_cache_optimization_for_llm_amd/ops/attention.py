@@ -116,8 +116,29 @@ def choose_lds_splits(groups: int, max_context: int, max_splits: int = None, hea
     return _cut_keys(min(want, max(1, max_context // min_keys)), max_context, max_splits)
 
 
+def _plan_for(batch, kv, num_q_heads: int, num_kv_heads: int, head_dim: int) -> list:
+    plans = batch.attention_plans
+    key = (num_q_heads, num_kv_heads, head_dim, kv.page_size)
+    plan = plans.get(key)
+    if plan is None:
+        plan = plans[key] = _plan(batch, num_q_heads // num_kv_heads, num_kv_heads, head_dim, kv.page_size)
+    return plan
+
+
+def rotates_in_kernel(batch, kv, num_q_heads: int, num_kv_heads: int, head_dim: int, dtype) -> bool:
+    """Whether :func:`paged_attention` can take the joined projection as the product left it and
+    do rotation and cache write itself (``rope=...``): a bfloat16 step of decoded tokens only, a
+    geometry the kernel takes, every token one work item whose record the host could make."""
+    if kv is None or dtype != torch.bfloat16 or batch.max_q_len != 1 or num_q_heads % num_kv_heads:
+        return False
+    if not K.attention_mfma_rope_supported(head_dim, kv.page_size, num_q_heads // num_kv_heads):
+        return False
+    plan = _plan_for(batch, kv, num_q_heads, num_kv_heads, head_dim)
+    return len(plan) == 1 and plan[0][0] == "wave" and plan[0][1][2] is not None
+
+
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads: int,
-                    num_kv_heads: int, head_dim: int, scale: float, window: int = 0) -> torch.Tensor:
+                    num_kv_heads: int, head_dim: int, scale: float, window: int = 0, rope=None) -> torch.Tensor:
     """Causal GQA attention of the step's tokens over the paged cache.  ``qkv`` is the fused
     projection output ``[T, (nq + 2 nkv) d]`` (or just its Q part) whose first ``nq * d`` columns
     are the (already position-encoded) queries; keys and values are read from ``kv``.
@@ -131,16 +152,21 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
     batch."""
     if kv is None:
         raise K.KernelError("paged_attention: the mixer has no cache view")
+    if rope is not None:
+        # decoded tokens whose rotation and cache write are still to be done: ``rope`` = (cos, sin)
+        # tables or (None, None); only where rotates_in_kernel() said yes
+        if not rotates_in_kernel(batch, kv, num_q_heads, num_kv_heads, head_dim, qkv.dtype):
+            raise K.KernelError("paged_attention: this step cannot rotate inside the attention kernel")
+        (_, (_, _, meta), _, splits, per, _, _, keep_cached), = _plan_for(batch, kv, num_q_heads, num_kv_heads, head_dim)
+        return K.attention_mfma_rope(qkv, out, kv.k_cache, kv.v_cache, kv.block_table, meta, num_q_heads,
+                                     num_kv_heads, head_dim, scale, rope[0], rope[1],
+                                     kv.slot_mapping if kv.writes else None, window, splits, per, keep_cached)
     if not (qkv.dtype == torch.bfloat16 and K.attention_mfma_supported(head_dim, kv.page_size)
             and qkv.shape[1] % 8 == 0):
         return K.attention_rowwise(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table,
                                    batch.tok_seat, batch.positions, num_q_heads, num_kv_heads,
                                    head_dim, scale, window)
-    plans = batch.attention_plans
-    key = (num_q_heads, num_kv_heads, head_dim, kv.page_size)
-    plan = plans.get(key)
-    if plan is None:
-        plan = plans[key] = _plan(batch, num_q_heads // num_kv_heads, num_kv_heads, head_dim, kv.page_size)
+    plan = _plan_for(batch, kv, num_q_heads, num_kv_heads, head_dim)
     stride = qkv.shape[1]
     for launch in plan:
         if launch[0] == "wave":

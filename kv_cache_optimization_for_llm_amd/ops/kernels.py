@@ -432,6 +432,51 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
     return out
 
 
+def attention_mfma_rope_supported(head_dim: int, page_size: int, group: int) -> bool:
+    """Whether the decode attention kernel that rotates and caches inside takes this geometry
+    (``group``: query heads per kv head)."""
+    return bool(hip_lib().kva_attention_mfma_rope_supported(int(head_dim), int(page_size), int(group)))
+
+
+def attention_mfma_rope(qkv: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                        block_table: torch.Tensor, item_meta: torch.Tensor, num_q_heads: int, num_kv_heads: int,
+                        head_dim: int, scale: float, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+                        slot_mapping: Optional[torch.Tensor], window: int = 0, splits: int = 1,
+                        keys_per_split: int = 0, keep_cached: bool = False) -> torch.Tensor:
+    """bf16 matrix-core attention of decoded tokens (one token per item) straight from the joined
+    Q/K/V projection ``qkv`` ``[T, (nq + 2 nkv) d]``, not yet rotated: the kernel rotates Q and the
+    token's K by its position (``cos`` / ``sin`` ``[positions, d / 2]`` fp32, both None: no
+    rotation), stores the rotated K and the V at ``slot_mapping[token]`` (None: the cache is only
+    read) and attends, the token's own key and value taken from registers.  ``item_meta``
+    ``[items, 8]`` int32: (token row, 1, position, seat, 0, 0, 0, 0)."""
+    tokens = out.shape[0]
+    if out.dtype != torch.bfloat16 or qkv.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16:
+        raise KernelError("attention_mfma_rope: bfloat16 only")
+    if out.shape != (tokens, num_q_heads * head_dim) or qkv.dim() != 2 or qkv.shape[0] != tokens \
+            or qkv.shape[1] != (num_q_heads + 2 * num_kv_heads) * head_dim or not qkv.is_contiguous():
+        raise KernelError("attention_mfma_rope: qkv must be [T, (nq + 2 nkv) d] and out [T, nq * d]")
+    check_cache_shapes("attention_mfma_rope", k_cache, v_cache, num_kv_heads, head_dim)
+    if item_meta.dim() != 2 or item_meta.shape[1] != 8 or block_table.dim() != 2:
+        raise KernelError("attention_mfma_rope: item_meta must be [items, 8] and the block table [seats, blocks]")
+    if (cos is None) != (sin is None) or (cos is not None and (cos.shape != sin.shape or cos.dim() != 2
+                                                               or cos.shape[1] != head_dim // 2)):
+        raise KernelError("attention_mfma_rope: cos and sin tables must both be [positions, d / 2]")
+    if slot_mapping is not None and slot_mapping.shape != (tokens,):
+        raise KernelError("attention_mfma_rope: one cache slot per token")
+    part_o = part_ml = None
+    if splits > 1:
+        part_o = torch.empty((tokens * num_q_heads, splits, head_dim), dtype=torch.float32, device=out.device)
+        part_ml = torch.empty((tokens * num_q_heads, splits, 2), dtype=torch.float32, device=out.device)
+    check(hip_lib().kva_attention_mfma_rope(
+        _dev(out, "out"), _opt(part_o, "part_o"), _opt(part_ml, "part_ml"), _dev(qkv, "qkv"), qkv.shape[1],
+        _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32),
+        block_table.shape[1], _dev(item_meta, "item_meta", torch.int32), item_meta.shape[0], tokens * num_q_heads,
+        num_q_heads, num_kv_heads, head_dim, k_cache.shape[2], float(scale), int(window), int(splits),
+        int(keys_per_split), 1 if keep_cached else 0, _opt(cos, "cos", torch.float32), _opt(sin, "sin", torch.float32),
+        _opt(slot_mapping, "slot_mapping", torch.int32), _stream()), "attention_mfma_rope")
+    return out
+
+
 def attention_lds_supported(head_dim: int, page_size: int) -> bool:
     return bool(hip_lib().kva_attention_lds_supported(int(head_dim), int(page_size)))
 
@@ -562,19 +607,27 @@ class TiledWeight:
 
 
 class TiledRows:
-    """At most 16 rows of ``width`` bf16 columns laid out ``[width / 8, 16, 8]``: element (m, c)
-    at ``[c // 8, m, c % 8]``, rows past ``rows`` unwritten.  It is the order in which the lanes of
-    a few-rows product read X (four neighbouring lanes take the same 8 columns of four
-    neighbouring rows: 64 contiguous bytes instead of four pieces a row apart), so a product that
-    feeds another can leave its result like this.  ``to_rows()`` gives the plain ``[rows, width]``."""
+    """At most 64 rows of ``width`` bf16 columns laid out ``[width / 8, R, 8]`` with ``R`` the row
+    count rounded up to a multiple of 16: element (m, c) at ``[c // 8, m, c % 8]``, rows past
+    ``rows`` unwritten.  It is the order in which the lanes of a few-rows product read X (sixteen
+    neighbouring lanes take the same 8 columns of sixteen neighbouring rows: 256 contiguous bytes
+    instead of sixteen pieces a row apart), so a product that feeds another can leave its result
+    like this.  ``to_rows()`` gives the plain ``[rows, width]``."""
 
-    MAX_ROWS = 16
+    MAX_ROWS = 64
 
     def __init__(self, rows: int, width: int, device):
         if not (1 <= rows <= self.MAX_ROWS) or width % 8:
-            raise KernelError(f"TiledRows: 1..16 rows and a multiple of 8 columns, not {rows} x {width}")
+            raise KernelError(f"TiledRows: 1..{self.MAX_ROWS} rows and a multiple of 8 columns, not {rows} x {width}")
         self.rows, self.width = rows, width
-        self.data = torch.empty((width // 8, 16, 8), dtype=torch.bfloat16, device=device)
+        self.padded = (rows + 15) // 16 * 16
+        self.data = torch.empty((width // 8, self.padded, 8), dtype=torch.bfloat16, device=device)
+
+    @classmethod
+    def from_rows(cls, x: torch.Tensor) -> "TiledRows":
+        t = cls(x.shape[0], x.shape[1], x.device)
+        t.data[:, :t.rows, :] = x.view(t.rows, t.width // 8, 8).permute(1, 0, 2)
+        return t
 
     @property
     def shape(self):
@@ -589,7 +642,7 @@ class TiledRows:
         return self.data.device
 
     def to_rows(self) -> torch.Tensor:
-        return self.data.permute(1, 0, 2).reshape(16, self.width)[:self.rows].contiguous()
+        return self.data.permute(1, 0, 2).reshape(self.padded, self.width)[:self.rows].contiguous()
 
 
 def gemm_skinny(x: torch.Tensor, w: TiledWeight, out: Optional[torch.Tensor], swiglu: bool = False, *,
@@ -855,6 +908,7 @@ KERNEL_CLASSES = {
     "residual_add": "elementwise", "scale_softcap": "elementwise", "cast": "elementwise",
     "silu_mul": "activation", "rope_kv_write": "rope + cache write",
     "attention_rowwise": "attention", "attention_mfma": "attention", "attention_lds": "attention",
+    "attention_mfma_rope": "attention",
     "gemm_nt_f32": "gemm fp32", "gemm_vendor": "gemm (vendor library)",
     "gemm_skinny": "gemm (few rows)", "gemm_skinny_qkv_rope": "gemm (few rows)",
     "gemv": "gemm (few rows)", "gemv_qkv_rope": "gemm (few rows)",

@@ -18,6 +18,7 @@ from ..config.registry import MIXERS, POSITION_ENCODINGS
 from ..models.spec import PartSpec, TensorSpec
 from ..ops import attention as attn_ops
 from ..ops import kernels as K
+from ..ops.gemm_bf16 import SKINNY_MAX_ROWS
 from .base import BranchTail, KVCacheSpec, Mixer, MixerContext, NormedRows, attention_cache_spec
 from .linear import Linear
 
@@ -29,25 +30,50 @@ class EncodedQKV:
     or none) and the product followed by the encoding's own kernel, so that a mixer - this one or
     another attention variant - only says ``qkv(x, batch, kv)``."""
 
+    # Above 16 decoded tokens the library's product followed by the attention kernel that rotates and
+    # caches inside is ahead of the few-rows product with that work in its epilogue, except for large
+    # matrices at many rows.  Whole decode steps at 768 keys, ms, epilogue -> attention kernel:
+    # 1B sizes (3,072 x 2,048) 17 / 24 / 32 requests 1.188 / 1.243 / 1.292 -> 1.133 / 1.194 / 1.245;
+    # 8 layers of the 3B sizes (5,120 x 3,072) 17 / 32 / 48: 0.855 / 0.929 / 1.040 -> 0.838 / 0.927 / 1.007;
+    # 8 layers of the 8B sizes (6,144 x 4,096) 17 / 24: 1.262 / 1.298 -> 1.259 / 1.281, but 32 / 40 / 48:
+    # 1.288 / 1.386 / 1.374 -> 1.292 / 1.400 / 1.416.
+    ROTATE_LATER_ROWS = 24
+    ROTATE_LATER_ELEMENTS = 1 << 24
+
     def __init__(self, linear: Linear, position, hidden_size: int, num_heads: int, num_kv_heads: int,
                  head_dim: int):
         self.linear, self.position = linear, position
         self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim = hidden_size, num_heads, num_kv_heads, head_dim
+        self.pending_rotation = None          # set by a call that left encoding and cache write to the attention kernel
 
     def __call__(self, x, batch, kv):
         """``x`` [T, hidden] (plain or NormedRows).  Returns a tensor whose first ``nq * d`` columns
         are the position-encoded queries; K (encoded) and V of the step's tokens are in the cache
-        when ``kv`` allows writing."""
+        when ``kv`` allows writing.  Or, with ``self.pending_rotation`` set to the (cos, sin) tables
+        (or (None, None)), the joined projection as the product left it: encoding and cache write
+        are then the attention kernel's (``ops.attention.paged_attention(..., rope=...)``)."""
+        self.pending_rotation = None
         tables, rows = None, x.shape[0]
         kernel = self.linear.fused_kernel(rows, x.dtype, rotated=True)
         if kernel == Linear.GEMV and not K.gemv_qkv_rope_supported(rows, self.hidden_size, self.head_dim):
             kernel = Linear.FEW_ROWS if self.linear.tiled is not None else None
         if kernel == Linear.FEW_ROWS and not K.gemm_skinny_qkv_rope_supported(rows, self.hidden_size, self.head_dim):
             kernel = None
+        if (kernel == Linear.FEW_ROWS and rows > SKINNY_MAX_ROWS
+                and (rows <= self.ROTATE_LATER_ROWS or self.linear.weight.numel() <= self.ROTATE_LATER_ELEMENTS)
+                and attn_ops.rotates_in_kernel(batch, kv, self.num_heads, self.num_kv_heads, self.head_dim, x.dtype)):
+            kernel = None
         if kernel is not None:
             tables = self.position.rotate_half_tables(x.device, self.head_dim)
         if tables is None:
             qkv = self.linear(x)
+            # decoded tokens only: rotation and cache write go into the attention kernel, which
+            # takes the product as it is (one launch less per layer where the product is the library's)
+            later = self.position.rotate_half_tables(x.device, self.head_dim)
+            if later is not None and attn_ops.rotates_in_kernel(batch, kv, self.num_heads, self.num_kv_heads,
+                                                                self.head_dim, qkv.dtype):
+                self.pending_rotation = later
+                return qkv
             self.position.apply_and_cache(qkv, batch.positions, self.num_heads, self.num_kv_heads,
                                           self.head_dim, kv)
             return qkv
@@ -117,7 +143,7 @@ class GQAAttention(Mixer):
         qkv = self.qkv(x, batch, kv)
         out = torch.empty((x.shape[0], self.num_heads * self.head_dim), dtype=x.dtype, device=x.device)
         attn_ops.paged_attention(qkv, out, kv, batch, self.num_heads, self.num_kv_heads,
-                                 self.head_dim, self.scale, self.window)
+                                 self.head_dim, self.scale, self.window, rope=self.qkv.pending_rotation)
         if tail is not None:
             fused = self.o.into_residual(out, tail)
             if fused is not None:

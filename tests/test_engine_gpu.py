@@ -73,11 +73,16 @@ def test_greedy_generation_through_the_entry_point(name, dtype, model_dirs, gpu)
     assert llm.engine.cache.free_seats == 4
 
 
-@pytest.mark.parametrize("name, batch", [("A", 20), ("C", 40), ("D", 64)])
-def test_many_requests_decoding_together(name, batch, model_dirs, gpu):
+@pytest.mark.parametrize("name, batch", [("A", 20), ("C", 40), ("D", 64), ("E", 24), ("F", 40), ("E", 64)])
+def test_many_requests_decoding_together(name, batch, model_dirs, gpu, monkeypatch):
     """17 to 64 decoded tokens per step: the shapes of the few-rows products whose waves share X
-    through LDS, of the vendor GEMM at few rows and of decode graphs for large batches.  Every
-    pick must be the plain model's (within bf16 rounding), for every request."""
+    through LDS, of the vendor GEMM at few rows and of decode graphs for large batches; at head
+    sizes 64 and 128 (E, F) also of the attention kernel that rotates and caches the tokens' keys
+    itself.  Every pick must be the plain model's (within bf16 rounding), for every request."""
+    from kv_cache_optimization_for_llm_amd.ops import kernels as K
+    calls = []
+    inside = K.attention_mfma_rope
+    monkeypatch.setattr(K, "attention_mfma_rope", lambda *a, **k: (calls.append(1), inside(*a, **k))[1])
     cfg, W = plain.load_model_dir(model_dirs[name])
     rng = np.random.default_rng(7)
     lengths = [int(n) for n in rng.integers(1, 12, batch)]
@@ -90,6 +95,7 @@ def test_many_requests_decoding_together(name, batch, model_dirs, gpu):
         assert len(g) == 10
         check_choices(cfg, W, p, g, "bfloat16")
     assert llm.engine.graphs.replays > 0
+    assert bool(calls) == (name in "EF"), "rotation inside the attention kernel: taken where it should not be, or not where it should"
     llm.engine.cache.check()
     assert llm.engine.cache.free_seats == batch
 

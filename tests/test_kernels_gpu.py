@@ -394,6 +394,85 @@ def test_attention_never_sees_what_a_page_held_before(nq, nkv, d, page, window, 
             close(out, want, torch.bfloat16, f"attention_lds over stale pages splits={splits}", tol16=8e-3)
 
 
+@pytest.mark.parametrize("nq, nkv, d, window", [(32, 8, 64, 0), (24, 8, 128, 0), (8, 2, 64, 45), (16, 1, 64, 0), (4, 4, 128, 0)])
+@pytest.mark.parametrize("splits", [1, 3, 8])
+@pytest.mark.parametrize("rotate", [True, False])
+def test_decode_attention_that_rotates_and_caches_inside(nq, nkv, d, window, splits, rotate, gpu):
+    """Decoded tokens straight from the joined projection: the attention kernel rotates Q and the
+    new K, caches K and V and attends.  Same output and same cache contents as the rotation kernel
+    followed by the attention kernel; positions at every place of a page and of a 32-key block,
+    position 0 included; a token without a cache slot is attended to but not stored; without a
+    slot mapping (a layer call that only reads another's cache) nothing is stored and the key
+    comes from the cache."""
+    assert K.attention_mfma_rope_supported(d, 16, nq // nkv) and not K.attention_mfma_rope_supported(48, 16, 2)
+    assert not K.attention_mfma_rope_supported(64, 8, 2) and not K.attention_mfma_rope_supported(64, 16, 32)
+    page = 16
+    positions = [0, 1, 15, 16, 17, 31, 32, 33, 47, 63, 64, 100, 255, 256, 300, 511, 5]
+    T = len(positions)
+    g = torch.Generator().manual_seed(d + nq + splits)
+    max_blocks = max(positions) // page + 2
+    n_pages = T * max_blocks + 3
+    perm = torch.randperm(n_pages, generator=g).to(torch.int32)
+    table = perm[:T * max_blocks].view(T, max_blocks).contiguous()
+    kc = (torch.randn(n_pages, nkv, page, d, generator=g)).to(torch.bfloat16)
+    vc = (torch.randn(n_pages, nkv, d, page, generator=g)).to(torch.bfloat16)
+    qkv = (torch.randn(T, (nq + 2 * nkv) * d, generator=g) * 1.5).to(torch.bfloat16)
+    pos_t = torch.tensor(positions, dtype=torch.int32)
+    slots = torch.tensor([int(table[t, p // page]) * page + p % page for t, p in enumerate(positions)], dtype=torch.int32)
+    inv = plain.rope_inv_freq(d, 500000.0, None)
+    cos, sin = (torch.from_numpy(a).to(gpu) for a in plain.rope_cos_sin(range(600), inv))
+    if not rotate:
+        cos = sin = None
+    meta = torch.zeros((T, 8), dtype=torch.int32)
+    meta[:, 0], meta[:, 1], meta[:, 2], meta[:, 3] = torch.arange(T), 1, pos_t, torch.arange(T)
+    order = torch.argsort(-pos_t.long(), stable=True)                 # most keys first, as the engine orders items
+    meta = meta[order].contiguous().to(gpu)
+    scale = 1.0 / math.sqrt(d)
+    per = ((max(positions) + 1 + splits - 1) // splits + 31) // 32 * 32 if splits > 1 else 0
+    ent = order.to(torch.int32).to(gpu)
+    zeros = torch.zeros(T, dtype=torch.int32, device=gpu)
+    seat = torch.arange(T, dtype=torch.int32, device=gpu)
+    qs = torch.arange(T + 1, dtype=torch.int32, device=gpu)
+
+    def separate(slot_map):
+        k, v, x = kc.clone().to(gpu), vc.clone().to(gpu), qkv.clone().to(gpu)
+        K.rope_kv_write(x, pos_t.to(gpu), nq, nkv, d, cos, sin, k, v, slot_map.to(gpu), page)
+        out = torch.full((T, nq * d), float("nan"), dtype=torch.bfloat16, device=gpu)
+        K.attention_mfma(x, x.shape[1], out, k, v, table.to(gpu), ent, zeros, seat, qs, pos_t.to(gpu), nq, nkv, d,
+                         scale, window, splits, per, 1, False, meta)
+        return out, k, v
+
+    def fused(slot_map, k=None, v=None):
+        k = kc.clone().to(gpu) if k is None else k
+        v = vc.clone().to(gpu) if v is None else v
+        out = torch.full((T, nq * d), float("nan"), dtype=torch.bfloat16, device=gpu)
+        K.attention_mfma_rope(qkv.to(gpu), out, k, v, table.to(gpu), meta, nq, nkv, d, scale, cos, sin,
+                              None if slot_map is None else slot_map.to(gpu), window, splits, per)
+        return out, k, v
+
+    want, k_want, v_want = separate(slots)
+    got, k_got, v_got = fused(slots)
+    assert torch.equal(k_got, k_want) and torch.equal(v_got, v_want), "the cache holds other keys or values"
+    assert torch.isfinite(got.float()).all()
+    close(got, want, torch.bfloat16, "rotation and cache write inside the attention kernel", tol16=4e-3)
+    assert (got.float() - want.float()).abs().max() <= 2 ** -6 * want.float().abs().max()
+    # a token without a slot: attended to (from registers), not stored
+    some = slots.clone()
+    some[3] = some[11] = -1
+    got2, k2, v2 = fused(some)
+    assert torch.equal(got2, got)
+    kw, vw = k_want.clone(), v_want.clone()
+    for t in (3, 11):
+        pg, off = int(slots[t]) // page, int(slots[t]) % page
+        kw[pg, :, off, :] = kc[pg, :, off, :].to(gpu)
+        vw[pg, :, :, off] = vc[pg, :, :, off].to(gpu)
+    assert torch.equal(k2, kw) and torch.equal(v2, vw)
+    # no slot mapping: the cache (which already holds the tokens' keys) is only read
+    got3, k3, v3 = fused(None, k_want.clone(), v_want.clone())
+    assert torch.equal(k3, k_want) and torch.equal(v3, v_want)
+    close(got3, want, torch.bfloat16, "rotation inside, keys from the cache", tol16=4e-3)
+
+
 LONG_ENTRIES = [(0, 300), (40, 1), (200, 131), (5, 64), (0, 33)]
 
 
