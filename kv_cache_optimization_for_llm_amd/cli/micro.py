@@ -76,7 +76,7 @@ def attention(args) -> None:
     ctx = max(s + n for s, n in entries)
     blocks = (ctx + page - 1) // page
     copies = max(1, min(8, int(600e6 / (len(entries) * blocks * page * nkv * d * 4)) + 1))
-    caches = [(torch.randn(len(entries) * blocks, nkv, page, d, device=dev).bfloat16(),
+    caches = [(K.keys_to_pages(torch.randn(len(entries) * blocks, nkv, page, d, device=dev).bfloat16()),
                torch.randn(len(entries) * blocks, nkv, d, page, device=dev).bfloat16()) for _ in range(copies)]
     table = torch.arange(len(entries) * blocks, dtype=torch.int32).view(len(entries), blocks).to(dev)
     lens = [n for _, n in entries]
@@ -148,7 +148,11 @@ def gemm(args) -> None:
             calls = [lambda w=w: product(x, w, out, swiglu=True) for w in tiled]
     else:
         out = torch.empty(m, n, device=dev, dtype=torch.float32 if mode == "f32" else torch.bfloat16)
-        calls = [lambda w=w: product(x, w, out) for w in tiled]
+        if args.x_tiled:
+            xt = K.TiledRows.from_rows(x)
+            calls = [lambda w=w: product(xt, w, out, x_tiled=True) for w in tiled]
+        else:
+            calls = [lambda w=w: product(x, w, out) for w in tiled]
     us = _time_in_graph(calls, args.reps) if args.graph else _time(calls, args.reps)
     name = "matrix-vector kernel" if gemv else "few-rows kernel"
     line = f"gemm {args.shape:8s} rows {m:3d} [{n} x {k}] {name} {us:8.2f} us  {n * k * 2 / us / 1e6:6.2f} TB/s of weights"

@@ -19,6 +19,7 @@
 // This kernel serves the fp32 path and every shape (head_dim any multiple of 4 up to 256);
 // the bf16 path uses it where the MFMA kernels do not apply.
 #include "common.h"
+#include "kv_layout.h"
 #include <math.h>
 
 #define ATTN_MAX_HEAD_DIM 256
@@ -74,13 +75,13 @@ attention_rowwise_kernel(T *__restrict__ out, const T *__restrict__ q, int q_row
         long long row_off = 0;
         if (valid) {
             const int page = bt[key / page_size];
-            row_off = (((long long)page * num_kv_heads + kvh) * page_size + key % page_size) *
-                      (long long)head_dim;
-            const T *krow = k_cache + row_off;
+            row_off = ((long long)page * num_kv_heads + kvh) * page_size * (long long)head_dim;
+            const T *kpage = k_cache + row_off;
+            const int krow = key % page_size, kc = kva_k_chunk(head_dim);
             float dot = 0.f;
             for (int j = 0; j < head_dim; j += 4) {
                 float kv[4];
-                Vec4<T>::load(krow + j, kv);
+                Vec4<T>::load(kpage + kva_k_at(krow, j, page_size, kc), kv);     // (4 elements never straddle a chunk)
                 dot += q_s[j] * kv[0];
                 dot += q_s[j + 1] * kv[1];
                 dot += q_s[j + 2] * kv[2];

@@ -24,6 +24,7 @@
 // from the cache.
 #include "common.h"
 #include "attention_frag.h"
+#include "kv_layout.h"
 #include <math.h>
 #include <type_traits>
 
@@ -127,7 +128,7 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, float *__restrict__ part
         for (int dt = 0; dt < NDT; ++dt) o[rt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    // ---- copies page -> registers -> LDS.  Chunk c of the K tile is 16 bytes of key c / (D/8);
+    // ---- copies page -> registers -> LDS.  Chunk c of the K tile is 16 bytes of key c % 16 of page c / 2D, dims 8 (c % 2D) / 16 ..;
     // chunk c of the V^T tile is 8 keys of value dimension (c % 2D) / 2 in page c / 2D.  A tile
     // outside the keys the workgroup needs is redirected to the nearest needed one (its page is
     // certainly mapped); its scores are masked away.
@@ -142,9 +143,9 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, float *__restrict__ part
 #pragma unroll
     for (int i = 0; i < Geo::PER_THREAD; ++i) {
         const int c = tid + i * 256;
-        const int key = c / (D / 8), kc = c % (D / 8);
-        k_sel[i] = __builtin_amdgcn_readfirstlane(key >> 4);
-        k_off[i] = (key & 15) * D + kc * 8;
+        // K pages are [D / 8][16 keys][8] (kv_layout.h): chunk c of the tile is 16 bytes number c % 2D of page c / 2D
+        k_sel[i] = __builtin_amdgcn_readfirstlane(c / (2 * D));
+        k_off[i] = (c % (2 * D)) * 8;
         const int rem = c % (2 * D);
         v_sel[i] = __builtin_amdgcn_readfirstlane(c / (2 * D));
         v_off[i] = (rem >> 1) * 16 + (rem & 1) * 8;
@@ -173,7 +174,7 @@ attention_lds_item(char *lds, bf16_t *__restrict__ out, float *__restrict__ part
         auto chunk = [&](int i, const uint4 &k, const uint4 &v) {
             const int c = tid + i * 256;
             if (Geo::CHUNKS % 256 == 0 || c < Geo::CHUNKS) {
-                const int key = c / (D / 8), kc = c % (D / 8);
+                const int key = (c / (2 * D)) * 16 + (c & 15), kc = (c % (2 * D)) >> 4;     // the page's chunk order: [dim / 8][key]
                 *reinterpret_cast<uint4 *>(buf + key * Geo::KROW + kc * 16) = k;
                 const int t = c / (2 * D), rem = c % (2 * D);
                 // rows of 72 bytes: 18 banks apart, so that the 16 lanes of an 8-byte operand read (rows r = 0..15

@@ -17,7 +17,7 @@
 // (lane group g, element j <-> key (j / 4) * 16 + 4 g + j % 4); it is applied to V^T's loads,
 // which is free because V pages are stored transposed ([kv_head, head_dim, page_size]) and a
 // lane's 4 keys are 8 contiguous bytes.  K is loaded straight from the page
-// ([kv_head, page_size, head_dim]) in operand layout too, so there is no LDS and no barrier.
+// ([kv_head, head_dim / 8, page_size, 8], kv_layout.h) in operand layout too, so there is no LDS and no barrier.
 // Operand registers are double-buffered: the loads of block i+1 are issued before block i is
 // computed.  With pages of 16 keys or a multiple, a 16-key tile lies in one page and the
 // block-table lookup is uniform over the wavefront.
@@ -34,6 +34,7 @@
 // kernel base/src/kernels.cu:361-466, which work one key at a time on CUDA cores.
 #include "common.h"
 #include "attention_frag.h"
+#include "kv_layout.h"
 #include <type_traits>
 #include <math.h>
 
@@ -219,7 +220,7 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
                 if (r == off) {
     #pragma unroll
                     for (int ks = 0; ks < NKS; ++ks)
-                        *reinterpret_cast<uint4 *>(const_cast<bf16_t *>(k_cache) + page_elems + (size_t)(slot & 15) * D + ks * 32 + g * 8) = k_new[ks].u4;
+                        *reinterpret_cast<uint4 *>(const_cast<bf16_t *>(k_cache) + page_elems + kva_k_at(slot & 15, ks * 32 + g * 8, 16, 8)) = k_new[ks].u4;
                 }
                 if (g == 0) {
     #pragma unroll
@@ -253,7 +254,11 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
     // unconditional: a tile outside the keys the item needs is redirected to the nearest needed
     // tile (whose page is certainly mapped) and its scores are masked away.
     const int lo_tile = item_lo & ~15, hi_tile = item_hi & ~15;
-    const uint32_t k_lane = (uint32_t)(r * D + g * (KSTEP / 4)) * 2u;          // bytes
+    // K pages are [D / 8][16 keys][8] (kv_layout.h): a lane's 16 bytes (8 with head-dim slices of 16)
+    // of key r are chunk (dim / 8) of that key, and a wavefront's load is one run of neighbouring bytes
+    const uint32_t k_lane = KSTEP == 32 ? (uint32_t)(g * 16 + r) * 16u
+                                        : (uint32_t)((g >> 1) * 16 + r) * 16u + (uint32_t)(g & 1) * 8u;   // bytes
+    constexpr uint32_t k_slice = KSTEP == 32 ? 4u * 256u : 2u * 256u;          // bytes from one head-dim slice to the next
     const uint32_t v_lane = (uint32_t)(r * 16 + 4 * g) * 2u;                   // bytes
     constexpr uint32_t v_tile_stride = 16u * 16u * 2u;                         // 16 value dims
     // STREAM: keys and values go past the caches (non-temporal loads).  Right for decoded tokens
@@ -281,11 +286,11 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
 #pragma unroll
                 for (int ks = 0; ks < NKS; ++ks) {
                     if (KSTEP == 32)
-                        f.k8[t][ks].u4 = STREAM ? load_streamed_u4(kb + k_lane + ks * 64)
-                                                : *reinterpret_cast<const uint4 *>(kb + k_lane + ks * 64);
+                        f.k8[t][ks].u4 = STREAM ? load_streamed_u4(kb + k_lane + ks * k_slice)
+                                                : *reinterpret_cast<const uint4 *>(kb + k_lane + ks * k_slice);
                     else
-                        f.k4[t][ks].u2 = STREAM ? load_streamed_u2(kb + k_lane + ks * 32)
-                                                : *reinterpret_cast<const uint2 *>(kb + k_lane + ks * 32);
+                        f.k4[t][ks].u2 = STREAM ? load_streamed_u2(kb + k_lane + ks * k_slice)
+                                                : *reinterpret_cast<const uint2 *>(kb + k_lane + ks * k_slice);
                 }
 #pragma unroll
                 for (int dt = 0; dt < NDT; ++dt)
@@ -302,19 +307,21 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
             const int key = tile0 + r, key0 = tile0 + 4 * g;
             const bool kvalid = key <= item_hi && key >= item_lo;       // pages outside may be unmapped
             const bool vvalid = key0 <= item_hi && key0 + 3 >= item_lo;
-            if (kvalid)
-                krow += (((size_t)bt[key / page_size] * num_kv_heads + kvh) * page_size +
-                         key % page_size) * D;
+            int krow_in_page = 0;
+            if (kvalid) {
+                krow += ((size_t)bt[key / page_size] * num_kv_heads + kvh) * page_size * D;     // the page of this kv head
+                krow_in_page = key % page_size;
+            }
             if (vvalid)
                 vbase = ((size_t)bt[key0 / page_size] * num_kv_heads + kvh) * D * page_size +
                         key0 % page_size;
 #pragma unroll
             for (int ks = 0; ks < NKS; ++ks) {
                 if (KSTEP == 32)
-                    f.k8[t][ks].u4 = kvalid ? *reinterpret_cast<const uint4 *>(krow + ks * 32 + g * 8)
+                    f.k8[t][ks].u4 = kvalid ? *reinterpret_cast<const uint4 *>(krow + kva_k_at(krow_in_page, ks * 32 + g * 8, page_size, 8))
                                             : make_uint4(0, 0, 0, 0);
                 else
-                    f.k4[t][ks].u2 = kvalid ? *reinterpret_cast<const uint2 *>(krow + ks * 16 + g * 4)
+                    f.k4[t][ks].u2 = kvalid ? *reinterpret_cast<const uint2 *>(krow + kva_k_at(krow_in_page, ks * 16 + g * 4, page_size, 8))
                                             : make_uint2(0, 0);
             }
 #pragma unroll

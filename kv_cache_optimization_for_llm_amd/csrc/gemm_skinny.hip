@@ -47,6 +47,7 @@
 //               to its place: Q to a [M, nq*d] buffer, K and V to the token's slot of the paged
 //               cache (reference scatterKVPackedKernel, paged_attention/src/kernels.cu:335-363).
 #include "common.h"
+#include "kv_layout.h"
 #include <math.h>
 #include <type_traits>
 
@@ -80,7 +81,7 @@ struct SkinnyArgs {
     const float *cos_t, *sin_t;   // [positions, head_dim / 2], both null: no rotation
     const int *positions;         // [M]
     const int *slots;             // [M] cache slot per token (negative: no write), null: no cache write
-    bf16_t *k_cache, *v_cache;    // [pages, nkv, page, d] and [pages, nkv, d, page]
+    bf16_t *k_cache, *v_cache;    // [pages, nkv, d / 8, page, 8] (kv_layout.h) and [pages, nkv, d, page]
     int nq, nkv, head_dim, page_size;
     // half tiles: a tile group takes 8 of its tiles' 16 rows (see choose_half_tiles)
     int half;
@@ -555,17 +556,21 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
 #pragma unroll
                     for (int i = 0; i < 4; ++i) { o1[i] = va[i]; o2[i] = vb[i]; }
                 }
-                bf16_t *dst;
+                bf16_t *dst, *dst2;
                 if (rope_head < a.nq) {
                     dst = reinterpret_cast<bf16_t *>(a.Y) + (size_t)m * a.ldy + (size_t)rope_head * D + f;
+                    dst2 = dst + D / 2;
                 } else {
                     if (slot < 0) continue;
-                    dst = a.k_cache + (((size_t)page * a.nkv + (rope_head - a.nq)) * a.page_size + off) * D + f;
+                    // (f is a multiple of 4 and D of 32: four neighbouring features lie inside one chunk of 8)
+                    bf16_t *pg = a.k_cache + ((size_t)page * a.nkv + (rope_head - a.nq)) * a.page_size * D;
+                    dst = pg + kva_k_at(off, f, a.page_size, 8);
+                    dst2 = pg + kva_k_at(off, f + D / 2, a.page_size, 8);
                 }
                 *reinterpret_cast<uint2 *>(dst) =
                     make_uint2((uint32_t)float_to_bf16_bits(o1[0]) | ((uint32_t)float_to_bf16_bits(o1[1]) << 16),
                                (uint32_t)float_to_bf16_bits(o1[2]) | ((uint32_t)float_to_bf16_bits(o1[3]) << 16));
-                *reinterpret_cast<uint2 *>(dst + D / 2) =
+                *reinterpret_cast<uint2 *>(dst2) =
                     make_uint2((uint32_t)float_to_bf16_bits(o2[0]) | ((uint32_t)float_to_bf16_bits(o2[1]) << 16),
                                (uint32_t)float_to_bf16_bits(o2[2]) | ((uint32_t)float_to_bf16_bits(o2[3]) << 16));
             } else {

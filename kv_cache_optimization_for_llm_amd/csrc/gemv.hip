@@ -19,6 +19,7 @@
 // both halves); residual add + preparation of the next norm; rotate-half rotation + cache write for
 // the joined Q/K/V matrix (a wavefront takes rows j and j + d/2 of a head).
 #include "common.h"
+#include "kv_layout.h"
 
 #include <algorithm>
 
@@ -299,11 +300,16 @@ __global__ void __launch_bounds__(64 * GV_WAVES) gemv_kernel(const GemvArgs a) {
                         o1 = va * e0 - vb * e1;
                         o2 = va * e1 + vb * e0;
                     }
-                    bf16_t *dst = head < a.nq
-                        ? reinterpret_cast<bf16_t *>(a.Y) + (size_t)my_m * a.ldy + (size_t)head * D + f
-                        : a.k_cache + (((size_t)page * a.nkv + (head - a.nq)) * a.page_size + off) * D + f;
-                    dst[0].bits = float_to_bf16_bits(o1);
-                    dst[D / 2].bits = float_to_bf16_bits(o2);
+                    if (head < a.nq) {
+                        bf16_t *dst = reinterpret_cast<bf16_t *>(a.Y) + (size_t)my_m * a.ldy + (size_t)head * D + f;
+                        dst[0].bits = float_to_bf16_bits(o1);
+                        dst[D / 2].bits = float_to_bf16_bits(o2);
+                    } else {
+                        bf16_t *pg = a.k_cache + ((size_t)page * a.nkv + (head - a.nq)) * a.page_size * D;
+                        const int kc = kva_k_chunk(D);
+                        pg[kva_k_at(off, f, a.page_size, kc)].bits = float_to_bf16_bits(o1);
+                        pg[kva_k_at(off, f + D / 2, a.page_size, kc)].bits = float_to_bf16_bits(o2);
+                    }
                 } else {
                     bf16_t *dst = a.v_cache + (((size_t)page * a.nkv + (head - a.nq - a.nkv)) * D + f) * a.page_size + off;
                     dst[0].bits = float_to_bf16_bits(va);

@@ -9,12 +9,14 @@
 // cos and sin come from fp32 tables [max_positions, rot/2] built once on the host.
 // K is rotated BEFORE it is cached, V is cached as it is.
 //
-// Cache layout: K is [num_pages, num_kv_heads, page_size, head_dim]; V is stored transposed
+// Cache layout: K is [num_pages, num_kv_heads, head_dim / 8, page_size, 8] (kv_layout.h: a key's
+// elements in chunks of 8, the chunks of all keys of a page next to each other); V is stored transposed
 // inside a page, [num_pages, num_kv_heads, head_dim, page_size], so that the attention kernels
 // can load "several keys of one value dimension" as one vector (the matrix-core operand layout
 // of P*V).  Slot s of the slot mapping is page s / page_size, row s % page_size.  A negative
 // slot skips the write.
 #include "common.h"
+#include "kv_layout.h"
 
 template <typename T>
 __global__ void rope_kv_write_kernel(T *__restrict__ qkv, T *__restrict__ k_cache,
@@ -71,9 +73,10 @@ __global__ void rope_kv_write_kernel(T *__restrict__ qkv, T *__restrict__ k_cach
             h[i2] = r2;
         } else if (slot >= 0) {
             const int kvh = head - num_q_heads;
-            T *dst = k_cache + (((size_t)page * num_kv_heads + kvh) * page_size + off) * head_dim;
-            dst[i1] = r1;
-            dst[i2] = r2;
+            T *dst = k_cache + ((size_t)page * num_kv_heads + kvh) * page_size * head_dim;
+            const int kc = kva_k_chunk(head_dim);
+            dst[kva_k_at(off, i1, page_size, kc)] = r1;
+            dst[kva_k_at(off, i2, page_size, kc)] = r2;
         }
     }
     if (slot >= 0) {
@@ -139,11 +142,15 @@ __global__ void rope_kv_write_vec_kernel(bf16_t *__restrict__ qkv, bf16_t *__res
             o1[j] = x1[j] * c[j] - x2[j] * s[j];
             o2[j] = x1[j] * s[j] + x2[j] * c[j];
         }
-        bf16_t *dst = h;
-        if (head >= num_q_heads)
-            dst = k_cache + (((size_t)page * num_kv_heads + (head - num_q_heads)) * page_size + off) * head_dim;
-        *reinterpret_cast<uint4 *>(dst + p0) = rk_pack8(o1);
-        *reinterpret_cast<uint4 *>(dst + half + p0) = rk_pack8(o2);
+        if (head >= num_q_heads) {
+            // (head_dim is a multiple of 16 here: p0 and half + p0 are whole chunks of 8)
+            bf16_t *dst = k_cache + ((size_t)page * num_kv_heads + (head - num_q_heads)) * page_size * head_dim;
+            *reinterpret_cast<uint4 *>(dst + kva_k_at(off, p0, page_size, 8)) = rk_pack8(o1);
+            *reinterpret_cast<uint4 *>(dst + kva_k_at(off, half + p0, page_size, 8)) = rk_pack8(o2);
+        } else {
+            *reinterpret_cast<uint4 *>(h + p0) = rk_pack8(o1);
+            *reinterpret_cast<uint4 *>(h + half + p0) = rk_pack8(o2);
+        }
     }
     if (slot >= 0) {
         const bf16_t *v = row + (size_t)(num_q_heads + num_kv_heads) * head_dim;

@@ -53,17 +53,45 @@ def _opt(t: Optional[torch.Tensor], name: str, dtype: Optional[torch.dtype] = No
     return None if t is None else _dev(t, name, dtype)
 
 
+def k_chunk(head_dim: int) -> int:
+    """Elements of a key that lie next to each other inside a K page (``csrc/kv_layout.h``)."""
+    return 4 if head_dim % 8 else 8
+
+
+def k_page_shape(num_kv_heads: int, head_dim: int) -> tuple:
+    """Per-token shape of the K cache array: a key as ``head_dim / C`` chunks of ``C`` elements; the
+    page's token axis lies between the two (``[kv_heads, head_dim / C, page_size, C]``)."""
+    c = k_chunk(head_dim)
+    return (num_kv_heads, head_dim // c, c)
+
+
+def keys_to_pages(k: torch.Tensor) -> torch.Tensor:
+    """Keys ``[..., page_size, head_dim]`` (row by row) in the cache's layout
+    ``[..., head_dim / C, page_size, C]``."""
+    *lead, page, d = k.shape
+    c = k_chunk(d)
+    return k.reshape(*lead, page, d // c, c).transpose(-3, -2).contiguous()
+
+
+def pages_to_keys(k: torch.Tensor) -> torch.Tensor:
+    """The inverse of :func:`keys_to_pages`: ``[..., head_dim / C, page_size, C]`` to ``[..., page_size, head_dim]``."""
+    *lead, chunks, page, c = k.shape
+    return k.transpose(-3, -2).reshape(*lead, page, chunks * c)
+
+
 def check_cache_shapes(what: str, k_cache: torch.Tensor, v_cache: torch.Tensor, num_kv_heads: int,
-                       head_dim: int) -> None:
-    """K pages are [kv_heads, page_size, head_dim]; V pages are transposed, [kv_heads, head_dim,
-    page_size]."""
-    if k_cache.dim() != 4 or v_cache.dim() != 4:
-        raise KernelError(f"{what}: cache arrays must be 4-D")
-    pages, nkv, ps, d = k_cache.shape
-    if (nkv, d) != (num_kv_heads, head_dim) or tuple(v_cache.shape) != (pages, nkv, d, ps):
+                       head_dim: int) -> int:
+    """K pages are [kv_heads, head_dim / C, page_size, C] (a key in chunks of C = 8 elements, the chunks
+    of a page's keys next to each other: ``csrc/kv_layout.h``); V pages are transposed, [kv_heads,
+    head_dim, page_size].  Returns the page size."""
+    if k_cache.dim() != 5 or v_cache.dim() != 4:
+        raise KernelError(f"{what}: the K cache must be 5-D and the V cache 4-D")
+    pages, nkv, chunks, ps, c = k_cache.shape
+    if (nkv, chunks, c) != k_page_shape(num_kv_heads, head_dim) or tuple(v_cache.shape) != (pages, nkv, head_dim, ps):
         raise KernelError(f"{what}: K cache {tuple(k_cache.shape)} / V cache {tuple(v_cache.shape)} are "
-                          f"not [pages, {num_kv_heads}, page, {head_dim}] / [pages, {num_kv_heads}, "
-                          f"{head_dim}, page]")
+                          f"not [pages, {num_kv_heads}, {head_dim} / C, page, C] / [pages, {num_kv_heads}, "
+                          f"{head_dim}, page] with C = {k_chunk(head_dim)}")
+    return int(ps)
 
 
 # --------------------------------------------------------------------------------------
@@ -251,8 +279,8 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, num_q_heads: int, 
         if v_cache is None or slot_mapping is None:
             raise KernelError("rope_kv_write: K and V cache and a slot mapping are all needed")
         check_cache_shapes("rope_kv_write", k_cache, v_cache, num_kv_heads, head_dim)
-        if k_cache.shape[2] != page_size:
-            raise KernelError(f"rope_kv_write: cache pages hold {k_cache.shape[2]} tokens, not {page_size}")
+        if k_cache.shape[3] != page_size:
+            raise KernelError(f"rope_kv_write: cache pages hold {k_cache.shape[3]} tokens, not {page_size}")
         if k_cache.dtype != qkv.dtype or slot_mapping.shape != (tokens,):
             raise KernelError("rope_kv_write: cache dtype or slot mapping shape does not fit")
     check(hip_lib().kva_rope_kv_write(
@@ -279,7 +307,7 @@ def attention_rowwise(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_c
         raise KernelError("attention: q, cache and out must share a dtype")
     if q.data_ptr() % 16 or q_row_stride < num_q_heads * head_dim:
         raise KernelError("attention: q view is misaligned or its stride is too small")
-    page_size = k_cache.shape[2]
+    page_size = k_cache.shape[3]
     check(hip_lib().kva_attention_rowwise(
         _dev(out, "out"), _dev(q, "q", contiguous=False), q_row_stride, _dev(k_cache, "k_cache"),
         _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32), block_table.shape[1],
@@ -426,7 +454,7 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
         _dev(item_entry, "item_entry", torch.int32), _dev(item_row0, "item_row0", torch.int32), n_items,
         int(row_tiles), _dev(entry_seat, "entry_seat", torch.int32), _dev(entry_q_start, "entry_q_start", torch.int32),
         _dev(entry_start_pos, "entry_start_pos", torch.int32), tokens * num_q_heads, num_q_heads,
-        num_kv_heads, head_dim, k_cache.shape[2], float(scale), int(window), int(splits),
+        num_kv_heads, head_dim, k_cache.shape[3], float(scale), int(window), int(splits),
         int(keys_per_split), 1 if pair else 0, 1 if covers_all_rows else 0, 1 if keep_cached else 0,
         _stream()), "attention_mfma")
     return out
@@ -471,7 +499,7 @@ def attention_mfma_rope(qkv: torch.Tensor, out: torch.Tensor, k_cache: torch.Ten
         _dev(out, "out"), _opt(part_o, "part_o"), _opt(part_ml, "part_ml"), _dev(qkv, "qkv"), qkv.shape[1],
         _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32),
         block_table.shape[1], _dev(item_meta, "item_meta", torch.int32), item_meta.shape[0], tokens * num_q_heads,
-        num_q_heads, num_kv_heads, head_dim, k_cache.shape[2], float(scale), int(window), int(splits),
+        num_q_heads, num_kv_heads, head_dim, k_cache.shape[3], float(scale), int(window), int(splits),
         int(keys_per_split), 1 if keep_cached else 0, _opt(cos, "cos", torch.float32), _opt(sin, "sin", torch.float32),
         _opt(slot_mapping, "slot_mapping", torch.int32), _stream()), "attention_mfma_rope")
     return out
@@ -512,7 +540,7 @@ def attention_lds(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cache
         _dev(q, "q", contiguous=False), q_row_stride, _dev(k_cache, "k_cache"),
         _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32), block_table.shape[1],
         _dev(item_meta, "item_meta", torch.int32), item_meta.shape[0], 1 if pair else 0, num_q_heads,
-        num_kv_heads, head_dim, k_cache.shape[2], float(scale), int(window), int(splits), int(keys_per_split),
+        num_kv_heads, head_dim, k_cache.shape[3], float(scale), int(window), int(splits), int(keys_per_split),
         tokens * num_q_heads, 1 if covers_all_rows else 0, _stream()), "attention_lds")
     return out
 
@@ -773,7 +801,7 @@ def gemm_skinny_qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, n
         if v_cache is None or slot_mapping is None or slot_mapping.shape != (m,):
             raise KernelError("gemm_skinny_qkv_rope: K and V cache and one slot per row are all needed")
         check_cache_shapes("gemm_skinny_qkv_rope", k_cache, v_cache, num_kv_heads, head_dim)
-        if k_cache.shape[2] != page_size or k_cache.dtype != torch.bfloat16:
+        if k_cache.shape[3] != page_size or k_cache.dtype != torch.bfloat16:
             raise KernelError("gemm_skinny_qkv_rope: cache page size or dtype does not fit")
     check(hip_lib().kva_gemm_skinny_qkv_rope(
         _dev(q_out, "q_out"), q_out.shape[1], _dev(x, "x"), _dev(w.data, "w"), m, k, k, num_q_heads,
@@ -873,7 +901,7 @@ def gemv_qkv_rope(x: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, num_q_h
         if v_cache is None or slot_mapping is None or slot_mapping.shape != (m,):
             raise KernelError("gemv_qkv_rope: K and V cache and one slot per row are all needed")
         check_cache_shapes("gemv_qkv_rope", k_cache, v_cache, num_kv_heads, head_dim)
-        if k_cache.shape[2] != page_size or k_cache.dtype != torch.bfloat16:
+        if k_cache.shape[3] != page_size or k_cache.dtype != torch.bfloat16:
             raise KernelError("gemv_qkv_rope: cache page size or dtype does not fit")
     check(hip_lib().kva_gemv_qkv_rope(
         _dev(q_out, "q_out"), q_out.shape[1], _dev(x, "x"), _dev(w, "w"), m, k, x.stride(0), num_q_heads,

@@ -91,10 +91,13 @@ class KVCacheSpec:
 
 def attention_cache_spec(num_kv_heads: int, head_dim: int, kind: str = "full", window: int = 0) -> KVCacheSpec:
     """Keys and values of ``num_kv_heads`` heads of ``head_dim``, as the attention kernels here
-    read them: K pages ``[kv_heads, page_size, head_dim]``, V pages transposed
+    read them: K pages ``[kv_heads, head_dim / C, page_size, C]`` (a key in chunks of C = 8
+    elements, 4 where the head size is no multiple of 8; the chunks of a page's keys next to each
+    other, so that a wavefront's matrix-core operand is one run of bytes), V pages transposed
     ``[kv_heads, head_dim, page_size]``."""
-    heads = (int(num_kv_heads), int(head_dim))
-    return KVCacheSpec((CacheArray("k", heads, token_axis=1), CacheArray("v", heads, token_axis=2)), kind, window)
+    chunk = 4 if head_dim % 8 else 8
+    return KVCacheSpec((CacheArray("k", (int(num_kv_heads), int(head_dim) // chunk, chunk), token_axis=2),
+                        CacheArray("v", (int(num_kv_heads), int(head_dim)), token_axis=2)), kind, window)
 
 
 @dataclass(frozen=True)

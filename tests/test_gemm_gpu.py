@@ -170,7 +170,7 @@ def test_qkv_product_rotates_and_writes_the_cache(m, nq, nkv, d, page, k, rotate
         c, s = plain.rope_cos_sin(pos, inv)
         q_want = plain.apply_rope(q_want, c, s)
         k_want = plain.apply_rope(k_want, c, s)
-    k_cache = torch.zeros(pages, nkv, page, d, dtype=torch.bfloat16, device=gpu)
+    k_cache = K.keys_to_pages(torch.zeros(pages, nkv, page, d, dtype=torch.bfloat16, device=gpu))
     v_cache = torch.zeros(pages, nkv, d, page, dtype=torch.bfloat16, device=gpu)
     q = torch.full((m, nq * d), float("nan"), dtype=torch.bfloat16, device=gpu)
     assert K.gemm_skinny_qkv_rope_supported(m, k, d)
@@ -181,7 +181,7 @@ def test_qkv_product_rotates_and_writes_the_cache(m, nq, nkv, d, page, k, rotate
                            k_cache, v_cache, slots.to(gpu), page, **extra)
     scale = y.abs().max()
     assert (q.float().cpu().view(m, nq, d) - q_want).abs().max() <= 1e-2 * scale
-    kc, vc = k_cache.float().cpu(), v_cache.float().cpu()
+    kc, vc = K.pages_to_keys(k_cache).float().cpu(), v_cache.float().cpu()
     for t in range(m):
         sl = int(slots[t])
         if sl < 0:
@@ -268,11 +268,11 @@ def test_partial_products_over_ranges_of_k_add_up_to_the_product(m, n, k, gpu):
         K.gemm_skinny_partials(x[:16].contiguous().to(gpu), K.TiledWeight(w.to(gpu)))
 
 
-@pytest.mark.parametrize("m", [1, 7, 16])
+@pytest.mark.parametrize("m", [1, 7, 16, 40, 64])
 @pytest.mark.parametrize("inter, hidden", [(8192, 2048), (256, 96), (96, 64)])
 def test_activations_pass_between_two_products_in_lane_order(m, inter, hidden, gpu):
-    """The gated product can leave its result as TiledRows ([columns / 8][16 rows][8]) and the
-    residual product can read its X in that layout: bit for bit what the row-major route gives."""
+    """The gated product can leave its result as TiledRows ([columns / 8][rows rounded up to 16][8])
+    and the residual product can read its X in that layout: bit for bit what the row-major route gives."""
     x = rnd(m, hidden).to(gpu)
     w_gu = K.TiledWeight(rnd(2 * inter, hidden, scale=0.2, seed=5).to(gpu), halves=2)
     w_down = K.TiledWeight(rnd(hidden, inter, scale=0.05, seed=6).to(gpu))
@@ -294,7 +294,7 @@ def test_activations_pass_between_two_products_in_lane_order(m, inter, hidden, g
     for u, v in zip(*results):
         assert torch.equal(u, v)
     with pytest.raises(K.KernelError):
-        K.TiledRows(17, 64, gpu)
+        K.TiledRows(65, 64, gpu)
 
 
 def test_vendor_product_keeps_the_fastest_algorithm_and_the_same_result(gpu):

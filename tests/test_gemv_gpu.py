@@ -156,14 +156,14 @@ def test_qkv_product_rotates_and_writes_the_cache(m, nq, nkv, d, page, k, rotate
         sl = slots.clone()
         if some_unwritten:
             sl[m - 1] = -1                          # a token whose keys are not kept
-        k_cache = torch.zeros(pages, nkv, page, d, dtype=torch.bfloat16, device=gpu)
+        k_cache = K.keys_to_pages(torch.zeros(pages, nkv, page, d, dtype=torch.bfloat16, device=gpu))
         v_cache = torch.zeros(pages, nkv, d, page, dtype=torch.bfloat16, device=gpu)
         q = torch.full((m, nq * d), float("nan"), dtype=torch.bfloat16, device=gpu)
         K.gemv_qkv_rope(x.to(gpu), w.to(gpu), q, nq, nkv, d, positions, *tables, k_cache, v_cache, sl.to(gpu), page,
                         **extra)
         scale = y.abs().max()
         assert (q.float().cpu().view(m, nq, d) - q_want).abs().max() <= 1e-2 * scale
-        kc, vc = k_cache.float().cpu(), v_cache.float().cpu()
+        kc, vc = K.pages_to_keys(k_cache).float().cpu(), v_cache.float().cpu()
         for t in range(m):
             s_ = int(sl[t])
             if s_ < 0:

@@ -197,7 +197,7 @@ def test_rope_and_cache_write(dtype, nq, nkv, d, rot, page, gpu):
     inv = plain.rope_inv_freq(rot, 20000.0, dict(rope_type="llama3", factor=4.0, low_freq_factor=1.0,
                                                  high_freq_factor=2.0, original_max_position_embeddings=64))
     cos, sin = plain.rope_cos_sin(range(400), inv)
-    k_cache = torch.zeros(pages, nkv, page, d, dtype=dt, device=gpu)
+    k_cache = K.keys_to_pages(torch.zeros(pages, nkv, page, d, dtype=dt, device=gpu))
     v_cache = torch.zeros(pages, nkv, d, page, dtype=dt, device=gpu)
     x = qkv.clone().to(gpu)
     K.rope_kv_write(x, torch.tensor(pos, dtype=torch.int32, device=gpu), nq, nkv, d,
@@ -209,7 +209,7 @@ def test_rope_and_cache_write(dtype, nq, nkv, d, rot, page, gpu):
     v_want = f[:, (nq + nkv) * d:].view(T, nkv, d)
     close(x[:, :nq * d].view(T, nq, d), q_want, dt, "rope q", tol16=5e-3)
     assert torch.equal(x[:, nq * d:].cpu(), qkv[:, nq * d:])       # K and V columns are not touched
-    kc, vc = k_cache.float().cpu(), v_cache.float().cpu()
+    kc, vc = K.pages_to_keys(k_cache).float().cpu(), v_cache.float().cpu()
     for t in range(T):
         s = int(slots[t])
         if s < 0:
@@ -270,7 +270,7 @@ def attention_case(dtype, nq, nkv, d, page, window, entries, seed, gpu, stale=0.
     q_start = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
     tok_seat = np.repeat(np.asarray(seats, dtype=np.int32), lens)
     tok_pos = np.concatenate([np.arange(s, s + n, dtype=np.int32) for s, n in entries])
-    dev = dict(qkv=qkv.to(dt).to(gpu), kc=kc.to(dt).to(gpu), vc=vc.to(dt).to(gpu), table=table.to(gpu),
+    dev = dict(qkv=qkv.to(dt).to(gpu), kc=K.keys_to_pages(kc.to(dt)).to(gpu), vc=vc.to(dt).to(gpu), table=table.to(gpu),
                tok_seat=torch.from_numpy(tok_seat).to(gpu), tok_pos=torch.from_numpy(tok_pos).to(gpu),
                entry_seat=torch.tensor(seats, dtype=torch.int32, device=gpu),
                q_start=torch.from_numpy(q_start).to(gpu),
@@ -435,7 +435,7 @@ def test_decode_attention_that_rotates_and_caches_inside(nq, nkv, d, window, spl
     qs = torch.arange(T + 1, dtype=torch.int32, device=gpu)
 
     def separate(slot_map):
-        k, v, x = kc.clone().to(gpu), vc.clone().to(gpu), qkv.clone().to(gpu)
+        k, v, x = K.keys_to_pages(kc).to(gpu), vc.clone().to(gpu), qkv.clone().to(gpu)
         K.rope_kv_write(x, pos_t.to(gpu), nq, nkv, d, cos, sin, k, v, slot_map.to(gpu), page)
         out = torch.full((T, nq * d), float("nan"), dtype=torch.bfloat16, device=gpu)
         K.attention_mfma(x, x.shape[1], out, k, v, table.to(gpu), ent, zeros, seat, qs, pos_t.to(gpu), nq, nkv, d,
@@ -443,7 +443,7 @@ def test_decode_attention_that_rotates_and_caches_inside(nq, nkv, d, window, spl
         return out, k, v
 
     def fused(slot_map, k=None, v=None):
-        k = kc.clone().to(gpu) if k is None else k
+        k = K.keys_to_pages(kc).to(gpu) if k is None else k
         v = vc.clone().to(gpu) if v is None else v
         out = torch.full((T, nq * d), float("nan"), dtype=torch.bfloat16, device=gpu)
         K.attention_mfma_rope(qkv.to(gpu), out, k, v, table.to(gpu), meta, nq, nkv, d, scale, cos, sin,
@@ -461,12 +461,12 @@ def test_decode_attention_that_rotates_and_caches_inside(nq, nkv, d, window, spl
     some[3] = some[11] = -1
     got2, k2, v2 = fused(some)
     assert torch.equal(got2, got)
-    kw, vw = k_want.clone(), v_want.clone()
+    kw, vw = K.pages_to_keys(k_want).clone(), v_want.clone()
     for t in (3, 11):
         pg, off = int(slots[t]) // page, int(slots[t]) % page
         kw[pg, :, off, :] = kc[pg, :, off, :].to(gpu)
         vw[pg, :, :, off] = vc[pg, :, :, off].to(gpu)
-    assert torch.equal(k2, kw) and torch.equal(v2, vw)
+    assert torch.equal(K.pages_to_keys(k2), kw) and torch.equal(v2, vw)
     # no slot mapping: the cache (which already holds the tokens' keys) is only read
     got3, k3, v3 = fused(None, k_want.clone(), v_want.clone())
     assert torch.equal(k3, k_want) and torch.equal(v3, v_want)
@@ -537,6 +537,7 @@ def test_attention_with_scores_that_keep_rising_or_falling(slope, gpu):
     for t in range(ctx):
         kc[t // page, :, t % page, :] = k[t]
         vc[t // page, :, :, t % page] = v[t]
+    kc = K.keys_to_pages(kc)
     table = torch.arange(pages, dtype=torch.int32).view(1, pages).to(gpu)
     i32 = lambda *x: torch.tensor(x, dtype=torch.int32, device=gpu)
     for splits, per in ((1, 0), (4, 160)):
@@ -567,6 +568,7 @@ def test_attention_finds_one_far_key_among_hundreds(gpu):
             for p in range(ctx):
                 kc[p // page, :, p % page] = k[p]
                 vc[p // page, :, :, p % page] = v[p]
+            kc = K.keys_to_pages(kc)
             table = torch.arange(pages, dtype=torch.int32)[None].to(gpu)
             qkv = torch.zeros(1, (nq + 2) * d)
             qkv[0, :nq * d] = q.reshape(-1)
@@ -616,6 +618,7 @@ def test_attention_of_one_decoded_token_over_a_very_long_context(nkv, ctx, gpu):
     vc = torch.empty(pages, nkv, d, page, dtype=torch.bfloat16)
     kc[perm] = k.view(pages, page, nkv, d).permute(0, 2, 1, 3)
     vc[perm] = v.view(pages, page, nkv, d).permute(0, 2, 3, 1)
+    kc = K.keys_to_pages(kc)
     # the last row of plain causal attention, written out for one query (the plain function
     # computes every row: 131,072 squared is too much)
     want = torch.empty(nq, d)

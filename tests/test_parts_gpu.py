@@ -122,7 +122,7 @@ def test_attention_part_whole_and_in_portions(dtype, nq, nkv, d, page, gpu):
     pos = PartSpec("rotary", dict(head_dim=d, max_positions=128, theta=50000.0, **LLAMA3))
     part = GQAAttention("a.", hidden_size=H, num_heads=nq, num_kv_heads=nkv, head_dim=d,
                         scale=1 / math.sqrt(d), position=pos)
-    assert part.kv_cache_spec().arrays[0].token_shape == (nkv, d) and part.state_spec() is None
+    assert part.kv_cache_spec().arrays[1].token_shape == (nkv, d) and part.state_spec() is None
     specs = part.tensor_specs()
     assert specs["a.q_proj.weight"].shape == (nq * d, H) and specs["a.o_proj.weight"].shape == (H, nq * d)
     W = load(part, {k: rnd(*s.shape, scale=0.2, seed=i) for i, (k, s) in enumerate(specs.items())}, dtype, gpu)

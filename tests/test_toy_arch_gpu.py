@@ -414,6 +414,7 @@ def test_a_mixer_whose_cache_entry_is_one_vector_per_token(dtype, tol, tmp_path,
     assert lat.slot_ids == [0, 2] and att.slot_ids == [1]
     assert lat.arrays["latent"].shape == (2, lat.num_pages, page, 12) and lat.arrays["gain"].dtype == torch.float32
     assert att.arrays["v"].shape == (1, att.num_pages, 2, 16, page)
+    assert att.arrays["k"].shape == (1, att.num_pages, 2, 16 // 8, page, 8)       # a key in chunks of 8 elements
     assert eng.cache.page_bytes() == page * (2 * (12 * elem + 4) + 2 * 2 * 16 * elem)
     assert lat.num_pages == 2 * 96 // page            # every seat at its longest: nothing more is worth having
 
