@@ -207,6 +207,22 @@ def stream(args) -> None:
     dev = torch.device("cuda:0")
     sink = torch.zeros(4, dtype=torch.int32, device=dev)
     print(f"plain read stream over 2 GiB: {K.probe_read_bandwidth(dev):.0f} GB/s")
+    # what a compute unit takes in from L2: every workgroup reads the same few hundred kilobytes (the
+    # rows of X of a few-rows product), over and over
+    for kb in (64, 256, 1024):
+        buf = torch.zeros(kb << 10, dtype=torch.uint8, device=dev)
+        for wgs in (256, 512, 1024):
+            reps = max(4, (64 << 20) // (kb << 10) // 8)
+            for _ in range(2):
+                K.stream_reread(buf, wgs, reps, sink)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            K.stream_reread(buf, wgs, reps, sink)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            total = wgs * reps * (kb << 10)
+            print(f"{wgs} workgroups of 256 each read the same {kb} KB {reps} times: {dt * 1e6:.0f} us = "
+                  f"{total / dt / 1e12:.2f} TB/s into the compute units ({total / dt / 1e9 / min(wgs, 256):.0f} GB/s per unit)")
     for mb in [float(x) for x in args.megabytes.split(",")]:
         n = int(mb * 1e6) // 16 * 16
         copies = max(2, min(200, int(3e9 // n)))

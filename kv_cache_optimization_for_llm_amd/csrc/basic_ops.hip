@@ -349,6 +349,35 @@ extern "C" int kva_stream_read(const void *p, long long bytes, int workgroups, v
     return KVA_OK;
 }
 
+// Another probe: EVERY workgroup reads all `count` 16-byte units, `repeats` times over, through the
+// caches (plain loads, four in flight per lane).  With a range that fits the L2 of a die this is
+// what a compute unit can take in from L2 - the rows of X that every workgroup of a few-rows
+// product has to read beside its share of the weights.
+__global__ void __launch_bounds__(256) stream_reread_kernel(const uint4 *__restrict__ p, size_t count, int repeats,
+                                                            unsigned *__restrict__ sink) {
+    unsigned acc = 0;
+    for (int rep = 0; rep < repeats; ++rep) {
+        size_t i = threadIdx.x;
+        for (; i + 3 * 256 < count; i += 4 * 256) {
+            const uint4 a = p[i], b = p[i + 256], c = p[i + 512], d = p[i + 768];
+            acc ^= a.x ^ b.y ^ c.z ^ d.w;
+        }
+        for (; i < count; i += 256) acc ^= p[i].x;
+        acc += rep;                                  // (the turns are not the same expression)
+    }
+    if (acc == 0x9E3779B9u && threadIdx.x == 255 && sink != nullptr) *sink = acc;
+}
+
+extern "C" int kva_stream_reread(const void *p, long long bytes, int workgroups, int repeats, void *sink,
+                                 hipStream_t stream) {
+    KVA_REQUIRE(workgroups >= 1 && workgroups <= 65535 && repeats >= 1, "stream_reread: 1..65535 workgroups, at least one turn");
+    KVA_REQUIRE(bytes >= 16 && p != nullptr && ((uintptr_t)p % 16) == 0, "stream_reread: a 16-byte aligned range is needed");
+    hipLaunchKernelGGL(stream_reread_kernel, dim3(workgroups), dim3(256), 0, stream, (const uint4 *)p,
+                       (size_t)(bytes / 16), repeats, (unsigned *)sink);
+    KVA_CHECK_LAUNCH("stream_reread");
+    return KVA_OK;
+}
+
 // ---------------------------------------------------------------------------------------
 // x <- x * scale, and then, with cap > 0, x <- cap * tanh(x / cap): the constants a model may put
 // on its embeddings and on its logits.  fp32 arithmetic, rounded to the storage type.

@@ -42,14 +42,17 @@ _LDS_MIN_MEAN_KEYS = 2048
 _LDS_SOME_GROUPS = 576
 _LDS_SOME_GROUPS_MEAN_KEYS = 1024
 # Head sizes above 96 do twice the matrix-core work per key and row for the same vector work, and
-# one wavefront with two row tiles of them fills its SIMD's registers alone: there the workgroup kernel
-# (two workgroups per compute unit) is ahead from 1,024 keys a row on (head size 128, a 2,048-token
-# prompt from position 0: 93 us against 107; 4,096 tokens: 235 against 375; 1,024: 45 against 41), and
-# with the keys cut into shorter ranges also for short portions deep in a context (256 tokens at
-# position 4,096: 48 us in 8 ranges against 71 for the one-wavefront kernel at its best split; 128 at
-# 8,192: 47 against 64; 64 at 8,192: 35 against 41; 256 at 2,048: 38 against 50; 128 at 2,048 and
-# 256 at 1,024 are ties or losses, hence the 2,048 keys a row for fewer than 128 workgroups).
-_LDS_MIN_MEAN_KEYS_WIDE_HEADS = 1024
+# one wavefront with two row tiles of them fills its SIMD's registers alone.  With keys laid out in
+# chunks of 8 elements across a page (one run of bytes per operand load) the one-wavefront kernel
+# holds out longer than it did: head size 128, one prompt from position 0, 24 heads, one-wavefront
+# against workgroup kernel: 1,024 tokens 31 against 36 us, 2,048 (384 workgroups) 61 against 71,
+# 2,560 (480) 80 against 91, but 3,072 (576) 163 against 112 and 4,096 221 against 161; 32 heads,
+# 2,560 tokens (640 workgroups) 142 against 97.  So: from 512 workgroups on, or where rows visit
+# 2,048 keys or more on average - with the keys cut into shorter ranges also for short portions deep
+# in a context (256 tokens at position 4,096: 48 us in 8 ranges against 71 for the one-wavefront
+# kernel at its best split; 128 at 8,192: 47 against 64; 64 at 8,192: 35 against 41).
+_LDS_MIN_MEAN_KEYS_WIDE_HEADS = 2048
+_LDS_MANY_GROUPS_WIDE_HEADS = 512
 _LDS_MIN_GROUPS_WIDE_HEADS = 16
 _LDS_TARGET_GROUPS_WIDE_HEADS = 512
 _LDS_MIN_KEYS_PER_SPLIT_WIDE_HEADS = 256
@@ -66,6 +69,8 @@ def use_lds_kernel(groups: int, mean_keys: float, head_dim: int) -> bool:
     if groups >= _LDS_MANY_GROUPS:
         return True
     if head_dim > 96:
+        if groups >= _LDS_MANY_GROUPS_WIDE_HEADS:
+            return True
         if groups >= _LDS_MIN_GROUPS:
             return mean_keys >= _LDS_MIN_MEAN_KEYS_WIDE_HEADS
         return groups >= _LDS_MIN_GROUPS_WIDE_HEADS and mean_keys >= _LDS_MIN_MEAN_KEYS

@@ -212,6 +212,13 @@ def stream_read(x: torch.Tensor, workgroups: int, sink: torch.Tensor) -> None:
                                     _dev(sink, "sink", torch.int32), _stream()), "stream_read")
 
 
+def stream_reread(x: torch.Tensor, workgroups: int, repeats: int, sink: torch.Tensor) -> None:
+    """A probe: every one of ``workgroups`` workgroups reads all of ``x``, ``repeats`` times over,
+    through the caches.  With an ``x`` that fits a die's L2: what a compute unit takes in from there."""
+    check(hip_lib().kva_stream_reread(_dev(x, "x"), x.numel() * x.element_size(), int(workgroups), int(repeats),
+                                      _dev(sink, "sink", torch.int32), _stream()), "stream_reread")
+
+
 def probe_read_bandwidth(device, megabytes: int = 2048, workgroups: int = 2048, reps: int = 5) -> float:
     """GB/s of a plain read stream over a buffer far larger than every cache, best of ``reps``."""
     x = torch.empty(megabytes << 20, dtype=torch.uint8, device=device)

@@ -38,6 +38,7 @@ _HIP_SIGNATURES = {
     "kva_residual_add": [P, P, LL, I, P],
     "kva_scale_softcap": [P, LL, F, F, I, P],
     "kva_stream_read": [P, LL, I, P, P],
+    "kva_stream_reread": [P, LL, I, I, P, P],
     "kva_silu_mul": [P, P, I, I, I, P],
     "kva_cast": [P, P, LL, I, I, P],
     "kva_rope_kv_write": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],

@@ -43,6 +43,10 @@ def test_which_prompt_rows_go_to_the_workgroup_kernel():
     # a 256-token portion at position 4,096: 64 workgroups
     assert not use_lds_kernel(64, 4224.5, 64) and use_lds_kernel(64, 4224.5, 128)
     assert not use_lds_kernel(64, 1152.5, 128)               # the same portion at position 1,024
+    # head size 128, 24 heads on 8 kv heads: a 2,048-token prompt (384 workgroups) and one of 2,560 (480)
+    # stay with the one-wavefront kernel, 3,072 tokens (576) do not; nor does a portion whose rows visit 2,048 keys
+    assert not use_lds_kernel(384, 1024.5, 128) and not use_lds_kernel(480, 1280.5, 128)
+    assert use_lds_kernel(576, 1536.5, 128) and use_lds_kernel(192, 2560.5, 128)
     assert not use_lds_kernel(8, 8000, 128)                  # a 32-token portion: too few rows to share a key block
     assert choose_lds_splits(64, 4352, KERNEL_MAX_SPLITS, head_dim=128) == (8, 544)
     assert choose_lds_splits(128, 4608, KERNEL_MAX_SPLITS, head_dim=64) == (4, 1152)
