@@ -223,6 +223,32 @@ def stream(args) -> None:
             total = wgs * reps * (kb << 10)
             print(f"{wgs} workgroups of 256 each read the same {kb} KB {reps} times: {dt * 1e6:.0f} us = "
                   f"{total / dt / 1e12:.2f} TB/s into the compute units ({total / dt / 1e9 / min(wgs, 256):.0f} GB/s per unit)")
+    # two streams into a compute unit at once: 256 workgroups, each with a range of its own from
+    # memory (a few-rows product's share of W) and a range all of them read (its rows of X)
+    wgs = 256
+    own_sets = [torch.zeros(wgs * (256 << 10), dtype=torch.uint8, device=dev) for _ in range(12)]
+    for shared_kb in (64, 128, 256):
+        shared = torch.zeros(shared_kb << 10, dtype=torch.uint8, device=dev)
+        line = []
+        for what in ("own", "shared", "both"):
+            calls = [(lambda o=o: K.stream_mixed(o if what != "shared" else None,
+                                                 shared if what != "own" else None, wgs, sink)) for o in own_sets]
+            g = torch.cuda.CUDAGraph()
+            for c in calls[:2]:
+                c()
+            torch.cuda.synchronize()
+            with torch.cuda.graph(g):
+                for i in range(120):
+                    calls[i % len(calls)]()
+            g.replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(5):
+                g.replay()
+            torch.cuda.synchronize()
+            line.append((time.perf_counter() - t0) / (5 * 120) * 1e6)
+        print(f"{wgs} workgroups, each 256 KB of its own from memory and the same {shared_kb} KB from L2: "
+              f"own alone {line[0]:.2f} us, shared alone {line[1]:.2f} us, both at once {line[2]:.2f} us")
     for mb in [float(x) for x in args.megabytes.split(",")]:
         n = int(mb * 1e6) // 16 * 16
         copies = max(2, min(200, int(3e9 // n)))

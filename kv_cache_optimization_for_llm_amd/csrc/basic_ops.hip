@@ -378,6 +378,51 @@ extern "C" int kva_stream_reread(const void *p, long long bytes, int workgroups,
     return KVA_OK;
 }
 
+// A probe of two streams into one compute unit at once.  Half of a workgroup's wavefronts read a
+// range of the workgroup's own (from memory: streamed loads, every workgroup another range), the
+// other half read a range that all workgroups share (from L2 after its first reader).  Either
+// range may be empty.  Against the two alone this shows whether bytes that hit in L2 come for less
+// than bytes from memory while a compute unit is also waiting for memory - the question behind
+// the rows of X in a few-rows product.
+__global__ void __launch_bounds__(512) stream_mixed_kernel(const uint4 *__restrict__ own, size_t own_count,
+                                                           const uint4 *__restrict__ shared, size_t shared_count,
+                                                           unsigned *__restrict__ sink) {
+    unsigned acc = 0;
+    const int t = threadIdx.x & 255;
+    if (threadIdx.x < 256) {
+        const uint4 *p = own + (size_t)blockIdx.x * own_count;
+        size_t i = t;
+        for (; i + 3 * 256 < own_count; i += 4 * 256) {
+            const uint4 a = load_streamed_u4(p + i), b = load_streamed_u4(p + i + 256);
+            const uint4 c = load_streamed_u4(p + i + 512), d = load_streamed_u4(p + i + 768);
+            acc ^= a.x ^ b.y ^ c.z ^ d.w;
+        }
+        for (; i < own_count; i += 256) acc ^= load_streamed_u4(p + i).x;
+    } else {
+        size_t i = t;
+        for (; i + 3 * 256 < shared_count; i += 4 * 256) {
+            const uint4 a = shared[i], b = shared[i + 256], c = shared[i + 512], d = shared[i + 768];
+            acc ^= a.x ^ b.y ^ c.z ^ d.w;
+        }
+        for (; i < shared_count; i += 256) acc ^= shared[i].x;
+    }
+    if (acc == 0x9E3779B9u && t == 255 && sink != nullptr) *sink = acc;
+}
+
+// own: workgroups x own_bytes; shared: shared_bytes (both may be 0 bytes, not both)
+extern "C" int kva_stream_mixed(const void *own, long long own_bytes, const void *shared, long long shared_bytes,
+                                int workgroups, void *sink, hipStream_t stream) {
+    KVA_REQUIRE(workgroups >= 1 && workgroups <= 65535, "stream_mixed: 1..65535 workgroups");
+    KVA_REQUIRE(own_bytes >= 0 && shared_bytes >= 0 && own_bytes + shared_bytes > 0 && own_bytes % 16 == 0 &&
+                shared_bytes % 16 == 0, "stream_mixed: ranges in multiples of 16 bytes, one of them not empty");
+    KVA_REQUIRE((own_bytes == 0 || (own && (uintptr_t)own % 16 == 0)) &&
+                (shared_bytes == 0 || (shared && (uintptr_t)shared % 16 == 0)), "stream_mixed: 16-byte aligned ranges are needed");
+    hipLaunchKernelGGL(stream_mixed_kernel, dim3(workgroups), dim3(512), 0, stream, (const uint4 *)own,
+                       (size_t)(own_bytes / 16), (const uint4 *)shared, (size_t)(shared_bytes / 16), (unsigned *)sink);
+    KVA_CHECK_LAUNCH("stream_mixed");
+    return KVA_OK;
+}
+
 // ---------------------------------------------------------------------------------------
 // x <- x * scale, and then, with cap > 0, x <- cap * tanh(x / cap): the constants a model may put
 // on its embeddings and on its logits.  fp32 arithmetic, rounded to the storage type.

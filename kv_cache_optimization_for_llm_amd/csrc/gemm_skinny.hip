@@ -283,18 +283,31 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
         const int sj = wave / k_waves;                          // place among the waves of this K range
         char *xbase = reinterpret_cast<char *>(red) + (size_t)kpart * 2 * ROWS * 128;
         const int n_chunks = (kper + KC - 1) / KC;
-        // X of a chunk is requested two chunks ahead, like W (one chunk ahead left every turn of the
-        // loop waiting for L2): two sets of staging registers (named, not arrays: an array here
-        // ends up in scratch memory).
+        // X and W of a chunk are requested NB chunks ahead (one chunk ahead left every turn of the
+        // loop waiting for L2; three and four ahead, 201 and 230 registers, were measured no
+        // faster: gate/up at 64 rows 19.6 / 20.0 / 19.8 us).  The staging registers are indexed by
+        // constants only (every loop over them is unrolled), or they would end up in scratch memory.
+        constexpr int NB = 2;
+        // Every workgroup reads the same rows of X, and workgroups that walk K in the same order ask
+        // L2 for the same lines at the same time.  Each workgroup of a die starts at a chunk of its
+        // own and wraps around (the sum over K has the same terms in another order).  Decode steps of
+        // 64 requests at the 1B sizes 1.379 -> 1.355 ms, the LM head at 64 rows 96 -> 91 us, gate/up
+        // 18.9 -> 18.8; starting at blockIdx % chunks instead (the same start within a die, another
+        // on every die) gave gate/up 17.9 but the LM head 99.8 and the step 1.398.  For the kernel
+        // below, whose waves read X themselves, the same rotation changed nothing.
+        const int rot = __builtin_amdgcn_readfirstlane((int)((blockIdx.x >> 3) % (unsigned)n_chunks));   // workgroups b, b + 8, .. share a die's L2
+        auto place = [&](int c) -> int { const int pc = c + rot; return pc >= n_chunks ? pc - n_chunks : pc; };
         struct XRegs { uint4 v0, v1, v2, v3; };
-        XRegs xsa = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
-        XRegs xsb = xsa;
+        XRegs xs[NB];
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+            xs[i] = XRegs{make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
         auto load_unit = [&](int i, int c) -> uint4 {
             int u = (i * J + sj) * 64 + lane;
             if (u >= UNITS) u = 0;
             const int q = u >> 3, c16 = u & 7;
             const int row = (q & ~15) | ((q >> 1) & 7) | ((q & 1) << 3);
-            int k = kbeg + c * KC + c16 * 8;
+            int k = kbeg + place(c) * KC + c16 * 8;
             if (k >= kend) k = kbeg;
             return *reinterpret_cast<const uint4 *>(a.X + (size_t)(row < a.M ? row : 0) * a.ldx + k);
         };
@@ -305,25 +318,23 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
             if (u < UNITS)
                 *reinterpret_cast<uint4 *>(xbase + (c & 1) * ROWS * 128 + q * 128 + ((c16 ^ (row & 7)) << 4)) = v;
         };
-        auto load_x = [&](XRegs &xs, int c) {
-            xs.v0 = load_unit(0, c);
-            if constexpr (MT > 1) xs.v1 = load_unit(1, c);
-            if constexpr (MT > 2) xs.v2 = load_unit(2, c);
-            if constexpr (MT > 3) xs.v3 = load_unit(3, c);
+        auto load_x = [&](XRegs &x, int c) {
+            x.v0 = load_unit(0, c);
+            if constexpr (MT > 1) x.v1 = load_unit(1, c);
+            if constexpr (MT > 2) x.v2 = load_unit(2, c);
+            if constexpr (MT > 3) x.v3 = load_unit(3, c);
         };
-        auto store_x = [&](const XRegs &xs, int c) {
-            store_unit(0, c, xs.v0);
-            if constexpr (MT > 1) store_unit(1, c, xs.v1);
-            if constexpr (MT > 2) store_unit(2, c, xs.v2);
-            if constexpr (MT > 3) store_unit(3, c, xs.v3);
+        auto store_x = [&](const XRegs &x, int c) {
+            store_unit(0, c, x.v0);
+            if constexpr (MT > 1) store_unit(1, c, x.v1);
+            if constexpr (MT > 2) store_unit(2, c, x.v2);
+            if constexpr (MT > 3) store_unit(3, c, x.v3);
         };
-        // W of a chunk goes straight to registers, NB chunks ahead (four were measured no faster)
-        constexpr int NB = 2;
         GFrag8 wbuf[NB][2][NTW];
         auto load_w = [&](GFrag8 (&w)[2][NTW], int c) {
 #pragma unroll
             for (int st = 0; st < 2; ++st) {
-                int k = kbeg + c * KC + st * 32;
+                int k = kbeg + place(c) * KC + st * 32;
                 if (k >= kend) k = kbeg;                        // half a chunk at the end: loaded from a valid place, not used
 #pragma unroll
                 for (int t = 0; t < NTW; ++t) w[st][t].u4 = load_streamed_u4(wp[t] + (size_t)k * 16);
@@ -333,7 +344,7 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
             const char *buf = xbase + (c & 1) * ROWS * 128 + (((r & 7) << 1) + (r >> 3)) * 128;
 #pragma unroll
             for (int st = 0; st < 2; ++st) {
-                if (kbeg + c * KC + st * 32 < kend) {
+                if (kbeg + place(c) * KC + st * 32 < kend) {
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt) {
                         GFrag8 x;
@@ -345,40 +356,34 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
                 }
             }
         };
-        static_assert(NB == 2, "the turns below are written out for two buffers");
-        load_x(xsa, 0);
-        if (n_chunks > 1) load_x(xsb, 1);
-        load_w(wbuf[0], 0);
-        if (n_chunks > 1) load_w(wbuf[1], 1);
-        // Two chunks per turn while every load of the turn exists: no branch in the body, so the
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+            if (i == 0 || i < n_chunks) load_x(xs[i], i);
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+            if (i == 0 || i < n_chunks) load_w(wbuf[i], i);
+        // NB chunks per turn while every load of the turn exists: no branch in the body, so the
         // waits count exactly and the loads issued last stay in flight across them.
         int c = 0;
-        for (; c + 3 < n_chunks; c += 2) {
-            store_x(xsa, c);
-            __syncthreads();
-            load_x(xsa, c + 2);
-            compute(wbuf[0], c);
-            load_w(wbuf[0], c + 2);
-            store_x(xsb, c + 1);
-            __syncthreads();
-            load_x(xsb, c + 3);
-            compute(wbuf[1], c + 1);
-            load_w(wbuf[1], c + 3);
-        }
-        // the last one to three chunks: chunk c in (xsa, wbuf[0]), c + 1 in (xsb, wbuf[1])
-        store_x(xsa, c);
-        __syncthreads();
-        if (c + 2 < n_chunks) load_x(xsa, c + 2);
-        compute(wbuf[0], c);
-        if (c + 2 < n_chunks) load_w(wbuf[0], c + 2);
-        if (c + 1 < n_chunks) {
-            store_x(xsb, c + 1);
-            __syncthreads();
-            compute(wbuf[1], c + 1);
-            if (c + 2 < n_chunks) {
-                store_x(xsa, c + 2);
+        for (; c + 2 * NB - 1 < n_chunks; c += NB) {
+#pragma unroll
+            for (int i = 0; i < NB; ++i) {
+                store_x(xs[i], c + i);
                 __syncthreads();
-                compute(wbuf[0], c + 2);
+                load_x(xs[i], c + i + NB);
+                compute(wbuf[i], c + i);
+                load_w(wbuf[i], c + i + NB);
+            }
+        }
+        // the last one to 2 NB - 1 chunks: chunk c + i is in set i % NB
+#pragma unroll
+        for (int i = 0; i < 2 * NB - 1; ++i) {
+            if (c + i < n_chunks) {
+                store_x(xs[i % NB], c + i);
+                __syncthreads();
+                if (i < NB - 1 && c + i + NB < n_chunks) load_x(xs[i % NB], c + i + NB);
+                compute(wbuf[i % NB], c + i);
+                if (i < NB - 1 && c + i + NB < n_chunks) load_w(wbuf[i % NB], c + i + NB);
             }
         }
         __syncthreads();                                        // the sums below reuse the buffer

@@ -219,6 +219,17 @@ def stream_reread(x: torch.Tensor, workgroups: int, repeats: int, sink: torch.Te
                                       _dev(sink, "sink", torch.int32), _stream()), "stream_reread")
 
 
+def stream_mixed(own: Optional[torch.Tensor], shared: Optional[torch.Tensor], workgroups: int,
+                 sink: torch.Tensor) -> None:
+    """A probe: half of each workgroup's wavefronts stream the workgroup's own 1/``workgroups`` of
+    ``own`` from memory while the other half read all of ``shared`` (from L2); either may be None."""
+    own_bytes = 0 if own is None else own.numel() * own.element_size() // int(workgroups) // 16 * 16
+    shared_bytes = 0 if shared is None else shared.numel() * shared.element_size() // 16 * 16
+    check(hip_lib().kva_stream_mixed(None if own is None else _dev(own, "own"), own_bytes,
+                                     None if shared is None else _dev(shared, "shared"), shared_bytes,
+                                     int(workgroups), _dev(sink, "sink", torch.int32), _stream()), "stream_mixed")
+
+
 def probe_read_bandwidth(device, megabytes: int = 2048, workgroups: int = 2048, reps: int = 5) -> float:
     """GB/s of a plain read stream over a buffer far larger than every cache, best of ``reps``."""
     x = torch.empty(megabytes << 20, dtype=torch.uint8, device=device)

@@ -39,6 +39,7 @@ _HIP_SIGNATURES = {
     "kva_scale_softcap": [P, LL, F, F, I, P],
     "kva_stream_read": [P, LL, I, P, P],
     "kva_stream_reread": [P, LL, I, I, P, P],
+    "kva_stream_mixed": [P, LL, P, LL, I, P, P],
     "kva_silu_mul": [P, P, I, I, I, P],
     "kva_cast": [P, P, LL, I, I, P],
     "kva_rope_kv_write": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
