@@ -26,6 +26,12 @@ _TARGET_WAVES_DECODE = 1024
 _UNSPLIT_WAVES_DECODE = 384
 _MIN_KEYS_PER_SPLIT_DECODE = 64
 _LONG_CONTEXT_DECODE = 2048         # above it a range holds at least _MIN_KEYS_PER_SPLIT keys
+# The merge kernel walks the ranges of a row one after the other, so one request alone with a long
+# context is not cut as far as the wavefront count asks: its attention at 32,768 keys takes 24.6 /
+# 18.6 / 22.0 / 28.4 us in 32 / 64 / 128 / 256 ranges, at 131,072 keys 76.0 / 50.0 / 49.6 / 56.7.
+# (8 kv heads: 512 wavefronts; with fewer heads the ranges go on until there are that many.)
+_MAX_SPLITS_DECODE = 64
+_MIN_WAVES_DECODE = 512
 _KEEP_CACHED_BYTES = 64 << 20       # keys and values of one call (one layer) that may stay in the caches
 
 # wide items (two row tiles per wave) are used when they alone give this many waves
@@ -107,6 +113,8 @@ def choose_splits(num_items: int, num_kv_heads: int, max_context: int, max_split
         target = _TARGET_WAVES_DECODE
         least = _MIN_KEYS_PER_SPLIT_DECODE if max_context <= _LONG_CONTEXT_DECODE else _MIN_KEYS_PER_SPLIT
     want = max(1, target // waves)
+    if decoding:
+        want = min(want, max(_MAX_SPLITS_DECODE, _MIN_WAVES_DECODE // waves))
     most = max(1, (max_context + least - 1) // least)
     return _cut_keys(min(want, most), max_context, max_splits)
 

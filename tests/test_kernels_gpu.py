@@ -602,7 +602,8 @@ def test_attention_of_one_decoded_token_over_a_very_long_context(nkv, ctx, gpu):
     nq, d, page = 2 * nkv, 64, 16
     splits, per = choose_splits(1, nkv, ctx, decoding=True)
     assert K.attention_max_splits() == 256 and splits * per >= ctx
-    assert splits == 256           # 1,024 wavefronts are wanted: more splits than the kernels take
+    # 512 wavefronts are wanted at least: with one or two kv heads more splits than the kernels take
+    assert splits == (256 if nkv <= 2 else 128)
     far = per * 101 - 1                                   # the last key of range 100
     g = torch.Generator().manual_seed(ctx + nkv)
     k = torch.randn(ctx, nkv, d, generator=g) * 0.1
@@ -653,6 +654,8 @@ def test_choose_splits():
     assert choose_splits(32, 8, 1024, decoding=True) == (4, 256)
     assert choose_splits(1, 8, 1024, decoding=True) == (16, 64)
     assert choose_splits(1, 8, 8192, decoding=True) == (64, 128)
+    assert choose_splits(1, 8, 32768, decoding=True) == (64, 512)      # never more ranges than the merge walks cheaply
+    assert choose_splits(2, 8, 32768, decoding=True) == (64, 512)
     assert choose_splits(8, 8, 8192, decoding=True) == (16, 512)
 
 
