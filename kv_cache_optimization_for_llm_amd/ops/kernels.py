@@ -223,6 +223,8 @@ def stream_mixed(own: Optional[torch.Tensor], shared: Optional[torch.Tensor], wo
                  sink: torch.Tensor) -> None:
     """A probe: half of each workgroup's wavefronts stream the workgroup's own 1/``workgroups`` of
     ``own`` from memory while the other half read all of ``shared`` (from L2); either may be None."""
+    if int(workgroups) < 1:
+        raise KernelError("stream_mixed: at least one workgroup")
     own_bytes = 0 if own is None else own.numel() * own.element_size() // int(workgroups) // 16 * 16
     shared_bytes = 0 if shared is None else shared.numel() * shared.element_size() // 16 * 16
     check(hip_lib().kva_stream_mixed(None if own is None else _dev(own, "own"), own_bytes,

@@ -763,3 +763,22 @@ def test_which_host_memory_a_kernel_may_write(gpu):
     assert K.host_memory_is_mapped(torch.zeros(8, dtype=torch.int32).pin_memory())
     assert not K.host_memory_is_mapped(torch.zeros(8, dtype=torch.int32))
     assert not K.host_memory_is_mapped(torch.zeros(8, dtype=torch.int32, device=gpu))
+
+
+def test_the_read_probes_take_their_ranges_and_refuse_bad_ones(gpu):
+    """The probes of the measurement programs store nothing; what can be checked is that they run
+    over odd sizes, alone and together, and that a bad range is refused before any launch."""
+    sink = torch.zeros(4, dtype=torch.int32, device=gpu)
+    own = torch.zeros(5 * 4096 + 48, dtype=torch.uint8, device=gpu)
+    shared = torch.zeros(3 * 1024 + 16, dtype=torch.uint8, device=gpu)
+    K.stream_read(own, 7, sink)
+    K.stream_reread(shared, 5, 3, sink)
+    K.stream_mixed(own, shared, 5, sink)
+    K.stream_mixed(own, None, 5, sink)
+    K.stream_mixed(None, shared, 5, sink)
+    torch.cuda.synchronize()
+    assert int(sink.abs().sum()) == 0
+    with pytest.raises(K.KernelError):
+        K.stream_mixed(None, None, 5, sink)
+    with pytest.raises(K.KernelError):
+        K.stream_mixed(own, shared, 0, sink)
