@@ -85,11 +85,13 @@ struct SkinnyArgs {
     int nq, nkv, head_dim, page_size;
     // half tiles: a tile group takes 8 of its tiles' 16 rows (see choose_half_tiles)
     int half;
-    // At most 16 rows: X (x_tiled) or the bf16 result (y_tiled) laid out [columns / 8][16 rows][8],
-    // the order in which the lanes of the consuming product read it (four neighbouring lanes, the
-    // same 8 columns of four neighbouring rows, then take 64 contiguous bytes; row-major they take
-    // four pieces 2 K bytes apart).  A private layout between two products of one part.
-    int x_tiled, y_tiled;
+    // X (x_tiled) or the bf16 result (y_tiled) laid out [columns / 8][tile_rows][8], the order in
+    // which the lanes of the consuming product read it (neighbouring lanes take the same 8 columns
+    // of neighbouring rows: contiguous bytes; row-major they take pieces a row apart).  tile_rows
+    // is M rounded up to 16, or 8 for up to 8 rows: lanes 8..15 of a lane group then read rows
+    // 0..7 again (the same addresses, no traffic) instead of 8 rows of padding.  A private layout
+    // between two products of one part.
+    int x_tiled, y_tiled, tile_rows;
     // K cut into k_slices ranges, one per blockIdx.y, each leaving its own fp32 partial product
     // [M, N] in Y (slice s at Y + s * M * ldy): for matrices with too few tiles to fill the chip
     // with whole-K workgroups when the rows go through LDS (see kva_gemm_skinny_partials)
@@ -156,7 +158,8 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = mt * 16 + r;
-        xr[mt] = a.x_tiled ? a.X + ((size_t)g * (MT * 16) + m) * 8 : a.X + (size_t)(m < a.M ? m : 0) * a.ldx + 8 * g;
+        xr[mt] = a.x_tiled ? a.X + ((size_t)g * a.tile_rows + (a.tile_rows == 8 ? (m & 7) : m)) * 8
+                           : a.X + (size_t)(m < a.M ? m : 0) * a.ldx + 8 * g;
     }
 
     gf32x4 acc[NTW][MT];
@@ -395,7 +398,7 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
         // trip to memory per step, 0.43 us each.)  What is left after the whole chunks goes in
         // chunks of S/2, S/4, .. 1 steps, each with its loads up front.
         constexpr int S = NTW + MT <= 2 ? 8 : ((MT == 1 && NTW == 2) ? 4 : (NTW * MT >= 12 ? 1 : 2));   // by registers
-        const size_t xstep = a.x_tiled ? MT * 16 : 1;          // a step of 32 columns is 4 chunks of (16 MT) rows x 8
+        const size_t xstep = a.x_tiled ? a.tile_rows : 1;      // a step of 32 columns is 4 chunks of tile_rows rows x 8
         const int kb = __builtin_amdgcn_readfirstlane(kbeg), ke = __builtin_amdgcn_readfirstlane(kend);
         const int steps = (ke - kb) / 32, full = steps / S;
         GFrag8 w[S][NTW], x[S][MT];
@@ -690,7 +693,7 @@ __global__ void __launch_bounds__(XL ? 512 : 1024) gemm_skinny_kernel(const Skin
                 }
             } else {
                 bf16_t *dst = reinterpret_cast<bf16_t *>(a.Y) + (size_t)m * a.ldy + n;
-                if (a.y_tiled) dst = reinterpret_cast<bf16_t *>(a.Y) + ((size_t)(n >> 3) * (MT * 16) + m) * 8 + (n & 7);
+                if (a.y_tiled) dst = reinterpret_cast<bf16_t *>(a.Y) + ((size_t)(n >> 3) * a.tile_rows + m) * 8 + (n & 7);
                 if (n + 3 < rows && (a.y_tiled || a.ldy % 4 == 0)) {
                     uint2 w;
                     w.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
@@ -750,6 +753,12 @@ extern "C" int kva_gemm_skinny_sumsq_parts(int N) {
     return choose_half_tiles(n_tiles) ? 2 * n_tiles : n_tiles;
 }
 
+// Rows of the [columns / 8][rows][8] layout that holds M rows (TiledRows of the Python side).  8
+// rows for up to 8: with 16 the down projection of 8 requests read as many bytes of padding as
+// of activations, in every workgroup (decode steps of 8 requests at 8,192 / 768 keys 1.194 / 0.877
+// -> 1.173 / 0.858 ms, of 4 at 768 keys 0.856 -> 0.836).
+extern "C" int kva_tiled_rows(int M) { return M <= 8 ? 8 : (M + 15) / 16 * 16; }
+
 template <int NTW, int EPI>
 static void launch_xl(const SkinnyArgs &a, dim3 grid, dim3 block, size_t lds, hipStream_t stream) {
     switch ((a.M + 15) / 16) {
@@ -801,6 +810,7 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
     KVA_REQUIRE(!y_tiled || (mode == 2 && (N / 2) % 8 == 0), "gemm_skinny: a tiled result is for the gated product with a multiple of 8 columns");
     KVA_REQUIRE(!x_tiled || K % 8 == 0, "gemm_skinny: tiled X");
     a.x_tiled = x_tiled ? 1 : 0; a.y_tiled = y_tiled ? 1 : 0;
+    a.tile_rows = kva_tiled_rows(M);
     const int rows = mode == 2 ? a.inter : N;
     KVA_REQUIRE(mode == 3 || ldy >= rows, "gemm_skinny: Y row stride %d is smaller than its %d columns", ldy, rows);
     const int n_tiles = (rows + 15) / 16;

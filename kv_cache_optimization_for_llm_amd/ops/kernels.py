@@ -656,8 +656,8 @@ class TiledWeight:
 
 class TiledRows:
     """At most 64 rows of ``width`` bf16 columns laid out ``[width / 8, R, 8]`` with ``R`` the row
-    count rounded up to a multiple of 16: element (m, c) at ``[c // 8, m, c % 8]``, rows past
-    ``rows`` unwritten.  It is the order in which the lanes of a few-rows product read X (sixteen
+    count rounded up to a multiple of 16, or 8 for up to 8 rows (the library says which:
+    ``kva_tiled_rows``): element (m, c) at ``[c // 8, m, c % 8]``, rows past ``rows`` unwritten.  It is the order in which the lanes of a few-rows product read X (sixteen
     neighbouring lanes take the same 8 columns of sixteen neighbouring rows: 256 contiguous bytes
     instead of sixteen pieces a row apart), so a product that feeds another can leave its result
     like this.  ``to_rows()`` gives the plain ``[rows, width]``."""
@@ -668,7 +668,7 @@ class TiledRows:
         if not (1 <= rows <= self.MAX_ROWS) or width % 8:
             raise KernelError(f"TiledRows: 1..{self.MAX_ROWS} rows and a multiple of 8 columns, not {rows} x {width}")
         self.rows, self.width = rows, width
-        self.padded = (rows + 15) // 16 * 16
+        self.padded = int(hip_lib().kva_tiled_rows(int(rows)))
         self.data = torch.empty((width // 8, self.padded, 8), dtype=torch.bfloat16, device=device)
 
     @classmethod
@@ -708,7 +708,7 @@ def gemm_skinny(x: torch.Tensor, w: TiledWeight, out: Optional[torch.Tensor], sw
       ``rsqrt(sum(sumsq[m]) / norm_width + eps)``.
     * ``hidden`` (instead of ``out``): ``hidden += x @ W^T`` in place (fp32 add, rounded), plus
       ``scaled_out = round(hidden * next_weight)`` and ``sumsq_out[M, ceil(N / 16)]``.
-    * ``out_tiled`` (gated product, at most 16 rows): ``out`` is ``[N / 2 / 8, 16, 8]``, element
+    * ``out_tiled`` (gated product): ``out`` is ``[N / 2 / 8, R, 8]`` (``R``: see :class:`TiledRows`), element
       (m, c) at ``[c // 8, m, c % 8]`` - the order in which the lanes of a following few-rows
       product read it (a :class:`TiledRows`); such a result is given to that product as ``x``
       with ``x_tiled``."""

@@ -54,6 +54,7 @@ _HIP_SIGNATURES = {
     "kva_attention_lds": [P, P, P, P, I, P, P, P, I, P, I, I, I, I, I, I, F, I, I, I, I, I, P],
     "kva_gemm_skinny": [P, P, P, I, I, I, I, I, I, P, I, I, F, P, P, I, P, P, I, I, P],
     "kva_gemm_skinny_sumsq_parts": [I],
+    "kva_tiled_rows": [I],
     "kva_gemm_skinny_partial_slices": [I, I, I],
     "kva_gemm_skinny_partials": [P, P, P, I, I, I, I, I, P],
     "kva_normed_rows_finish": [P, P, P, I, I, P, I, F, P],

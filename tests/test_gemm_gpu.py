@@ -273,10 +273,10 @@ def test_partial_products_over_ranges_of_k_add_up_to_the_product(m, n, k, gpu):
         K.gemm_skinny_partials(x[:16].contiguous().to(gpu), K.TiledWeight(w.to(gpu)))
 
 
-@pytest.mark.parametrize("m", [1, 7, 16, 40, 64])
+@pytest.mark.parametrize("m", [1, 7, 8, 9, 16, 40, 64])
 @pytest.mark.parametrize("inter, hidden", [(8192, 2048), (256, 96), (96, 64)])
 def test_activations_pass_between_two_products_in_lane_order(m, inter, hidden, gpu):
-    """The gated product can leave its result as TiledRows ([columns / 8][rows rounded up to 16][8])
+    """The gated product can leave its result as TiledRows ([columns / 8][rows rounded up to 16, or 8 rows for up to 8][8])
     and the residual product can read its X in that layout: bit for bit what the row-major route gives."""
     x = rnd(m, hidden).to(gpu)
     w_gu = K.TiledWeight(rnd(2 * inter, hidden, scale=0.2, seed=5).to(gpu), halves=2)
