@@ -826,6 +826,14 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
     if (a.half) groups *= 2;
     int kw = choose_k_waves(groups, K, ntw);
     int groups_per_wg = kw >= 4 ? 1 : 4 / kw;
+    // The gated product has two tile groups or more per compute unit.  Two of them in a workgroup,
+    // K over two wavefronts each, leave a unit one workgroup's reads of X where two workgroups of
+    // K over 8 wavefronts made two: decode steps of 12 / 16 requests at the 1B sizes 0.920 /
+    // 0.978 -> 0.908 / 0.954 ms (the product alone at 16 rows 13.8 -> 12.75 us), at 8 requests
+    // the same, at 3 / 4 requests 0.831 / 0.836 -> 0.837 / 0.844; 16 requests at the 3B / 8B sizes
+    // 1-6 % faster.  For every row count up to 16 alike, so that a token's result does not
+    // depend on how many share its step.
+    if (mode == 2 && M <= 16 && kw > 2 && groups % 2 == 0 && groups >= 2 * compute_units()) { kw = 2; groups_per_wg = 2; }
     // More than 16 tokens and several tiles per wave: workgroups of several tile groups that
     // share X through LDS (at most 4 K ranges of 2 x 64 tokens x 128 bytes: 64 KiB).
     const bool xl = M > 16 && ntw >= 2 && groups >= 2 && !x_tiled;      // tiled rows are read in whole cache lines as they are
