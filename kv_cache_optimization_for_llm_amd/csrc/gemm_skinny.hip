@@ -834,6 +834,10 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
     // 1-6 % faster.  For every row count up to 16 alike, so that a token's result does not
     // depend on how many share its step.
     if (mode == 2 && M <= 16 && kw > 2 && groups % 2 == 0 && groups >= 2 * compute_units()) { kw = 2; groups_per_wg = 2; }
+    // The products into the residual stream: K over at most 8 wavefronts (16 left each of them 4
+    // steps of the output projection; 1B sizes, 8 / 16 rows: output 5.40 / 6.24 -> 5.14 / 5.85 us,
+    // down 10.6 / 13.7 -> 10.3 / 13.2; decode steps of 4-16 requests 1 % faster, 8B sizes the same).
+    if (mode == 3 && M <= 16 && kw > 8) kw = 8;
     // More than 16 tokens and several tiles per wave: workgroups of several tile groups that
     // share X through LDS (at most 4 K ranges of 2 x 64 tokens x 128 bytes: 64 KiB).
     const bool xl = M > 16 && ntw >= 2 && groups >= 2 && !x_tiled;      // tiled rows are read in whole cache lines as they are
@@ -912,6 +916,7 @@ extern "C" int kva_gemm_skinny_qkv_rope(void *q_out, int ldq, const void *X, con
     a.half = xl ? 0 : choose_half_tiles(groups);
     if (a.half) groups *= 2;
     int kw = choose_k_waves(groups, K, 2);
+    if (!xl && kw > 8) kw = 8;                                  // as for the products into the residual stream
     int groups_per_wg = kw >= 4 ? 1 : 4 / kw;
     if (xl) {
         kw = kw < 4 ? kw : 4;
