@@ -6,7 +6,9 @@
 // G = num_q_heads / num_kv_heads.  A decoded token of a model with G <= 16 is one item of one
 // row tile (RT = 1); prompt portions may use RT = 2 so that every key and value a wavefront
 // loads serves 32 query rows.  One 64-lane wavefront runs one
-// (item, kv head, key split).
+// (item, kv head, key split); up to four wavefronts of one workgroup may take neighbouring key
+// splits of the same item and add their results up in LDS (one barrier, at the end), which leaves
+// the merge kernel fewer partial results, or none and no launch.
 //
 // Everything is computed transposed so that no operand ever has to change layout:
 //     S^T = K  * Q^T     A = K rows (16 keys x head-dim slice), B = Q^T  -> lane holds, for its
@@ -41,6 +43,8 @@
 // STREAM: keys and values are loaded with the non-temporal hint (see load_block).
 // a wavefront's key range from which a third block of keys is kept in flight (decoded tokens)
 #define LONG_RANGE_KEYS 1536
+// wavefronts of one workgroup that may share an item (decoded tokens, head sizes up to 128)
+#define KVA_ATTN_MAX_WAVES 4
 
 // ROPE: the item is one decoded token whose Q, K and V lie in `q` as the joined projection left them
 // ([.., q heads | k heads | v heads] per row, not yet rotated, nothing cached).  The wavefront
@@ -84,7 +88,7 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
                       const int *__restrict__ entry_seat, const int *__restrict__ entry_q_start,
                       const int *__restrict__ entry_start_pos, int num_q_heads, int num_kv_heads,
                       int page_size, float scale, int window, int splits, int keys_per_split, const int item, const int kvh, const int split,
-                      const RopeArgs rope = RopeArgs{nullptr, nullptr, nullptr}) {
+                      const RopeArgs rope = RopeArgs{nullptr, nullptr, nullptr}, const int ws = 1, const int wv = 0) {
     constexpr int KSTEP = (D % 32 == 0) ? 32 : 16;   // head-dim slice per S^T product
     static_assert(!ROPE || (RT == 1 && FAST && D % 64 == 0), "rotation inside the kernel: one row tile, pages of 16, head sizes that are multiples of 64");
     constexpr int NKS = D / KSTEP;
@@ -518,12 +522,57 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
         }
     }
 
+    // ---- Several wavefronts of a workgroup on one item (ws > 1): each has walked a range of its
+    // own; all but the first leave (o, m, l) in LDS, lane by lane, and the first adds them to its
+    // own as the merge kernel would - one launch less where the workgroup's ranges are all there
+    // are, fewer partial results for the merge kernel otherwise.  Every wavefront reaches the barrier.
+    int out_splits = splits, out_split = split;
+    if (ws > 1) {
+        extern __shared__ float xch[];
+        constexpr int PER = RT * (NDT * 4 + 2);                 // floats per lane
+        if (wv > 0) {
+            float *mine = xch + ((size_t)(wv - 1) * PER) * KVA_WAVE + lane;
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) mine[(size_t)((rt * NDT + dt) * 4 + i) * KVA_WAVE] = o[rt][dt][i];
+                mine[(size_t)(RT * NDT * 4 + 2 * rt) * KVA_WAVE] = m[rt];
+                mine[(size_t)(RT * NDT * 4 + 2 * rt + 1) * KVA_WAVE] = l[rt];
+            }
+        }
+        __syncthreads();
+        if (wv > 0) return;
+        for (int w = 1; w < ws; ++w) {
+            const float *theirs = xch + ((size_t)(w - 1) * PER) * KVA_WAVE + lane;
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                const float m_w = theirs[(size_t)(RT * NDT * 4 + 2 * rt) * KVA_WAVE];
+                const float l_w = theirs[(size_t)(RT * NDT * 4 + 2 * rt + 1) * KVA_WAVE];
+                const float m_new = fmaxf(m[rt], m_w);
+                // a range without a visible key has m = -inf and weighs nothing
+                const float c_me = (m[rt] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m[rt] - m_new) * scale2);
+                const float c_w = (m_w == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_w - m_new) * scale2);
+                l[rt] = l[rt] * c_me + l_w * c_w;
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        o[rt][dt][i] = o[rt][dt][i] * c_me + theirs[(size_t)((rt * NDT + dt) * 4 + i) * KVA_WAVE] * c_w;
+                m[rt] = m_new;
+            }
+        }
+        out_splits = splits / ws;
+        out_split = split / ws;
+    }
+
     // lane (r, g) holds O[row r][dt * 16 + 4g + i]
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         if (!row_valid[rt]) continue;
         const size_t orow = (size_t)(q_start + tq[rt]) * num_q_heads + head[rt];
-        if (splits == 1) {
+        if (out_splits == 1) {
             const float inv = 1.f / l[rt];
             bf16_t *dst = out + orow * D;
 #pragma unroll
@@ -534,14 +583,14 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
                 *reinterpret_cast<uint2 *>(dst + dt * 16 + 4 * g) = w.u2;
             }
         } else {
-            float *dst = part_o + (orow * splits + split) * D;
+            float *dst = part_o + (orow * out_splits + out_split) * D;
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt)
                 *reinterpret_cast<float4 *>(dst + dt * 16 + 4 * g) =
                     make_float4(o[rt][dt][0], o[rt][dt][1], o[rt][dt][2], o[rt][dt][3]);
             if (g == 0) {
-                part_ml[(orow * splits + split) * 2] = m[rt] * scale2;   // the merge works in the base-2 domain
-                part_ml[(orow * splits + split) * 2 + 1] = l[rt];
+                part_ml[(orow * out_splits + out_split) * 2] = m[rt] * scale2;   // the merge works in the base-2 domain
+                part_ml[(orow * out_splits + out_split) * 2 + 1] = l[rt];
             }
         }
     }
@@ -553,7 +602,7 @@ attention_item(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__re
 // list: the caller orders the list by the number of keys an item visits (most first), so every
 // wavefront gets about the same work - rows late in a prompt visit many keys, early rows few.
 template <int D, int RT, bool FAST, bool STREAM>
-__global__ void __launch_bounds__(KVA_WAVE)
+__global__ void __launch_bounds__(KVA_WAVE * KVA_ATTN_MAX_WAVES)
 attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
                       const bf16_t *__restrict__ q, int q_row_stride,
                       const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
@@ -563,11 +612,14 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
                       const int *__restrict__ entry_seat, const int *__restrict__ entry_q_start,
                       const int *__restrict__ entry_start_pos, int num_q_heads, int num_kv_heads,
                       int page_size, float scale, int window, int splits, int keys_per_split, int num_items, int pair) {
-    const int kvh = blockIdx.x % num_kv_heads, split = blockIdx.z;
+    // (blockDim.x / 64 wavefronts of a workgroup take neighbouring key ranges of one item; `splits` counts all ranges)
+    const int ws = blockDim.x / KVA_WAVE, wv = threadIdx.x / KVA_WAVE;
+    const int kvh = blockIdx.x % num_kv_heads, split = blockIdx.z * ws + wv;
     const int w = blockIdx.x / num_kv_heads;
     attention_item<D, RT, FAST, STREAM>(out, part_o, part_ml, q, q_row_stride, k_cache, v_cache, block_table, max_blocks,
                                 item_meta, item_entry, item_row0, entry_seat, entry_q_start, entry_start_pos, num_q_heads,
-                                num_kv_heads, page_size, scale, window, splits, keys_per_split, w, kvh, split);
+                                num_kv_heads, page_size, scale, window, splits, keys_per_split, w, kvh, split,
+                                RopeArgs{nullptr, nullptr, nullptr}, ws, wv);
     const int other = num_items - 1 - w;
     if (pair && other > w)
         attention_item<D, RT, FAST, STREAM>(out, part_o, part_ml, q, q_row_stride, k_cache, v_cache, block_table, max_blocks,
@@ -577,18 +629,19 @@ attention_mfma_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, floa
 
 // One wavefront per (decoded token, kv head, key split), with rotation and cache write inside.
 template <int D, bool STREAM>
-__global__ void __launch_bounds__(KVA_WAVE)
+__global__ void __launch_bounds__(KVA_WAVE * KVA_ATTN_MAX_WAVES)
 attention_mfma_rope_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
                            const bf16_t *__restrict__ qkv, int row_stride,
                            bf16_t *k_cache, bf16_t *v_cache,
                            const int *__restrict__ block_table, int max_blocks,
                            const int *__restrict__ item_meta, int num_q_heads, int num_kv_heads,
                            float scale, int window, int splits, int keys_per_split, const RopeArgs rope) {
-    const int kvh = blockIdx.x % num_kv_heads, split = blockIdx.z;
+    const int ws = blockDim.x / KVA_WAVE, wv = threadIdx.x / KVA_WAVE;
+    const int kvh = blockIdx.x % num_kv_heads, split = blockIdx.z * ws + wv;
     const int w = blockIdx.x / num_kv_heads;
     attention_item<D, 1, true, STREAM, true>(out, part_o, part_ml, qkv, row_stride, k_cache, v_cache, block_table, max_blocks,
                                              item_meta, nullptr, nullptr, nullptr, nullptr, nullptr, num_q_heads,
-                                             num_kv_heads, 16, scale, window, splits, keys_per_split, w, kvh, split, rope);
+                                             num_kv_heads, 16, scale, window, splits, keys_per_split, w, kvh, split, rope, ws, wv);
 }
 
 // out[row, :] = sum_s o_s * exp(m_s - M) / sum_s l_s * exp(m_s - M),  M = max_s m_s.
@@ -706,6 +759,20 @@ extern "C" int kva_attention_mfma_row_tiles(int head_dim, int wide) {
     return 1;
 }
 
+// Wavefronts of one workgroup that share an item (each a key range of its own, added up in LDS):
+// 1, 2 or 4; more than one for items of one row tile, not in pairs, head sizes up to 128, and a
+// number of key ranges they divide.
+static bool kva_attention_mfma_waves_ok(int waves, int splits, int head_dim, int row_tiles, int pair) {
+    if (waves == 1) return true;
+    return (waves == 2 || waves == KVA_ATTN_MAX_WAVES) && row_tiles == 1 && !pair && head_dim <= 128 &&
+           splits >= waves && splits % waves == 0;
+}
+
+// LDS in which all but the first of them leave their (o, m, l): head_dim + 2 floats per lane each.
+static size_t kva_attention_mfma_exchange_bytes(int waves, int head_dim) {
+    return waves > 1 ? (size_t)(waves - 1) * (head_dim / 16 * 4 + 2) * KVA_WAVE * sizeof(float) : 0;
+}
+
 extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, const void *q,
                                   int q_row_stride, const void *k_cache, const void *v_cache,
                                   const int *block_table, int max_blocks, const int *item_meta,
@@ -714,9 +781,12 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
                                   const int *entry_start_pos, int total_rows, int num_q_heads,
                                   int num_kv_heads, int head_dim, int page_size, float scale, int window,
                                   int splits, int keys_per_split, int pair, int all_rows,
-                                  int keep_cached, hipStream_t stream) {
+                                  int keep_cached, int waves, hipStream_t stream) {
     KVA_REQUIRE(num_items >= 0 && num_q_heads > 0 && num_kv_heads > 0 && max_blocks > 0,
                 "attention_mfma: bad sizes");
+    KVA_REQUIRE(kva_attention_mfma_waves_ok(waves, splits, head_dim, row_tiles, pair),
+                "attention_mfma: %d wavefronts per item need one row tile, no pairs, a head size up to 128 and a "
+                "number of key ranges (%d) they divide", waves, splits);
     KVA_REQUIRE(num_q_heads % num_kv_heads == 0, "attention_mfma: %d query heads is not a multiple of %d kv heads",
                 num_q_heads, num_kv_heads);
     KVA_REQUIRE(kva_attention_mfma_supported(head_dim, page_size),
@@ -725,8 +795,9 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
     KVA_REQUIRE(q_row_stride % 8 == 0, "attention_mfma: query row stride %d must be a multiple of 8", q_row_stride);
     KVA_REQUIRE(splits >= 1 && splits <= MERGE_MAX_SPLITS && num_kv_heads <= 65535,
                 "attention_mfma: at most %d splits and 65535 kv heads", MERGE_MAX_SPLITS);
-    KVA_REQUIRE(splits == 1 || (keys_per_split > 0 && keys_per_split % 32 == 0 && part_o && part_ml),
-                "attention_mfma: splits need a key count that is a multiple of 32 and a workspace");
+    KVA_REQUIRE(splits == 1 || (keys_per_split > 0 && keys_per_split % 32 == 0),
+                "attention_mfma: splits need a key count that is a multiple of 32");
+    KVA_REQUIRE(splits == waves || (part_o && part_ml), "attention_mfma: key ranges of several workgroups need a workspace");
     KVA_REQUIRE(window >= 0, "attention_mfma: negative window");
     KVA_REQUIRE(scale > 0.f, "attention_mfma: the score scale must be positive");
     KVA_REQUIRE(row_tiles == 1 || row_tiles == kva_attention_mfma_row_tiles(head_dim, 1),
@@ -734,10 +805,11 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
     if (num_items == 0) return KVA_OK;
     KVA_REQUIRE((long)num_items * num_kv_heads < (1L << 31), "attention_mfma: too many work items");
     const int waves_x = pair ? (num_items + 1) / 2 : num_items;
-    dim3 grid(waves_x * num_kv_heads, 1, splits), block(KVA_WAVE);
+    dim3 grid(waves_x * num_kv_heads, 1, splits / waves), block(KVA_WAVE * waves);
+    const size_t lds = kva_attention_mfma_exchange_bytes(waves, head_dim);
     const bool fast = page_size == 16;
 #define LAUNCH(DD, RR, FF, SS)                                                                  \
-    hipLaunchKernelGGL((attention_mfma_kernel<DD, RR, FF, SS>), grid, block, 0, stream, (bf16_t *)out, \
+    hipLaunchKernelGGL((attention_mfma_kernel<DD, RR, FF, SS>), grid, block, lds, stream, (bf16_t *)out, \
                        part_o, part_ml, (const bf16_t *)q, q_row_stride, (const bf16_t *)k_cache, \
                        (const bf16_t *)v_cache, block_table, max_blocks, item_meta, item_entry,  \
                        item_row0,                                                               \
@@ -762,8 +834,8 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
 #undef CASE
 #undef LAUNCH
     KVA_CHECK_LAUNCH("attention_mfma");
-    if (splits > 1)
-        return kva_attention_merge_launch(out, part_o, part_ml, head_dim, splits, item_meta, item_entry, item_row0,
+    if (splits / waves > 1)
+        return kva_attention_merge_launch(out, part_o, part_ml, head_dim, splits / waves, item_meta, item_entry, item_row0,
                                           entry_q_start, num_items, 16 * row_tiles, total_rows, num_q_heads,
                                           num_kv_heads, all_rows, stream);
     return KVA_OK;
@@ -784,7 +856,9 @@ extern "C" int kva_attention_mfma_rope(void *out, float *part_o, float *part_ml,
                                        const int *item_meta, int num_items, int total_rows, int num_q_heads,
                                        int num_kv_heads, int head_dim, int page_size, float scale, int window,
                                        int splits, int keys_per_split, int keep_cached, const float *cos_t,
-                                       const float *sin_t, const int *slots, hipStream_t stream) {
+                                       const float *sin_t, const int *slots, int waves, hipStream_t stream) {
+    KVA_REQUIRE(kva_attention_mfma_waves_ok(waves, splits, head_dim, 1, 0),
+                "attention_mfma_rope: %d wavefronts per item must be 1, 2 or 4 and divide the %d key ranges", waves, splits);
     KVA_REQUIRE(num_items >= 0 && num_q_heads > 0 && num_kv_heads > 0 && max_blocks > 0 && item_meta != nullptr,
                 "attention_mfma_rope: bad sizes");
     KVA_REQUIRE(num_q_heads % num_kv_heads == 0, "attention_mfma_rope: %d query heads is not a multiple of %d kv heads",
@@ -796,16 +870,18 @@ extern "C" int kva_attention_mfma_rope(void *out, float *part_o, float *part_ml,
                 "attention_mfma_rope: row stride %d does not hold the joined projection", row_stride);
     KVA_REQUIRE(splits >= 1 && splits <= MERGE_MAX_SPLITS && num_kv_heads <= 65535,
                 "attention_mfma_rope: at most %d splits and 65535 kv heads", MERGE_MAX_SPLITS);
-    KVA_REQUIRE(splits == 1 || (keys_per_split > 0 && keys_per_split % 32 == 0 && part_o && part_ml),
-                "attention_mfma_rope: splits need a key count that is a multiple of 32 and a workspace");
+    KVA_REQUIRE(splits == 1 || (keys_per_split > 0 && keys_per_split % 32 == 0),
+                "attention_mfma_rope: splits need a key count that is a multiple of 32");
+    KVA_REQUIRE(splits == waves || (part_o && part_ml), "attention_mfma_rope: key ranges of several workgroups need a workspace");
     KVA_REQUIRE(window >= 0 && scale > 0.f, "attention_mfma_rope: window must not be negative and the scale positive");
     KVA_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "attention_mfma_rope: one table missing");
     if (num_items == 0) return KVA_OK;
     KVA_REQUIRE((long)num_items * num_kv_heads < (1L << 31), "attention_mfma_rope: too many work items");
-    dim3 grid(num_items * num_kv_heads, 1, splits), block(KVA_WAVE);
+    dim3 grid(num_items * num_kv_heads, 1, splits / waves), block(KVA_WAVE * waves);
+    const size_t lds = kva_attention_mfma_exchange_bytes(waves, head_dim);
     const RopeArgs rope{cos_t, sin_t, slots};
 #define LAUNCH(DD, SS)                                                                               \
-    hipLaunchKernelGGL((attention_mfma_rope_kernel<DD, SS>), grid, block, 0, stream, (bf16_t *)out, part_o, \
+    hipLaunchKernelGGL((attention_mfma_rope_kernel<DD, SS>), grid, block, lds, stream, (bf16_t *)out, part_o, \
                        part_ml, (const bf16_t *)qkv, row_stride, (bf16_t *)k_cache, (bf16_t *)v_cache,     \
                        block_table, max_blocks, item_meta, num_q_heads, num_kv_heads, scale, window,  \
                        splits, keys_per_split, rope)
@@ -813,8 +889,8 @@ extern "C" int kva_attention_mfma_rope(void *out, float *part_o, float *part_ml,
     else { if (keep_cached) LAUNCH(128, false); else LAUNCH(128, true); }
 #undef LAUNCH
     KVA_CHECK_LAUNCH("attention_mfma_rope");
-    if (splits > 1)
-        return kva_attention_merge_launch(out, part_o, part_ml, head_dim, splits, item_meta, nullptr, nullptr,
+    if (splits / waves > 1)
+        return kva_attention_merge_launch(out, part_o, part_ml, head_dim, splits / waves, item_meta, nullptr, nullptr,
                                           nullptr, num_items, 16, total_rows, num_q_heads, num_kv_heads, 1, stream);
     return KVA_OK;
 }
@@ -891,5 +967,5 @@ extern "C" int kva_attention_mfma_static(void *out, const void *q, int q_row_str
     return kva_attention_mfma(out, part_o, part_ml, q, q_row_stride, k_cache, v_cache, block_table, max_blocks,
                               item_meta, item_entry, item_row0, num_items, row_tiles, entry_seat, entry_q_start,
                               entry_start_pos, total_rows, num_q_heads, num_kv_heads, head_dim, page_size, scale,
-                              window, splits, keys_per_split, pair, all_rows, /*keep_cached=*/0, stream);
+                              window, splits, keys_per_split, pair, all_rows, /*keep_cached=*/0, /*waves=*/1, stream);
 }

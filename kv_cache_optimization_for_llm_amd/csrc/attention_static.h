@@ -3,8 +3,8 @@
 //
 // This entry point has no counterpart in the reference.  It is for callers that cannot allocate
 // device memory: code under HIP graph capture, tight serving loops, harnesses that forbid
-// hipMalloc.  It is kva_attention_mfma (same arguments, same kernels, same results) without the
-// two buffers for the partial results of key splits: those live in a file-scope device array of
+// hipMalloc.  It is kva_attention_mfma (same arguments, same kernels, same results; one wavefront
+// per key split) without the two buffers for the partial results of key splits: those live in a file-scope device array of
 // KVA_ATTENTION_STATIC_SCRATCH_BYTES that every GPU the library runs on holds until the process
 // ends.  The call makes no hipMalloc, hipFree or other allocating call; inputs and outputs are
 // still the caller's.

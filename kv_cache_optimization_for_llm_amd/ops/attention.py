@@ -119,6 +119,48 @@ def choose_splits(num_items: int, num_kv_heads: int, max_context: int, max_split
     return _cut_keys(min(want, most), max_context, max_splits)
 
 
+# Wavefronts of one workgroup that take neighbouring key ranges of a decoded token and add their
+# results up themselves (ops.kernels.attention_mfma, ``waves``).  Where two or four ranges are all
+# there are, no partial result is written and no merge kernel runs: whole decode steps at 768 keys,
+# 1B sizes, 32 requests (four ranges) 1.246 -> 1.188 ms, 48 requests (unsplit before) 1.293 -> 1.259;
+# 17 / 24 / 56 requests 1.125 / 1.192 / 1.381 -> 1.098 / 1.139 / 1.356, 20 requests at 200 keys 1.061 ->
+# 1.018, 24 at 4,096 keys 1.568 -> 1.503, 48 at 2,048 / 8,192 keys (unsplit before, one wavefront on
+# all keys of a request) 1.722 / 3.709 -> 1.631 / 3.229; so between 128 and 512 (item, kv head) pairs
+# the keys go in four ranges, whatever the wavefront count asked for, and from 4,096 keys on up to
+# 1,100 pairs (64 requests at 4,096 / 8,192 keys 2.57 / 4.08 -> 2.52 / 3.86 ms, 128 at 4,096 4.32 ->
+# 4.27; but 128 at 768 keys 2.03 -> 2.11).  With more ranges than four it pays only where the merge kernel has much to
+# read: 8 requests at 8,192 / 32,768 keys (16 ranges of 512 / 2,048 keys) 1.156 / 2.167 -> 1.135 /
+# 2.134 ms, one request at 8,192 keys (64 ranges) 0.755 -> 0.740; but 8 requests at 768 / 2,048 /
+# 4,096 keys 0.846 / 0.932 / 1.024 -> 0.852 / 0.942 / 1.037 and one request at 768 keys 0.688 -> 0.705.
+_SHARED_MAX_HEAD_DIM = 128
+_SHARED_FOUR_FROM = 128             # more (item, kv head) pairs than this ...
+_SHARED_FOUR_BELOW = 512            # ... and fewer than this: four ranges in one workgroup
+_SHARED_LONG_CONTEXT = 4096         # from this many keys on ...
+_SHARED_FOUR_BELOW_LONG = 1100      # ... up to this many pairs
+_SHARED_MIN_KEYS = 512              # many ranges: wavefronts share a workgroup from this many keys a range ...
+_SHARED_MIN_SPLITS = 64             # ... or from this many ranges
+
+
+def choose_decode_ranges(num_items: int, num_kv_heads: int, max_context: int, head_dim: int,
+                         max_splits: int = None) -> tuple:
+    """(key ranges, keys per range, wavefronts per workgroup) for decoded tokens."""
+    pairs = max(1, num_items * num_kv_heads)
+    below = _SHARED_FOUR_BELOW if max_context < _SHARED_LONG_CONTEXT else _SHARED_FOUR_BELOW_LONG
+    if head_dim <= _SHARED_MAX_HEAD_DIM and _SHARED_FOUR_FROM < pairs < below \
+            and max_context >= 4 * _MIN_KEYS_PER_SPLIT_DECODE:
+        splits, per = _cut_keys(4, max_context, 4)
+        if splits in (2, 4):
+            return splits, per, splits
+    splits, per = choose_splits(num_items, num_kv_heads, max_context, max_splits, decoding=True)
+    waves = 1
+    if head_dim <= _SHARED_MAX_HEAD_DIM:
+        if splits in (2, 4):
+            waves = splits
+        elif splits % 4 == 0 and (per >= _SHARED_MIN_KEYS or splits >= _SHARED_MIN_SPLITS):
+            waves = 4
+    return splits, per, waves
+
+
 def choose_lds_splits(groups: int, max_context: int, max_splits: int = None, head_dim: int = 64) -> tuple:
     """(splits, keys_per_split) for the workgroup kernel, under the same limit."""
     if max_splits is None:
@@ -170,10 +212,10 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
         # tables or (None, None); only where rotates_in_kernel() said yes
         if not rotates_in_kernel(batch, kv, num_q_heads, num_kv_heads, head_dim, qkv.dtype):
             raise K.KernelError("paged_attention: this step cannot rotate inside the attention kernel")
-        (_, (_, _, meta), _, splits, per, _, _, keep_cached), = _plan_for(batch, kv, num_q_heads, num_kv_heads, head_dim)
+        (_, (_, _, meta), _, splits, per, _, _, keep_cached, waves), = _plan_for(batch, kv, num_q_heads, num_kv_heads, head_dim)
         return K.attention_mfma_rope(qkv, out, kv.k_cache, kv.v_cache, kv.block_table, meta, num_q_heads,
                                      num_kv_heads, head_dim, scale, rope[0], rope[1],
-                                     kv.slot_mapping if kv.writes else None, window, splits, per, keep_cached)
+                                     kv.slot_mapping if kv.writes else None, window, splits, per, keep_cached, waves)
     if not (qkv.dtype == torch.bfloat16 and K.attention_mfma_supported(head_dim, kv.page_size)
             and qkv.shape[1] % 8 == 0):
         return K.attention_rowwise(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table,
@@ -183,11 +225,11 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
     stride = qkv.shape[1]
     for launch in plan:
         if launch[0] == "wave":
-            _, (item_entry, item_row0, meta), tiles, splits, per, pair, covers_all, keep_cached = launch
+            _, (item_entry, item_row0, meta), tiles, splits, per, pair, covers_all, keep_cached, waves = launch
             K.attention_mfma(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table, item_entry, item_row0,
                              batch.entry_seat, batch.entry_q_start, batch.entry_start_pos, num_q_heads,
                              num_kv_heads, head_dim, scale, window, splits, per, tiles, pair, meta,
-                             covers_all_rows=covers_all, keep_cached=keep_cached)
+                             covers_all_rows=covers_all, keep_cached=keep_cached, waves=waves)
         else:
             _, meta, splits, per, covers_all = launch
             K.attention_lds(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table, meta, num_q_heads,
@@ -204,13 +246,13 @@ def _plan(batch, group: int, num_kv_heads: int, head_dim: int, page_size: int) -
     def decoded(which):
         items = batch.attention_items(group, 1, which)
         n = items[0].shape[0]
-        splits, per = choose_splits(n, num_kv_heads, batch.max_context, decoding=True)
         # a few short contexts: what this call reads is small enough to still be in the
         # memory-side cache at the next step if it is let in (whole steps of the 1B shape, 8 requests
         # of 768 keys, 12.6 MB a layer: 0.913 -> 0.902 ms; 8 of 8,192, 134 MB a layer: 1.27 -> 1.30,
         # so only the small ones)
         small = n * batch.max_context * num_kv_heads * head_dim * 4 <= _KEEP_CACHED_BYTES
-        plan.append(("wave", items, 1, splits, per, False, which == "all", small))
+        splits, per, waves = choose_decode_ranges(n, num_kv_heads, batch.max_context, head_dim)
+        plan.append(("wave", items, 1, splits, per, False, which == "all", small, waves))
 
     if batch.max_q_len * group <= 16:
         decoded("all")
@@ -234,12 +276,12 @@ def _plan(batch, group: int, num_kv_heads: int, head_dim: int, page_size: int) -
         if waves >= _WIDE_MIN_WAVES:
             # items come ordered by work: a wavefront that takes the i-th and the i-th last does
             # about the average; worth it while every SIMD still gets a wavefront
-            plan.append(("wave", items, tiles, 1, 0, waves >= _PAIR_MIN_WAVES, which == "all", False))
+            plan.append(("wave", items, tiles, 1, 0, waves >= _PAIR_MIN_WAVES, which == "all", False, 1))
         else:
             # too few items to fill the chip: the keys are split over wavefronts as well (portions
             # of 256 tokens late in an 8,192-token prompt: 16 % faster than one row tile per wave)
             splits, per = choose_splits(items[0].shape[0], num_kv_heads, batch.max_context)
-            plan.append(("wave", items, tiles, splits, per, False, which == "all", False))
+            plan.append(("wave", items, tiles, splits, per, False, which == "all", False, 1))
     if mixed:
         decoded("short")
     return plan

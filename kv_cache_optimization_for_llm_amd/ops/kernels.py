@@ -436,7 +436,7 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
                    scale: float, window: int = 0, splits: int = 1, keys_per_split: int = 0,
                    row_tiles: int = 1, pair: bool = False,
                    item_meta: Optional[torch.Tensor] = None, covers_all_rows: bool = True,
-                   keep_cached: bool = False) -> torch.Tensor:
+                   keep_cached: bool = False, waves: int = 1) -> torch.Tensor:
     """bf16 matrix-core attention over the paged cache.  Items are (entry, first query row) pairs
     of ``16 * row_tiles`` query rows each, row = token_in_step * (nq / nkv) + head_in_group.
     With ``pair`` one wavefront takes item i and item n-1-i of the list (give the list ordered by
@@ -446,10 +446,15 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
     ``covers_all_rows=False``: the items are only some of the step's rows (the others belong to
     another launch) and a split merge must leave those alone.  ``keep_cached`` (items of one row
     tile): keys and values are loaded through the caches instead of past them - for the few
-    short contexts that are still in the memory-side cache when the next step reads them."""
+    short contexts that are still in the memory-side cache when the next step reads them.
+    ``waves`` (1, 2 or 4; items of one row tile, head sizes up to 128): so many of the ``splits``
+    key ranges go to the wavefronts of one workgroup, which adds their results up itself; only
+    ``splits // waves`` partial results per row are left for the merge (none: no merge launch)."""
     tokens = out.shape[0]
     if out.dtype != torch.bfloat16 or q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16:
         raise KernelError("attention_mfma: bfloat16 only")
+    if waves < 1 or splits % waves:
+        raise KernelError(f"attention_mfma: {waves} wavefronts per item do not divide {splits} key ranges")
     if out.shape != (tokens, num_q_heads * head_dim):
         raise KernelError("attention_mfma: out must be [T, nq * d]")
     check_cache_shapes("attention_mfma", k_cache, v_cache, num_kv_heads, head_dim)
@@ -463,9 +468,9 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
     if item_meta is not None and item_meta.shape != (n_items, 8):
         raise KernelError("attention_mfma: item_meta must be [items, 8]")
     part_o = part_ml = None
-    if splits > 1:
-        part_o = torch.empty((tokens * num_q_heads, splits, head_dim), dtype=torch.float32, device=out.device)
-        part_ml = torch.empty((tokens * num_q_heads, splits, 2), dtype=torch.float32, device=out.device)
+    if splits // waves > 1:
+        part_o = torch.empty((tokens * num_q_heads, splits // waves, head_dim), dtype=torch.float32, device=out.device)
+        part_ml = torch.empty((tokens * num_q_heads, splits // waves, 2), dtype=torch.float32, device=out.device)
     check(hip_lib().kva_attention_mfma(
         _dev(out, "out"), _opt(part_o, "part_o"), _opt(part_ml, "part_ml"),
         _dev(q, "q", contiguous=False), q_row_stride, _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
@@ -476,7 +481,7 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
         _dev(entry_start_pos, "entry_start_pos", torch.int32), tokens * num_q_heads, num_q_heads,
         num_kv_heads, head_dim, k_cache.shape[3], float(scale), int(window), int(splits),
         int(keys_per_split), 1 if pair else 0, 1 if covers_all_rows else 0, 1 if keep_cached else 0,
-        _stream()), "attention_mfma")
+        int(waves), _stream()), "attention_mfma")
     return out
 
 
@@ -490,16 +495,19 @@ def attention_mfma_rope(qkv: torch.Tensor, out: torch.Tensor, k_cache: torch.Ten
                         block_table: torch.Tensor, item_meta: torch.Tensor, num_q_heads: int, num_kv_heads: int,
                         head_dim: int, scale: float, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
                         slot_mapping: Optional[torch.Tensor], window: int = 0, splits: int = 1,
-                        keys_per_split: int = 0, keep_cached: bool = False) -> torch.Tensor:
+                        keys_per_split: int = 0, keep_cached: bool = False, waves: int = 1) -> torch.Tensor:
     """bf16 matrix-core attention of decoded tokens (one token per item) straight from the joined
     Q/K/V projection ``qkv`` ``[T, (nq + 2 nkv) d]``, not yet rotated: the kernel rotates Q and the
     token's K by its position (``cos`` / ``sin`` ``[positions, d / 2]`` fp32, both None: no
     rotation), stores the rotated K and the V at ``slot_mapping[token]`` (None: the cache is only
     read) and attends, the token's own key and value taken from registers.  ``item_meta``
-    ``[items, 8]`` int32: (token row, 1, position, seat, 0, 0, 0, 0)."""
+    ``[items, 8]`` int32: (token row, 1, position, seat, 0, 0, 0, 0).  ``waves``: as for
+    :func:`attention_mfma`."""
     tokens = out.shape[0]
     if out.dtype != torch.bfloat16 or qkv.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16:
         raise KernelError("attention_mfma_rope: bfloat16 only")
+    if waves < 1 or splits % waves:
+        raise KernelError(f"attention_mfma_rope: {waves} wavefronts per item do not divide {splits} key ranges")
     if out.shape != (tokens, num_q_heads * head_dim) or qkv.dim() != 2 or qkv.shape[0] != tokens \
             or qkv.shape[1] != (num_q_heads + 2 * num_kv_heads) * head_dim or not qkv.is_contiguous():
         raise KernelError("attention_mfma_rope: qkv must be [T, (nq + 2 nkv) d] and out [T, nq * d]")
@@ -512,16 +520,16 @@ def attention_mfma_rope(qkv: torch.Tensor, out: torch.Tensor, k_cache: torch.Ten
     if slot_mapping is not None and slot_mapping.shape != (tokens,):
         raise KernelError("attention_mfma_rope: one cache slot per token")
     part_o = part_ml = None
-    if splits > 1:
-        part_o = torch.empty((tokens * num_q_heads, splits, head_dim), dtype=torch.float32, device=out.device)
-        part_ml = torch.empty((tokens * num_q_heads, splits, 2), dtype=torch.float32, device=out.device)
+    if splits // waves > 1:
+        part_o = torch.empty((tokens * num_q_heads, splits // waves, head_dim), dtype=torch.float32, device=out.device)
+        part_ml = torch.empty((tokens * num_q_heads, splits // waves, 2), dtype=torch.float32, device=out.device)
     check(hip_lib().kva_attention_mfma_rope(
         _dev(out, "out"), _opt(part_o, "part_o"), _opt(part_ml, "part_ml"), _dev(qkv, "qkv"), qkv.shape[1],
         _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32),
         block_table.shape[1], _dev(item_meta, "item_meta", torch.int32), item_meta.shape[0], tokens * num_q_heads,
         num_q_heads, num_kv_heads, head_dim, k_cache.shape[3], float(scale), int(window), int(splits),
         int(keys_per_split), 1 if keep_cached else 0, _opt(cos, "cos", torch.float32), _opt(sin, "sin", torch.float32),
-        _opt(slot_mapping, "slot_mapping", torch.int32), _stream()), "attention_mfma_rope")
+        _opt(slot_mapping, "slot_mapping", torch.int32), int(waves), _stream()), "attention_mfma_rope")
     return out
 
 

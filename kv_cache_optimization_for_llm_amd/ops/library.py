@@ -44,8 +44,8 @@ _HIP_SIGNATURES = {
     "kva_cast": [P, P, LL, I, I, P],
     "kva_rope_kv_write": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
     "kva_attention_rowwise": [P, P, I, P, P, P, I, P, P, I, I, I, I, I, F, I, I, P],
-    "kva_attention_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, I, I, P, P, P, I, I, I, I, I, F, I, I, I, I, I, I, P],
-    "kva_attention_mfma_rope": [P, P, P, P, I, P, P, P, I, P, I, I, I, I, I, I, F, I, I, I, I, P, P, P, P],
+    "kva_attention_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, I, I, P, P, P, I, I, I, I, I, F, I, I, I, I, I, I, I, P],
+    "kva_attention_mfma_rope": [P, P, P, P, I, P, P, P, I, P, I, I, I, I, I, I, F, I, I, I, I, P, P, P, I, P],
     "kva_attention_mfma_rope_supported": [I, I, I],
     "kva_attention_max_splits": [],
     "kva_attention_mfma_row_tiles": [I, I],

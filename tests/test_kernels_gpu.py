@@ -395,15 +395,16 @@ def test_attention_never_sees_what_a_page_held_before(nq, nkv, d, page, window, 
 
 
 @pytest.mark.parametrize("nq, nkv, d, window", [(32, 8, 64, 0), (24, 8, 128, 0), (8, 2, 64, 45), (16, 1, 64, 0), (4, 4, 128, 0)])
-@pytest.mark.parametrize("splits", [1, 3, 8])
+@pytest.mark.parametrize("splits, waves", [(1, 1), (3, 1), (8, 1), (2, 2), (4, 4), (8, 4), (8, 2), (12, 4)])
 @pytest.mark.parametrize("rotate", [True, False])
-def test_decode_attention_that_rotates_and_caches_inside(nq, nkv, d, window, splits, rotate, gpu):
+def test_decode_attention_that_rotates_and_caches_inside(nq, nkv, d, window, splits, waves, rotate, gpu):
     """Decoded tokens straight from the joined projection: the attention kernel rotates Q and the
     new K, caches K and V and attends.  Same output and same cache contents as the rotation kernel
     followed by the attention kernel; positions at every place of a page and of a 32-key block,
     position 0 included; a token without a cache slot is attended to but not stored; without a
     slot mapping (a layer call that only reads another's cache) nothing is stored and the key
-    comes from the cache."""
+    comes from the cache.  With ``waves`` > 1 so many key ranges go to the wavefronts of one
+    workgroup, which adds their results up itself (all of them: no merge launch), in both kernels."""
     assert K.attention_mfma_rope_supported(d, 16, nq // nkv) and not K.attention_mfma_rope_supported(48, 16, 2)
     assert not K.attention_mfma_rope_supported(64, 8, 2) and not K.attention_mfma_rope_supported(64, 16, 32)
     page = 16
@@ -434,12 +435,12 @@ def test_decode_attention_that_rotates_and_caches_inside(nq, nkv, d, window, spl
     seat = torch.arange(T, dtype=torch.int32, device=gpu)
     qs = torch.arange(T + 1, dtype=torch.int32, device=gpu)
 
-    def separate(slot_map):
+    def separate(slot_map, waves=1):
         k, v, x = K.keys_to_pages(kc).to(gpu), vc.clone().to(gpu), qkv.clone().to(gpu)
         K.rope_kv_write(x, pos_t.to(gpu), nq, nkv, d, cos, sin, k, v, slot_map.to(gpu), page)
         out = torch.full((T, nq * d), float("nan"), dtype=torch.bfloat16, device=gpu)
         K.attention_mfma(x, x.shape[1], out, k, v, table.to(gpu), ent, zeros, seat, qs, pos_t.to(gpu), nq, nkv, d,
-                         scale, window, splits, per, 1, False, meta)
+                         scale, window, splits, per, 1, False, meta, waves=waves)
         return out, k, v
 
     def fused(slot_map, k=None, v=None):
@@ -447,10 +448,16 @@ def test_decode_attention_that_rotates_and_caches_inside(nq, nkv, d, window, spl
         v = vc.clone().to(gpu) if v is None else v
         out = torch.full((T, nq * d), float("nan"), dtype=torch.bfloat16, device=gpu)
         K.attention_mfma_rope(qkv.to(gpu), out, k, v, table.to(gpu), meta, nq, nkv, d, scale, cos, sin,
-                              None if slot_map is None else slot_map.to(gpu), window, splits, per)
+                              None if slot_map is None else slot_map.to(gpu), window, splits, per, waves=waves)
         return out, k, v
 
     want, k_want, v_want = separate(slots)
+    if waves > 1:
+        shared, _, _ = separate(slots, waves)
+        assert torch.isfinite(shared.float()).all()
+        close(shared, want, torch.bfloat16, f"{waves} wavefronts of a workgroup on one item", tol16=4e-3)
+        with pytest.raises(K.KernelError):
+            separate(slots, 3)
     got, k_got, v_got = fused(slots)
     assert torch.equal(k_got, k_want) and torch.equal(v_got, v_want), "the cache holds other keys or values"
     assert torch.isfinite(got.float()).all()

@@ -3,7 +3,8 @@ cache pool is made from leftover device memory."""
 import pytest
 
 from kv_cache_optimization_for_llm_amd.engine.engine import EngineError, pool_pages_from_memory
-from kv_cache_optimization_for_llm_amd.ops.attention import choose_lds_splits, choose_splits, use_lds_kernel
+from kv_cache_optimization_for_llm_amd.ops.attention import (choose_decode_ranges, choose_lds_splits, choose_splits,
+                                                             use_lds_kernel)
 
 KERNEL_MAX_SPLITS = 256         # what the kernels and their merge take (kva_attention_max_splits)
 
@@ -30,6 +31,36 @@ def test_the_clamp_is_what_bites_for_few_kv_heads():
     assert choose_splits(1, 4, 65536, KERNEL_MAX_SPLITS) == (256, 256)
     assert choose_splits(4096, 8, 2048, KERNEL_MAX_SPLITS) == (1, 0)      # a big prompt fills the GPU by itself
     assert choose_splits(1, 8, 100, KERNEL_MAX_SPLITS) == (1, 0)          # too short to split
+
+
+@pytest.mark.parametrize("nkv", [1, 2, 5, 8])
+@pytest.mark.parametrize("items", [1, 2, 8, 17, 31, 48, 64, 100, 128, 300])
+@pytest.mark.parametrize("context", [1, 40, 200, 768, 4096, 8192, 131072])
+@pytest.mark.parametrize("head_dim", [64, 128, 256])
+def test_key_ranges_of_decoded_tokens_and_the_wavefronts_that_share_them(nkv, items, context, head_dim):
+    """Whatever the batch: the ranges cover every key, there are no more of them than the kernels
+    take, the wavefronts of a workgroup divide them, and head sizes above 128 get one."""
+    splits, per, waves = choose_decode_ranges(items, nkv, context, head_dim, KERNEL_MAX_SPLITS)
+    assert 1 <= splits <= KERNEL_MAX_SPLITS and waves in (1, 2, 4) and splits % waves == 0
+    if splits > 1:
+        assert per % 32 == 0 and splits * per >= context and (splits - 1) * per < context
+    if head_dim > 128:
+        assert waves == 1
+
+
+def test_where_decoded_tokens_need_no_merge_launch():
+    # 17 to 63 requests of 8 kv heads: four ranges, all in one workgroup
+    for items in (17, 24, 32, 48, 63):
+        assert choose_decode_ranges(items, 8, 768, 64, KERNEL_MAX_SPLITS) == (4, 192, 4)
+    assert choose_decode_ranges(64, 8, 768, 64, KERNEL_MAX_SPLITS) == (1, 0, 1)          # enough wavefronts as they are
+    assert choose_decode_ranges(64, 8, 8192, 64, KERNEL_MAX_SPLITS) == (4, 2048, 4)      # but not for long contexts
+    assert choose_decode_ranges(20, 8, 100, 64, KERNEL_MAX_SPLITS) == (2, 64, 2)
+    # many ranges share a workgroup only where the merge has much to read
+    assert choose_decode_ranges(8, 8, 8192, 64, KERNEL_MAX_SPLITS) == (16, 512, 4)
+    assert choose_decode_ranges(8, 8, 4096, 64, KERNEL_MAX_SPLITS) == (16, 256, 1)
+    assert choose_decode_ranges(1, 8, 8192, 64, KERNEL_MAX_SPLITS) == (64, 128, 4)
+    assert choose_decode_ranges(1, 8, 768, 64, KERNEL_MAX_SPLITS) == (12, 64, 1)
+    assert choose_decode_ranges(32, 8, 768, 256, KERNEL_MAX_SPLITS)[2] == 1               # head size 256: one wavefront
 
 
 def test_which_prompt_rows_go_to_the_workgroup_kernel():
