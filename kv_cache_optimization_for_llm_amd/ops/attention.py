@@ -99,10 +99,11 @@ def _cut_keys(want: int, max_context: int, max_splits: int) -> tuple:
 
 
 def choose_splits(num_items: int, num_kv_heads: int, max_context: int, max_splits: int = None,
-                  decoding: bool = False) -> tuple:
+                  decoding: bool = False, merged_by_fours: bool = False) -> tuple:
     """(splits, keys_per_split) for the matrix-core kernel; never more splits than the kernels
     and their merge take (``max_splits``, by default what the library says).  ``decoding``: the
-    items are decoded tokens (one row tile each)."""
+    items are decoded tokens (one row tile each); ``merged_by_fours``: four ranges at a time are
+    added up by their own workgroup, so the merge kernel's limit of ranges a row does not hold."""
     if max_splits is None:
         max_splits = K.attention_max_splits()
     waves = max(1, num_items * num_kv_heads)
@@ -114,7 +115,8 @@ def choose_splits(num_items: int, num_kv_heads: int, max_context: int, max_split
         least = _MIN_KEYS_PER_SPLIT_DECODE if max_context <= _LONG_CONTEXT_DECODE else _MIN_KEYS_PER_SPLIT
     want = max(1, target // waves)
     if decoding:
-        want = min(want, max(_MAX_SPLITS_DECODE, _MIN_WAVES_DECODE // waves))
+        if not merged_by_fours:
+            want = min(want, max(_MAX_SPLITS_DECODE, _MIN_WAVES_DECODE // waves))
     most = max(1, (max_context + least - 1) // least)
     return _cut_keys(min(want, most), max_context, max_splits)
 
@@ -135,10 +137,16 @@ def choose_splits(num_items: int, num_kv_heads: int, max_context: int, max_split
 _SHARED_MAX_HEAD_DIM = 128
 _SHARED_FOUR_FROM = 128             # more (item, kv head) pairs than this ...
 _SHARED_FOUR_BELOW = 512            # ... and fewer than this: four ranges in one workgroup
+_SHARED_SHORT_CONTEXT = 1024        # up to this many keys already from ...
+_SHARED_FOUR_FROM_SHORT = 63        # ... this many pairs (8 / 12 / 16 requests at 768 keys 0.854 / 0.912 / 0.959 ->
+                                    # 0.852 / 0.900 / 0.945 ms; but 8 at 2,048 keys 0.930 -> 0.978, 16 at 8,192 1.56 -> 1.73)
 _SHARED_LONG_CONTEXT = 4096         # from this many keys on ...
 _SHARED_FOUR_BELOW_LONG = 1100      # ... up to this many pairs
 _SHARED_MIN_KEYS = 512              # many ranges: wavefronts share a workgroup from this many keys a range ...
 _SHARED_MIN_SPLITS = 64             # ... or from this many ranges
+_SHARED_MANY = 16                   # (8 ranges in two workgroups of four: 16 requests at 8,192 keys 1.550 -> 1.561 ms)
+_SHARED_MIN_WORKGROUPS = 192
+_SHARED_FEW_BYTES_CONTEXT = 8192
 
 
 def choose_decode_ranges(num_items: int, num_kv_heads: int, max_context: int, head_dim: int,
@@ -146,18 +154,25 @@ def choose_decode_ranges(num_items: int, num_kv_heads: int, max_context: int, he
     """(key ranges, keys per range, wavefronts per workgroup) for decoded tokens."""
     pairs = max(1, num_items * num_kv_heads)
     below = _SHARED_FOUR_BELOW if max_context < _SHARED_LONG_CONTEXT else _SHARED_FOUR_BELOW_LONG
-    if head_dim <= _SHARED_MAX_HEAD_DIM and _SHARED_FOUR_FROM < pairs < below \
+    frm = _SHARED_FOUR_FROM_SHORT if max_context <= _SHARED_SHORT_CONTEXT else _SHARED_FOUR_FROM
+    if head_dim <= _SHARED_MAX_HEAD_DIM and frm < pairs < below \
             and max_context >= 4 * _MIN_KEYS_PER_SPLIT_DECODE:
         splits, per = _cut_keys(4, max_context, 4)
         if splits in (2, 4):
             return splits, per, splits
-    splits, per = choose_splits(num_items, num_kv_heads, max_context, max_splits, decoding=True)
-    waves = 1
     if head_dim <= _SHARED_MAX_HEAD_DIM:
-        if splits in (2, 4):
-            waves = splits
-        elif splits % 4 == 0 and (per >= _SHARED_MIN_KEYS or splits >= _SHARED_MIN_SPLITS):
-            waves = 4
+        # many ranges, four to a workgroup - if that still leaves a workgroup for most compute units
+        # (one request at 32,768 / 131,072 keys: 64 ranges in 128 workgroups 0.979 / 1.616 ms, 128
+        # ranges in 256 workgroups 0.918 / 1.344, 64 ranges of one wavefront each 0.950 / 1.427) or the
+        # context is short enough for its bytes not to matter (one request at 8,192 keys, 64 ranges:
+        # 0.755 -> 0.740)
+        splits, per = choose_splits(num_items, num_kv_heads, max_context, max_splits, decoding=True,
+                                    merged_by_fours=True)
+        if splits % 4 == 0 and splits >= _SHARED_MANY and (per >= _SHARED_MIN_KEYS or splits >= _SHARED_MIN_SPLITS) \
+                and (pairs * (splits // 4) >= _SHARED_MIN_WORKGROUPS or max_context <= _SHARED_FEW_BYTES_CONTEXT):
+            return splits, per, 4
+    splits, per = choose_splits(num_items, num_kv_heads, max_context, max_splits, decoding=True)
+    waves = splits if splits in (2, 4) and head_dim <= _SHARED_MAX_HEAD_DIM else 1
     return splits, per, waves
 
 

@@ -60,7 +60,17 @@ def test_where_decoded_tokens_need_no_merge_launch():
     assert choose_decode_ranges(8, 8, 4096, 64, KERNEL_MAX_SPLITS) == (16, 256, 1)
     assert choose_decode_ranges(1, 8, 8192, 64, KERNEL_MAX_SPLITS) == (64, 128, 4)
     assert choose_decode_ranges(1, 8, 768, 64, KERNEL_MAX_SPLITS) == (12, 64, 1)
+    # short contexts: four ranges from 8 requests of 8 kv heads on
+    assert choose_decode_ranges(8, 8, 768, 64, KERNEL_MAX_SPLITS) == (4, 192, 4)
+    assert choose_decode_ranges(7, 8, 768, 64, KERNEL_MAX_SPLITS)[2] == 1
+    assert choose_decode_ranges(8, 8, 2048, 64, KERNEL_MAX_SPLITS) == (16, 128, 1)
     assert choose_decode_ranges(32, 8, 768, 256, KERNEL_MAX_SPLITS)[2] == 1               # head size 256: one wavefront
+    # one request and a long context: twice the ranges the merge kernel is given otherwise, four to a
+    # workgroup, so that there is still a workgroup for every compute unit
+    assert choose_decode_ranges(1, 8, 32768, 64, KERNEL_MAX_SPLITS) == (128, 256, 4)
+    assert choose_decode_ranges(1, 8, 131072, 64, KERNEL_MAX_SPLITS) == (128, 1024, 4)
+    assert choose_decode_ranges(1, 1, 65536, 64, KERNEL_MAX_SPLITS) == (256, 256, 1)      # 64 workgroups would be too few
+    assert choose_decode_ranges(16, 8, 8192, 64, KERNEL_MAX_SPLITS) == (8, 1024, 1)
 
 
 def test_which_prompt_rows_go_to_the_workgroup_kernel():
