@@ -135,6 +135,13 @@ def choose_splits(num_items: int, num_kv_heads: int, max_context: int, max_split
 # 2.134 ms, one request at 8,192 keys (64 ranges) 0.755 -> 0.740; but 8 requests at 768 / 2,048 /
 # 4,096 keys 0.846 / 0.932 / 1.024 -> 0.852 / 0.942 / 1.037 and one request at 768 keys 0.688 -> 0.705.
 _SHARED_MAX_HEAD_DIM = 128
+# Head size 128 (8 layers of the 8B sizes, ms a step, one wavefront a range -> this rule): 24 / 32
+# requests at 768 keys 1.194 / 1.213 -> 1.147 / 1.177 and 24 at 8,448 keys 2.281 -> 2.161, but 48
+# requests (384 pairs, unsplit before) 1.324 -> 1.373 and 3.109 -> 3.176, and 8 requests at 8,448 keys
+# in 16 ranges, four to a workgroup, 1.319 -> 1.337: there the four ranges end at 384 pairs and many
+# ranges keep a wavefront each.
+_SHARED_TUNED_HEAD_DIM = 64
+_SHARED_FOUR_BELOW_WIDE = 384
 _SHARED_FOUR_FROM = 128             # more (item, kv head) pairs than this ...
 _SHARED_FOUR_BELOW = 512            # ... and fewer than this: four ranges in one workgroup
 _SHARED_SHORT_CONTEXT = 1024        # up to this many keys already from ...
@@ -154,13 +161,16 @@ def choose_decode_ranges(num_items: int, num_kv_heads: int, max_context: int, he
     """(key ranges, keys per range, wavefronts per workgroup) for decoded tokens."""
     pairs = max(1, num_items * num_kv_heads)
     below = _SHARED_FOUR_BELOW if max_context < _SHARED_LONG_CONTEXT else _SHARED_FOUR_BELOW_LONG
+    wide = head_dim > _SHARED_TUNED_HEAD_DIM
+    if wide:
+        below = _SHARED_FOUR_BELOW_WIDE
     frm = _SHARED_FOUR_FROM_SHORT if max_context <= _SHARED_SHORT_CONTEXT else _SHARED_FOUR_FROM
     if head_dim <= _SHARED_MAX_HEAD_DIM and frm < pairs < below \
             and max_context >= 4 * _MIN_KEYS_PER_SPLIT_DECODE:
         splits, per = _cut_keys(4, max_context, 4)
         if splits in (2, 4):
             return splits, per, splits
-    if head_dim <= _SHARED_MAX_HEAD_DIM:
+    if head_dim <= _SHARED_MAX_HEAD_DIM and not wide:
         # many ranges, four to a workgroup - if that still leaves a workgroup for most compute units
         # (one request at 32,768 / 131,072 keys: 64 ranges in 128 workgroups 0.979 / 1.616 ms, 128
         # ranges in 256 workgroups 0.918 / 1.344, 64 ranges of one wavefront each 0.950 / 1.427) or the
