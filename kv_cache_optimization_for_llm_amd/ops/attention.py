@@ -264,8 +264,8 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
 
 def _plan(batch, group: int, num_kv_heads: int, head_dim: int, page_size: int) -> list:
     """The launches of one attention call over ``batch``: ("wave", items, row tiles, splits, keys per
-    split, pair, covers all rows, keep cached) and ("lds", item records, splits, keys per split,
-    covers all rows)."""
+    split, pair, covers all rows, keep cached, wavefronts of a workgroup that share an item) and
+    ("lds", item records, splits, keys per split, covers all rows)."""
     plan = []
 
     def decoded(which):
