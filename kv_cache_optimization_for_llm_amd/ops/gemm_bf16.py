@@ -35,6 +35,11 @@ from . import kernels as K
 SKINNY_MAX_ROWS = 16            # every shape
 SKINNY_MID_ROWS = 32            # small or tall matrices, and the Q/K/V product with its epilogue
 SKINNY_MID_ELEMENTS = 3 << 22
+# Small matrices whole (with their epilogue) only up to 20 rows since their partial products over
+# ranges of K, added up by the norm kernel, exist: decode steps of 17 / 24 / 32 requests, output
+# projection whole -> in ranges: 1B sizes 1.108 / 1.141 / 1.204 -> 1.125 / 1.126 / 1.176 ms, 8 layers
+# of the 3B sizes 18 / 24 / 32 requests 0.806 / 0.834 / 0.881 -> 0.806 / 0.828 / 0.858.
+SKINNY_SMALL_ROWS = 20
 SKINNY_ROTATED_ROWS = 48        # the Q/K/V product with its epilogue, matrices above SKINNY_MID_ELEMENTS
 SKINNY_WIDE_ROWS = 64           # matrices whose waves share X through LDS
 SKINNY_WIDE_N = 32768
@@ -48,7 +53,7 @@ def use_skinny(m: int, n: int, k: int, gated: bool = False, rotated: bool = Fals
         return False
     if m <= SKINNY_MAX_ROWS:
         return True
-    if m <= SKINNY_MID_ROWS and (rotated or n * k <= SKINNY_MID_ELEMENTS or n >= 4 * k):
+    if m <= SKINNY_MID_ROWS and (rotated or (n * k <= SKINNY_MID_ELEMENTS and m <= SKINNY_SMALL_ROWS) or n >= 4 * k):
         return True
     if rotated and m <= SKINNY_ROTATED_ROWS and n * k > SKINNY_MID_ELEMENTS:
         return True
