@@ -277,6 +277,10 @@ def _plan(batch, group: int, num_kv_heads: int, head_dim: int, page_size: int) -
         # so only the small ones)
         small = n * batch.max_context * num_kv_heads * head_dim * 4 <= _KEEP_CACHED_BYTES
         splits, per, waves = choose_decode_ranges(n, num_kv_heads, batch.max_context, head_dim)
+        # (not where wavefronts share a workgroup: 8 / 16 / 32 requests of 768 keys in four ranges
+        # 0.854 / 0.942 / 1.154 ms through the caches, 0.848 / 0.938 / 1.124 past them; 4 requests of
+        # 2,048 keys, a wavefront a range, 0.863 against 0.875)
+        small = small and waves == 1
         plan.append(("wave", items, 1, splits, per, False, which == "all", small, waves))
 
     if batch.max_q_len * group <= 16:
