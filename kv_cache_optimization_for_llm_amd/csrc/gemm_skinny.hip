@@ -838,6 +838,9 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
     // steps of the output projection; 1B sizes, 8 / 16 rows: output 5.40 / 6.24 -> 5.14 / 5.85 us,
     // down 10.6 / 13.7 -> 10.3 / 13.2; decode steps of 4-16 requests 1 % faster, 8B sizes the same).
     if (mode == 3 && M <= 16 && kw > 8) kw = 8;
+    // Vocabulary-sized matrices (four tiles a wavefront, all of K each): eight wavefronts a workgroup
+    // rather than four, 251 workgroups (LM head of the 1B sizes at 8 / 16 rows 89.4 / 90.5 -> 84.1 / 85.4 us).
+    if (ntw == 4 && M <= 16 && kw == 1) groups_per_wg = 8;
     // More than 16 tokens and several tiles per wave: workgroups of several tile groups that
     // share X through LDS (at most 4 K ranges of 2 x 64 tokens x 128 bytes: 64 KiB).
     const bool xl = M > 16 && ntw >= 2 && groups >= 2 && !x_tiled;      // tiled rows are read in whole cache lines as they are
@@ -850,6 +853,7 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
         // workgroup takes four groups (8B sizes, 896 groups: decode steps of 48 / 64 requests
         // 5.05 / 5.48 -> 4.96 / 5.30 ms; with 512 groups, 128 workgroups, 5 % slower).
         if (kw == 4 && groups / 4 >= compute_units() * 7 / 8) { kw = 2; groups_per_wg = 4; }
+        if (kw == 1) groups_per_wg = 8;                          // (LM head at 32 / 64 rows 85.6 / 91.9 -> 84.1 / 90.3 us)
     }
     // the waves of a K range bring X to LDS together, 64 of a chunk's 128 units per row tile each
     KVA_REQUIRE(!xl || groups_per_wg >= 2, "gemm_skinny: the shared-X form needs two tile groups per workgroup");
