@@ -854,6 +854,11 @@ extern "C" int kva_gemm_skinny(void *Y, const void *X, const void *W, int M, int
         // 5.05 / 5.48 -> 4.96 / 5.30 ms; with 512 groups, 128 workgroups, 5 % slower).
         if (kw == 4 && groups / 4 >= compute_units() * 7 / 8) { kw = 2; groups_per_wg = 4; }
         if (kw == 1) groups_per_wg = 8;                          // (LM head at 32 / 64 rows 85.6 / 91.9 -> 84.1 / 90.3 us)
+        // Three or four row tiles: K over two ranges, four wavefronts a workgroup (fewer, longer
+        // streams and half the barriers' company; the gated product of the 1B sizes at 48 / 64 rows
+        // 17.0 / 19.2 -> 16.2 / 17.7 us, decode steps of 64 requests 1.404 -> 1.382 ms; at 17-32 rows
+        // the same either way).
+        if (kw == 4 && groups_per_wg == 2 && M > 32) kw = 2;
     }
     // the waves of a K range bring X to LDS together, 64 of a chunk's 128 units per row tile each
     KVA_REQUIRE(!xl || groups_per_wg >= 2, "gemm_skinny: the shared-X form needs two tile groups per workgroup");
