@@ -20,10 +20,19 @@ import argparse
 import sys
 import time
 
-GEMM_SHAPES = {          # name: (N, K, mode)   mode: plain | resid | swiglu | f32
-    "qkv": (3072, 2048, "plain"), "o": (2048, 2048, "resid"), "gate_up": (16384, 2048, "swiglu"),
-    "down": (2048, 8192, "resid"), "lm_head": (128256, 2048, "f32"),
-}
+GEMM_MODES = {"qkv": "plain", "o": "resid", "gate_up": "swiglu", "down": "resid", "lm_head": "f32"}
+
+
+def gemm_shape(name: str, sizes: str = "1b"):
+    """(N, K, mode) of a layer's product at the layer sizes of ``cli.sweep.SHAPES[sizes]``;
+    mode: plain | resid | swiglu | f32 (the epilogue the model runs it with)."""
+    from .sweep import SHAPES
+    cfg = SHAPES[sizes]
+    hidden, inter, d = cfg["hidden_size"], cfg["intermediate_size"], cfg["head_dim"]
+    q, kv = cfg["num_attention_heads"] * d, cfg["num_key_value_heads"] * d
+    n, k = {"qkv": (q + 2 * kv, hidden), "o": (hidden, q), "gate_up": (2 * inter, hidden),
+            "down": (hidden, inter), "lm_head": (cfg["vocab_size"], hidden)}[name]
+    return n, k, GEMM_MODES[name]
 
 
 def _time(calls, reps: int) -> float:
@@ -122,7 +131,7 @@ def gemm(args) -> None:
     from ..ops import kernels as K
 
     dev = torch.device("cuda:0")
-    n, k, mode = GEMM_SHAPES[args.shape]
+    n, k, mode = gemm_shape(args.shape, args.sizes)
     m = args.rows
     copies = min(48, max(4, int(600e6 / (n * k * 2)) + 1))
     x = torch.randn(m, k, device=dev).bfloat16()
@@ -292,7 +301,8 @@ def main(argv=None) -> int:
     a.add_argument("--pair", action="store_true", help="workgroup kernel: a workgroup takes item i and item n-1-i")
     a.add_argument("--graph", action="store_true", help="time the calls inside a HIP graph (no host launch cost)")
     g = sub.add_parser("gemm")
-    g.add_argument("--shape", choices=sorted(GEMM_SHAPES), default="gate_up")
+    g.add_argument("--shape", choices=sorted(GEMM_MODES), default="gate_up")
+    g.add_argument("--sizes", choices=["1b", "3b", "8b"], default="1b", help="whose layer sizes (cli.sweep.SHAPES)")
     g.add_argument("--rows", type=int, default=8)
     g.add_argument("--vendor", action="store_true", help="also time the vendor GEMM on the plain weight")
     g.add_argument("--kernel", choices=["few-rows", "gemv"], default="few-rows",

@@ -72,10 +72,23 @@ def use_partial_sums(m: int, n: int, k: int) -> bool:
 # 12.6 / 8.6 microseconds for Q/K/V, output, gate/up and down against the few-rows kernel's 7.3 /
 # 5.8 / 13.5 / 13.1, and a decode step of one request 0.70 ms against 0.85 (two: 0.78 against 0.86).
 GEMV_MAX_ROWS = 2
+# From 5,120 inputs on a wavefront of that kernel has one row of W in flight, and with two tokens
+# its dot products, not the stream, set its time; the few-rows kernel's time does not depend on
+# one or two tokens.  Alone in a graph, residual epilogue, microseconds for one / two tokens,
+# matrix-vector against few-rows kernel: [3072 x 5120] 7.6 / 10.4 against 9.8 / 9.8, [4096 x 7168]
+# 12.4 / 17.4 against 13.1 / 13.1, [3072 x 8192] 12.8 / 15.5 against 11.9 / 11.9, [8192 x 8192]
+# 26.6 / 33.4 against 24.6 / 24.7; with 2,048 rows of W the matrix-vector kernel wins at every K
+# ([2048 x 8192]: 8.8 / 10.6 against 10.7 / 10.9), and at K up to 4,096 the two are within 4 %.
+# Decode steps of one / two requests at the 3B sizes (8 layers; the down projection is
+# [3072 x 8192]): 0.552 / 0.614 -> 0.535 / 0.577 ms.
+GEMV_WIDE_N = 3072
+GEMV_LONG_K = {1: 8192, 2: 5120}
 
 
 def use_gemv(m: int, n: int, k: int) -> bool:
-    return m <= GEMV_MAX_ROWS and K.gemv_supported(m, n, k)
+    if m > GEMV_MAX_ROWS or not K.gemv_supported(m, n, k):
+        return False
+    return not (n >= GEMV_WIDE_N and k >= GEMV_LONG_K[m] and K.gemm_skinny_supported(m, n, k))
 
 
 def decode_tune_rows(max_rows: int) -> list:

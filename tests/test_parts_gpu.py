@@ -283,6 +283,13 @@ def test_linear_chooses_its_kernel_by_rows_and_width(gpu):
         want = plain.linear(x.float(), w512.to(torch.bfloat16).float())
         assert err(lin512(x.to(gpu)), want) <= TOL["bfloat16"]
         assert err(lin512(x.to(gpu), out_dtype=torch.float32), want) <= 2e-5
+    # many long rows: a second token costs the matrix-vector kernel more than the few-rows kernel takes
+    wide = rnd(3072, 5120, scale=0.02).to(torch.bfloat16)
+    lin = Linear(wide.to(gpu))
+    assert lin.fused_kernel(1, torch.bfloat16) == Linear.GEMV and lin.fused_kernel(2, torch.bfloat16) == Linear.FEW_ROWS
+    for rows in (1, 2):
+        x = rnd(rows, 5120).to(torch.bfloat16)
+        assert err(lin(x.to(gpu), out_dtype=torch.float32), plain.linear(x.float(), wide.float())) <= 2e-5
 
 
 @pytest.mark.parametrize("rows", [1, 2, 5])

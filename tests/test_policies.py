@@ -129,3 +129,20 @@ def test_row_counts_timed_for_decode_batches_cover_every_batch_above_the_few_row
         rows = decode_tune_rows(seats)
         for batch in range(17, seats + 1):
             assert any(batch <= r <= 2 * batch for r in rows), (seats, batch)
+
+
+def test_which_products_of_one_or_two_tokens_take_the_matrix_vector_kernel():
+    from kv_cache_optimization_for_llm_amd.ops.gemm_bf16 import use_gemv
+    # the four products of a layer and the head at the 1B and 8B sizes: every one the kernel has an instance for
+    for n, k in ((3072, 2048), (2048, 2048), (16384, 2048), (2048, 8192), (128256, 2048),
+                 (6144, 4096), (4096, 4096), (28672, 4096), (128256, 4096)):
+        assert use_gemv(1, n, k) and use_gemv(2, n, k), (n, k)
+    assert not use_gemv(1, 4096, 14336)                 # no instance for that K
+    assert not use_gemv(3, 2048, 2048)
+    # the 3B sizes: all but the down projection, whose rows are long and many
+    for n, k in ((5120, 3072), (3072, 3072), (16384, 3072), (128256, 3072)):
+        assert use_gemv(1, n, k) and use_gemv(2, n, k), (n, k)
+    assert not use_gemv(1, 3072, 8192) and not use_gemv(2, 3072, 8192)
+    # long rows cost a second token more than a first one
+    assert use_gemv(1, 4096, 5120) and not use_gemv(2, 4096, 5120)
+    assert use_gemv(1, 2048, 8192) and use_gemv(2, 2048, 8192)
