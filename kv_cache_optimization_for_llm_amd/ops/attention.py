@@ -138,10 +138,16 @@ _SHARED_MAX_HEAD_DIM = 128
 # Head size 128 (8 layers of the 8B sizes, ms a step, one wavefront a range -> this rule): 24 / 32
 # requests at 768 keys 1.194 / 1.213 -> 1.147 / 1.177 and 24 at 8,448 keys 2.281 -> 2.161, but 48
 # requests (384 pairs, unsplit before) 1.324 -> 1.373 and 3.109 -> 3.176, and 8 requests at 8,448 keys
-# in 16 ranges, four to a workgroup, 1.319 -> 1.337: there the four ranges end at 384 pairs and many
-# ranges keep a wavefront each.
+# in 16 ranges, four to a workgroup, 1.319 -> 1.337: there the four ranges ended at 384 pairs and many
+# ranges keep a wavefront each.  Measured again from 20 to 47 requests (8 layers of the 3B / 8B sizes,
+# four ranges in a workgroup against what else is chosen - two ranges in a workgroup or three with
+# the merge kernel): up to 24 requests the four win (3B, 20 / 24 requests at 700 keys 0.848 / 0.869
+# -> 0.821 / 0.831 ms, at 2,000 keys 1.010 / 1.060 -> 0.972 / 1.009), at 28 and 32 a tie, from 33 on
+# they lose (3B, 36 / 44 requests at 700 keys 0.974 / 1.001 -> 0.954 / 0.952, 33 / 40 / 47 at 2,000 keys
+# 1.287 / 1.320 / 1.365 -> 1.211 / 1.268 / 1.331, at 8,100 keys 2.21 / 2.38 / 2.50 -> 2.08 / 2.32 / 2.47;
+# 8B 1-4 % alike): they end at 256 pairs.
 _SHARED_TUNED_HEAD_DIM = 64
-_SHARED_FOUR_BELOW_WIDE = 384
+_SHARED_FOUR_BELOW_WIDE = 257
 _SHARED_FOUR_FROM = 128             # more (item, kv head) pairs than this ...
 _SHARED_FOUR_BELOW = 512            # ... and fewer than this: four ranges in one workgroup
 _SHARED_SHORT_CONTEXT = 1024        # up to this many keys already from ...
