@@ -145,7 +145,12 @@ _SHARED_MAX_HEAD_DIM = 128
 # -> 0.821 / 0.831 ms, at 2,000 keys 1.010 / 1.060 -> 0.972 / 1.009), at 28 and 32 a tie, from 33 on
 # they lose (3B, 36 / 44 requests at 700 keys 0.974 / 1.001 -> 0.954 / 0.952, 33 / 40 / 47 at 2,000 keys
 # 1.287 / 1.320 / 1.365 -> 1.211 / 1.268 / 1.331, at 8,100 keys 2.21 / 2.38 / 2.50 -> 2.08 / 2.32 / 2.47;
-# 8B 1-4 % alike): they end at 256 pairs.
+# 8B 1-4 % alike): they end at 256 pairs.  What followed them there was three ranges and the merge
+# kernel, or two ranges in a workgroup; a wavefront on all keys of its pair, as from 384 pairs on, is
+# ahead of both (33 / 40 / 47 requests, three or two ranges -> one: 3B at 700 keys 0.940 / 0.972 / 0.966 ->
+# 0.904 / 0.925 / 0.961, at 2,000 keys 1.217 / 1.275 / 1.346 -> 1.223 / 1.247 / 1.318, at 8,100 keys
+# 2.09 / 2.31 / 2.48 -> 2.13 / 2.26 / 2.40; 8B 1.27 / 1.30 / 1.27 -> 1.21 / 1.26 / 1.26, 1.49 / 1.54 / 1.63
+# -> 1.47 / 1.49 / 1.62, 2.46 / 2.59 / 2.79 -> 2.41 / 2.54 / 2.70).
 _SHARED_TUNED_HEAD_DIM = 64
 _SHARED_FOUR_BELOW_WIDE = 257
 _SHARED_FOUR_FROM = 128             # more (item, kv head) pairs than this ...
@@ -187,6 +192,8 @@ def choose_decode_ranges(num_items: int, num_kv_heads: int, max_context: int, he
         if splits % 4 == 0 and splits >= _SHARED_MANY and (per >= _SHARED_MIN_KEYS or splits >= _SHARED_MIN_SPLITS) \
                 and (pairs * (splits // 4) >= _SHARED_MIN_WORKGROUPS or max_context <= _SHARED_FEW_BYTES_CONTEXT):
             return splits, per, 4
+    if wide and head_dim <= _SHARED_MAX_HEAD_DIM and pairs >= _SHARED_FOUR_BELOW_WIDE:
+        return 1, 0, 1
     splits, per = choose_splits(num_items, num_kv_heads, max_context, max_splits, decoding=True)
     waves = splits if splits in (2, 4) and head_dim <= _SHARED_MAX_HEAD_DIM else 1
     return splits, per, waves

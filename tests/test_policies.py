@@ -73,8 +73,9 @@ def test_where_decoded_tokens_need_no_merge_launch():
     assert choose_decode_ranges(16, 8, 8192, 64, KERNEL_MAX_SPLITS) == (8, 1024, 1)
     # head size 128: four ranges up to 256 pairs only, and many ranges keep a wavefront each
     assert choose_decode_ranges(32, 8, 768, 128, KERNEL_MAX_SPLITS) == (4, 192, 4)
-    assert choose_decode_ranges(33, 8, 768, 128, KERNEL_MAX_SPLITS) == (3, 256, 1)
-    assert choose_decode_ranges(47, 8, 2048, 128, KERNEL_MAX_SPLITS) == (2, 1024, 2)
+    assert choose_decode_ranges(33, 8, 768, 128, KERNEL_MAX_SPLITS) == (1, 0, 1)
+    assert choose_decode_ranges(47, 8, 2048, 128, KERNEL_MAX_SPLITS) == (1, 0, 1)
+    assert choose_decode_ranges(33, 8, 768, 64, KERNEL_MAX_SPLITS) == (4, 192, 4)
     assert choose_decode_ranges(48, 8, 768, 128, KERNEL_MAX_SPLITS) == (1, 0, 1)
     assert choose_decode_ranges(64, 8, 8192, 128, KERNEL_MAX_SPLITS) == (1, 0, 1)
     assert choose_decode_ranges(8, 8, 8448, 128, KERNEL_MAX_SPLITS)[2] == 1
