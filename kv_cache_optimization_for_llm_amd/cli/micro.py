@@ -180,7 +180,7 @@ def prompt(args) -> None:
     from ..engine.engine import Engine, EngineOptions
     from .sweep import SHAPES
 
-    cfg = dict(SHAPES["1b"])
+    cfg = dict(SHAPES[args.sizes])
     cfg["max_position_embeddings"] = max(8192, args.tokens)
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
@@ -202,8 +202,14 @@ def prompt(args) -> None:
         best = min(best, time.perf_counter() - t0)
         eng.release("p")
     steps = (args.tokens + args.portion - 1) // args.portion
-    print(f"prompt of {args.tokens} in portions of {args.portion} ({steps} steps): {best * 1e3:8.2f} ms  "
-          f"{args.tokens / best:9.0f} tok/s", flush=True)
+    from .sweep import weight_bytes
+    # matrix products: two flops per weight and token (the head only at the wanted row); attention: causal
+    layers, nq, d = cfg["num_hidden_layers"], cfg["num_attention_heads"], cfg["head_dim"]
+    head = cfg["vocab_size"] * cfg["hidden_size"]
+    flops = 2.0 * (weight_bytes(cfg, 1) - head) * args.tokens + 2.0 * head
+    flops += layers * 4.0 * nq * d * args.tokens * (args.tokens + 1) / 2
+    print(f"prompt of {args.tokens} in portions of {args.portion} ({steps} steps, {cfg['num_hidden_layers']} layers of the "
+          f"{args.sizes} sizes): {best * 1e3:8.2f} ms  {args.tokens / best:9.0f} tok/s  {flops / best / 1e12:6.0f} TFLOP/s", flush=True)
 
 
 def stream(args) -> None:
@@ -313,7 +319,8 @@ def main(argv=None) -> int:
     pr = sub.add_parser("prompt")
     pr.add_argument("--tokens", type=int, default=8192)
     pr.add_argument("--portion", type=int, default=512)
-    pr.add_argument("--layers", type=int, default=0, help="fewer layers than the 16 of the shape")
+    pr.add_argument("--sizes", choices=["1b", "3b", "8b"], default="1b", help="whose layer sizes (cli.sweep.SHAPES)")
+    pr.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has")
     pr.add_argument("--reps", type=int, default=4)
     pr.add_argument("--no-graphs", action="store_true")
     pr.add_argument("--tune-gemm", action="store_true", help="time the vendor library's algorithms for the portion's rows first")
