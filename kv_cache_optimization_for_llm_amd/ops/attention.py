@@ -153,6 +153,10 @@ _SHARED_MAX_HEAD_DIM = 128
 # -> 1.47 / 1.49 / 1.62, 2.46 / 2.59 / 2.79 -> 2.41 / 2.54 / 2.70).
 _SHARED_TUNED_HEAD_DIM = 64
 _SHARED_FOUR_BELOW_WIDE = 257
+# ... and at short contexts they begin at 128 pairs, not at 64: 8 / 12 / 16 requests at 700 keys, 16-8
+# ranges with the merge kernel -> four in a workgroup, 3B 0.635 / 0.667 / 0.701 -> 0.639 / 0.676 / 0.694,
+# 8B 0.953 / 1.024 / 1.113 -> 0.960 / 1.040 / 1.095 ms
+_SHARED_FOUR_FROM_SHORT_WIDE = 127
 _SHARED_FOUR_FROM = 128             # more (item, kv head) pairs than this ...
 _SHARED_FOUR_BELOW = 512            # ... and fewer than this: four ranges in one workgroup
 _SHARED_SHORT_CONTEXT = 1024        # up to this many keys already from ...
@@ -176,6 +180,8 @@ def choose_decode_ranges(num_items: int, num_kv_heads: int, max_context: int, he
     if wide:
         below = _SHARED_FOUR_BELOW_WIDE
     frm = _SHARED_FOUR_FROM_SHORT if max_context <= _SHARED_SHORT_CONTEXT else _SHARED_FOUR_FROM
+    if wide and frm < _SHARED_FOUR_FROM_SHORT_WIDE:
+        frm = _SHARED_FOUR_FROM_SHORT_WIDE
     if head_dim <= _SHARED_MAX_HEAD_DIM and frm < pairs < below \
             and max_context >= 4 * _MIN_KEYS_PER_SPLIT_DECODE:
         splits, per = _cut_keys(4, max_context, 4)

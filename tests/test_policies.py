@@ -76,6 +76,10 @@ def test_where_decoded_tokens_need_no_merge_launch():
     assert choose_decode_ranges(33, 8, 768, 128, KERNEL_MAX_SPLITS) == (1, 0, 1)
     assert choose_decode_ranges(47, 8, 2048, 128, KERNEL_MAX_SPLITS) == (1, 0, 1)
     assert choose_decode_ranges(33, 8, 768, 64, KERNEL_MAX_SPLITS) == (4, 192, 4)
+    # ... and from 128 pairs on, where head size 64 shares from 64
+    assert choose_decode_ranges(8, 8, 768, 64, KERNEL_MAX_SPLITS) == (4, 192, 4)
+    assert choose_decode_ranges(12, 8, 768, 128, KERNEL_MAX_SPLITS) == (8, 96, 1)
+    assert choose_decode_ranges(16, 8, 768, 128, KERNEL_MAX_SPLITS) == (4, 192, 4)
     assert choose_decode_ranges(48, 8, 768, 128, KERNEL_MAX_SPLITS) == (1, 0, 1)
     assert choose_decode_ranges(64, 8, 8192, 128, KERNEL_MAX_SPLITS) == (1, 0, 1)
     assert choose_decode_ranges(8, 8, 8448, 128, KERNEL_MAX_SPLITS)[2] == 1
