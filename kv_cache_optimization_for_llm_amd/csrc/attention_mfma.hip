@@ -773,6 +773,8 @@ static size_t kva_attention_mfma_exchange_bytes(int waves, int head_dim) {
     return waves > 1 ? (size_t)(waves - 1) * (head_dim / 16 * 4 + 2) * KVA_WAVE * sizeof(float) : 0;
 }
 
+// `out` null (more than one partial result a row left, splits / waves > 1): no merge launch; the
+// partial results in part_o / part_ml are the call's result (kva_gemv_merged adds them up).
 extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, const void *q,
                                   int q_row_stride, const void *k_cache, const void *v_cache,
                                   const int *block_table, int max_blocks, const int *item_meta,
@@ -798,6 +800,8 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
     KVA_REQUIRE(splits == 1 || (keys_per_split > 0 && keys_per_split % 32 == 0),
                 "attention_mfma: splits need a key count that is a multiple of 32");
     KVA_REQUIRE(splits == waves || (part_o && part_ml), "attention_mfma: key ranges of several workgroups need a workspace");
+    // without `out` the partial results (splits / waves a row) are left to the caller: no merge launch
+    KVA_REQUIRE(out != nullptr || splits / waves > 1, "attention_mfma: no output");
     KVA_REQUIRE(window >= 0, "attention_mfma: negative window");
     KVA_REQUIRE(scale > 0.f, "attention_mfma: the score scale must be positive");
     KVA_REQUIRE(row_tiles == 1 || row_tiles == kva_attention_mfma_row_tiles(head_dim, 1),
@@ -834,7 +838,7 @@ extern "C" int kva_attention_mfma(void *out, float *part_o, float *part_ml, cons
 #undef CASE
 #undef LAUNCH
     KVA_CHECK_LAUNCH("attention_mfma");
-    if (splits / waves > 1)
+    if (splits / waves > 1 && out != nullptr)
         return kva_attention_merge_launch(out, part_o, part_ml, head_dim, splits / waves, item_meta, item_entry, item_row0,
                                           entry_q_start, num_items, 16 * row_tiles, total_rows, num_q_heads,
                                           num_kv_heads, all_rows, stream);

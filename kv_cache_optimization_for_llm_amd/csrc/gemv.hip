@@ -44,6 +44,11 @@ struct GemvArgs {
     bf16_t *scaled_out;
     float *sumsq_out;            // [M, one part per workgroup and round]
     int parts_out;
+    // GV_RESID with X given as the partial results of an attention kernel's key ranges (X null):
+    // part_o [M * heads, parts, part_head_dim], part_ml [M * heads, parts] (maximum in the base-2
+    // domain, sum), heads = K / part_head_dim
+    const float *part_o, *part_ml;
+    int parts, part_head_dim;
     // GV_ROPE (Y is the Q output, row stride ldy)
     const float *cos_t, *sin_t;
     const int *positions, *slots;
@@ -77,6 +82,8 @@ constexpr int GV_WAVES = 4;          // wavefronts per workgroup
 // load, wait, add takes over, and that wait is for every load in flight, the rows of W included:
 // 0.8 us of the Q/K/V product's 5.5 when four were asked for here.
 constexpr int GV_NORM_LOADS = 8;
+// Partial results of key ranges per row that the merged form adds up (a lane holds 10 floats of each).
+constexpr int GV_MERGE_MAX_PARTS = 4;
 
 // KV: 16-byte vectors per lane and row (K = 512 KV); M: tokens; RB: rows a wavefront has in flight.
 // Row r of unit u: plain / residual: u RB + r.  SwiGLU (RB even): pair t = r / 2 of the unit is
@@ -87,7 +94,14 @@ constexpr int GV_NORM_LOADS = 8;
 // W, the partial sums that finish the input's norm, and what its epilogue needs (the residual
 // stream and the next norm's weight, or the rotation's cosines and sines).  After the wavefront
 // reductions every lane has every sum, and lane l finishes pair (row l % RB, token l / RB).
-template <int KV, int M, int RB, int EPI>
+//
+// MERGED (residual epilogue, K up to 4,096): the token(s) are not read but made - the output
+// projection of an attention layer takes the partial results that the attention kernel left per
+// key range (at most GV_MERGE_MAX_PARTS a row) and adds them up itself, as the merge kernel would
+// (weights 2^(m_s - max m), the sum divided by the weighted sum of the l_s, rounded to bf16), so
+// that one or two decoded tokens need no merge launch.  The wavefronts of a workgroup share the
+// work: wavefront w makes the columns of vectors c = w, w + GV_WAVES, ... and leaves them in LDS.
+template <int KV, int M, int RB, int EPI, bool MERGED = false>
 __global__ void __launch_bounds__(64 * GV_WAVES) gemv_kernel(const GemvArgs a) {
     const int lane = threadIdx.x & 63, wave_in_block = threadIdx.x >> 6;
     const int K = a.K;
@@ -131,11 +145,36 @@ __global__ void __launch_bounds__(64 * GV_WAVES) gemv_kernel(const GemvArgs a) {
 
     // the token(s), kept packed: lane l owns columns (64 c + l) * 8 .. + 8
     uint4 xp[M][KV];
+    constexpr int MINE = MERGED ? (KV + GV_WAVES - 1) / GV_WAVES : 1;     // vectors this wavefront makes per token
+    float2 pml[MINE][M][GV_MERGE_MAX_PARTS];
+    float4 pov[MINE][M][GV_MERGE_MAX_PARTS][2];
+    if constexpr (MERGED) {
+        const int heads = K / a.part_head_dim;
 #pragma unroll
-    for (int m = 0; m < M; ++m)
+        for (int i = 0; i < MINE; ++i) {
+            const int c = min(wave_in_block + i * GV_WAVES, KV - 1);
+            const int col = (c * 64 + lane) * 8;
+            const int head = col / a.part_head_dim, j0 = col - head * a.part_head_dim;
 #pragma unroll
-        for (int c = 0; c < KV; ++c)
-            xp[m][c] = *reinterpret_cast<const uint4 *>(a.X + (size_t)m * a.ldx + (c * 64 + lane) * 8);
+            for (int m = 0; m < M; ++m) {
+                const size_t row = (size_t)m * heads + head;
+#pragma unroll
+                for (int sp = 0; sp < GV_MERGE_MAX_PARTS; ++sp) {
+                    const int ss = min(sp, a.parts - 1);                      // masked where they are added
+                    pml[i][m][sp] = reinterpret_cast<const float2 *>(a.part_ml)[row * a.parts + ss];
+                    const float4 *po = reinterpret_cast<const float4 *>(a.part_o + (row * a.parts + ss) * a.part_head_dim + j0);
+                    pov[i][m][sp][0] = po[0];
+                    pov[i][m][sp][1] = po[1];
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+#pragma unroll
+            for (int c = 0; c < KV; ++c)
+                xp[m][c] = *reinterpret_cast<const uint4 *>(a.X + (size_t)m * a.ldx + (c * 64 + lane) * 8);
+    }
     uint4 w[RB][KV];
     // asks for the rows of W of unit u (an index past the end takes the last unit's rows again)
     auto ask_for_rows = [&](int u) {
@@ -166,6 +205,43 @@ __global__ void __launch_bounds__(64 * GV_WAVES) gemv_kernel(const GemvArgs a) {
     const float inv_width = a.sumsq != nullptr ? 1.f / (float)a.norm_width : 1.f;
     // everything is asked for before anything is waited for
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (MERGED) {
+        __shared__ uint4 merged_x[M][KV * 64];
+#pragma unroll
+        for (int i = 0; i < MINE; ++i) {
+            const int c = wave_in_block + i * GV_WAVES;
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                float mx = -INFINITY;
+#pragma unroll
+                for (int sp = 0; sp < GV_MERGE_MAX_PARTS; ++sp)
+                    if (sp < a.parts) mx = fmaxf(mx, pml[i][m][sp].x);
+                float denom = 0.f, acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int sp = 0; sp < GV_MERGE_MAX_PARTS; ++sp) {
+                    if (sp < a.parts) {
+                        const float wgt = pml[i][m][sp].x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(pml[i][m][sp].x - mx);
+                        denom += pml[i][m][sp].y * wgt;
+                        const float4 lo = pov[i][m][sp][0], hi = pov[i][m][sp][1];
+                        acc[0] += lo.x * wgt; acc[1] += lo.y * wgt; acc[2] += lo.z * wgt; acc[3] += lo.w * wgt;
+                        acc[4] += hi.x * wgt; acc[5] += hi.y * wgt; acc[6] += hi.z * wgt; acc[7] += hi.w * wgt;
+                    }
+                }
+                const float inv = 1.f / denom;
+                uint32_t pk[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    pk[j] = (uint32_t)float_to_bf16_bits(acc[2 * j] * inv) |
+                            ((uint32_t)float_to_bf16_bits(acc[2 * j + 1] * inv) << 16);
+                if (c < KV) merged_x[m][c * 64 + lane] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+#pragma unroll
+            for (int c = 0; c < KV; ++c) xp[m][c] = merged_x[m][c * 64 + lane];
+    }
     float rinv[M];
 #pragma unroll
     for (int m = 0; m < M; ++m) {
@@ -344,6 +420,29 @@ int launch(const GemvArgs &a, hipStream_t stream) {
     else if (EPI == GV_ROPE) units = (long)(a.nq + 2 * a.nkv) * (a.head_dim / 2 / (rb / 2));
     else units = (a.N + rb - 1) / rb;
     const dim3 grid((unsigned)std::min<long>(2048, (units + GV_WAVES - 1) / GV_WAVES)), block(64 * GV_WAVES);
+    if constexpr (EPI == GV_RESID) {
+        if (a.part_o != nullptr) {
+#define GVP(KVV, RBB)                                                                                          \
+    if (a.M == 1) hipLaunchKernelGGL((gemv_kernel<KVV, 1, RBB, GV_RESID, true>), grid, block, 0, stream, a);  \
+    else hipLaunchKernelGGL((gemv_kernel<KVV, 2, RBB, GV_RESID, true>), grid, block, 0, stream, a)
+            switch (kv) {
+            case 1: GVP(1, 8); break;
+            case 2: GVP(2, 8); break;
+            case 3: GVP(3, 2); break;
+            case 4: GVP(4, 2); break;
+            case 5: GVP(5, 2); break;
+            case 6: GVP(6, 2); break;
+            case 7: GVP(7, 2); break;
+            case 8: GVP(8, 2); break;
+            default:
+                kva_set_error("gemv: K=%d has no instance that adds up partial results", a.K);
+                return KVA_ERR_ARG;
+            }
+#undef GVP
+            KVA_CHECK_LAUNCH("gemv");
+            return KVA_OK;
+        }
+    }
 #define GV(KVV, MM, RBB) hipLaunchKernelGGL((gemv_kernel<KVV, MM, RBB, EPI>), grid, block, 0, stream, a)
 #define GVM(KVV, RBB)                                                                          \
     if (a.M == 1) GV(KVV, 1, RBB); else GV(KVV, 2, RBB)
@@ -438,6 +537,35 @@ extern "C" int kva_gemv(void *Y, const void *X, const void *W, int M, int N, int
     }
     KVA_REQUIRE(ldy >= N, "gemv: Y row stride %d is smaller than its %d columns", ldy, N);
     return launch<GV_PLAIN>(a, stream);
+}
+
+// Whether kva_gemv_merged takes these sizes: one or two tokens, K up to 4,096 with an instance,
+// heads of a multiple of 8 features that divide K, 2 to GV_MERGE_MAX_PARTS partial results a row.
+extern "C" int kva_gemv_merged_supported(int M, int N, int K, int head_dim, int parts) {
+    return (kva_gemv_supported(M, N, K) && K <= 4096 && head_dim >= 8 && head_dim % 8 == 0 && K % head_dim == 0 &&
+            parts >= 2 && parts <= GV_MERGE_MAX_PARTS) ? 1 : 0;
+}
+extern "C" int kva_gemv_merge_max_parts() { return GV_MERGE_MAX_PARTS; }
+
+// kva_gemv's mode 3 (hidden[M, N] += X W^T, the next norm prepared) with X = the attention output
+// of M decoded tokens given as what the attention kernel left per key range: part_o
+// [M * (K / head_dim), parts, head_dim] fp32, part_ml [M * (K / head_dim), parts, 2] fp32
+// (maximum in the base-2 domain, sum).  Stands for the merge kernel followed by kva_gemv.
+extern "C" int kva_gemv_merged(const float *part_o, const float *part_ml, int parts, int head_dim, const void *W,
+                               int M, int N, int K, void *hidden, const void *next_w, int next_w_f32,
+                               void *scaled_out, float *sumsq_out, hipStream_t stream) {
+    KVA_REQUIRE(kva_gemv_merged_supported(M, N, K, head_dim, parts),
+                "gemv_merged: M=%d N=%d K=%d head_dim=%d parts=%d not supported", M, N, K, head_dim, parts);
+    KVA_REQUIRE(part_o && part_ml && ((uintptr_t)part_o % 16) == 0 && ((uintptr_t)part_ml % 8) == 0,
+                "gemv_merged: aligned partial results are needed");
+    KVA_REQUIRE(hidden && scaled_out && sumsq_out && W, "gemv_merged: hidden, scaled_out, sumsq_out and W are needed");
+    GemvArgs a = {};
+    a.W = (const bf16_t *)W; a.M = M; a.N = N; a.K = K; a.ldx = K;
+    a.part_o = part_o; a.part_ml = part_ml; a.parts = parts; a.part_head_dim = head_dim;
+    a.hidden = (bf16_t *)hidden; a.next_w = next_w; a.next_w_f32 = next_w_f32;
+    a.scaled_out = (bf16_t *)scaled_out; a.sumsq_out = sumsq_out;
+    a.parts_out = kva_gemv_sumsq_parts(N, K);
+    return launch<GV_RESID>(a, stream);
 }
 
 // The joined Q/K/V projection of one or two tokens with rotation and cache write: as

@@ -205,6 +205,34 @@ def choose_decode_ranges(num_items: int, num_kv_heads: int, max_context: int, he
     return splits, per, waves
 
 
+# One or two decoded tokens whose output projection adds partial results up itself
+# (ops.kernels.gemv_merged): four ranges to a workgroup and one partial result per workgroup, so the
+# merge kernel (3.7 us a layer for kilobytes) is not launched.  Whole decode steps at the 1B sizes,
+# ms, merge kernel -> this: one request at 400 / 768 / 1,900 keys 0.686 / 0.688 / 0.703 -> 0.667 / 0.660 /
+# 0.681, two requests at 768 / 1,900 keys 0.769 / 0.783 -> 0.741 / 0.766.  Up to 2,048 keys (contexts are
+# rounded up to a power of two when a step is captured): with at most 4 partial results a row 4,096
+# keys are 16 ranges of 256, and one request at 3,000 / 8,000 keys went 0.719 / 0.741 -> 0.722 / 0.805.
+# Head sizes up to 64, where it was measured (at 128, with wider output projections: parts/linear.py).
+_LEFT_MAX_ITEMS = 2
+_LEFT_MIN_KEYS = 64
+_LEFT_MAX_CONTEXT = 2048
+
+
+def choose_left_ranges(num_items: int, max_context: int, head_dim: int, max_parts: int):
+    """(key ranges, keys per range, 4) for decoded tokens whose consumer takes up to ``max_parts``
+    partial results a row, or None where the ordinary choice stands."""
+    if num_items > _LEFT_MAX_ITEMS or head_dim > _SHARED_TUNED_HEAD_DIM or max_parts < 2 \
+            or max_context > _LEFT_MAX_CONTEXT:
+        return None
+    # a multiple of four ranges whatever the context: the last ones may hold few keys or none (a
+    # range without a key weighs nothing when the results are added up)
+    want = min(4 * max_parts, max_context // _LEFT_MIN_KEYS) // 4 * 4
+    if want < 8:
+        return None
+    per = ((max_context + want - 1) // want + 31) // 32 * 32
+    return want, per, 4
+
+
 def choose_lds_splits(groups: int, max_context: int, max_splits: int = None, head_dim: int = 64) -> tuple:
     """(splits, keys_per_split) for the workgroup kernel, under the same limit."""
     if max_splits is None:
@@ -215,12 +243,12 @@ def choose_lds_splits(groups: int, max_context: int, max_splits: int = None, hea
     return _cut_keys(min(want, max(1, max_context // min_keys)), max_context, max_splits)
 
 
-def _plan_for(batch, kv, num_q_heads: int, num_kv_heads: int, head_dim: int) -> list:
+def _plan_for(batch, kv, num_q_heads: int, num_kv_heads: int, head_dim: int, max_parts: int = 0) -> list:
     plans = batch.attention_plans
-    key = (num_q_heads, num_kv_heads, head_dim, kv.page_size)
+    key = (num_q_heads, num_kv_heads, head_dim, kv.page_size, max_parts)
     plan = plans.get(key)
     if plan is None:
-        plan = plans[key] = _plan(batch, num_q_heads // num_kv_heads, num_kv_heads, head_dim, kv.page_size)
+        plan = plans[key] = _plan(batch, num_q_heads // num_kv_heads, num_kv_heads, head_dim, kv.page_size, max_parts)
     return plan
 
 
@@ -237,7 +265,8 @@ def rotates_in_kernel(batch, kv, num_q_heads: int, num_kv_heads: int, head_dim: 
 
 
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads: int,
-                    num_kv_heads: int, head_dim: int, scale: float, window: int = 0, rope=None) -> torch.Tensor:
+                    num_kv_heads: int, head_dim: int, scale: float, window: int = 0, rope=None,
+                    max_parts: int = 0):
     """Causal GQA attention of the step's tokens over the paged cache.  ``qkv`` is the fused
     projection output ``[T, (nq + 2 nkv) d]`` (or just its Q part) whose first ``nq * d`` columns
     are the (already position-encoded) queries; keys and values are read from ``kv``.
@@ -248,7 +277,11 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
     chip, else the one-wavefront kernel with two row tiles.  A step that holds both is two
     launches, each over its own entries.  Which kernels, over which work items and key splits, is
     decided once per step and geometry (every layer of a model asks the same) and kept with the
-    batch."""
+    batch.
+
+    ``max_parts`` > 0: the caller can take the output of one or two decoded tokens as up to so
+    many partial results a row (``ops.kernels.AttentionPartials``, returned instead of ``out``,
+    which is then not written) - where the keys are cut that way no merge kernel runs."""
     if kv is None:
         raise K.KernelError("paged_attention: the mixer has no cache view")
     if rope is not None:
@@ -265,15 +298,19 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
         return K.attention_rowwise(qkv, qkv.shape[1], out, kv.k_cache, kv.v_cache, kv.block_table,
                                    batch.tok_seat, batch.positions, num_q_heads, num_kv_heads,
                                    head_dim, scale, window)
-    plan = _plan_for(batch, kv, num_q_heads, num_kv_heads, head_dim)
+    plan = _plan_for(batch, kv, num_q_heads, num_kv_heads, head_dim, max_parts)
     stride = qkv.shape[1]
     for launch in plan:
         if launch[0] == "wave":
             _, (item_entry, item_row0, meta), tiles, splits, per, pair, covers_all, keep_cached, waves = launch
-            K.attention_mfma(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table, item_entry, item_row0,
-                             batch.entry_seat, batch.entry_q_start, batch.entry_start_pos, num_q_heads,
-                             num_kv_heads, head_dim, scale, window, splits, per, tiles, pair, meta,
-                             covers_all_rows=covers_all, keep_cached=keep_cached, waves=waves)
+            left = max_parts > 0 and len(plan) == 1 and covers_all and 2 <= splits // waves <= max_parts
+            got = K.attention_mfma(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table, item_entry, item_row0,
+                                   batch.entry_seat, batch.entry_q_start, batch.entry_start_pos, num_q_heads,
+                                   num_kv_heads, head_dim, scale, window, splits, per, tiles, pair, meta,
+                                   covers_all_rows=covers_all, keep_cached=keep_cached, waves=waves,
+                                   leave_partials=left)
+            if left:
+                return got
         else:
             _, meta, splits, per, covers_all = launch
             K.attention_lds(qkv, stride, out, kv.k_cache, kv.v_cache, kv.block_table, meta, num_q_heads,
@@ -281,7 +318,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, kv, batch, num_q_heads
     return out
 
 
-def _plan(batch, group: int, num_kv_heads: int, head_dim: int, page_size: int) -> list:
+def _plan(batch, group: int, num_kv_heads: int, head_dim: int, page_size: int, max_parts: int = 0) -> list:
     """The launches of one attention call over ``batch``: ("wave", items, row tiles, splits, keys per
     split, pair, covers all rows, keep cached, wavefronts of a workgroup that share an item) and
     ("lds", item records, splits, keys per split, covers all rows)."""
@@ -296,6 +333,9 @@ def _plan(batch, group: int, num_kv_heads: int, head_dim: int, page_size: int) -
         # so only the small ones)
         small = n * batch.max_context * num_kv_heads * head_dim * 4 <= _KEEP_CACHED_BYTES
         splits, per, waves = choose_decode_ranges(n, num_kv_heads, batch.max_context, head_dim)
+        if max_parts > 0 and which == "all":
+            splits, per, waves = choose_left_ranges(batch.num_tokens, batch.max_context, head_dim, max_parts) \
+                or (splits, per, waves)
         # (not where wavefronts share a workgroup: 8 / 16 / 32 requests of 768 keys in four ranges
         # 0.854 / 0.942 / 1.154 ms through the caches, 0.848 / 0.938 / 1.124 past them; 4 requests of
         # 2,048 keys, a wavefront a range, 0.863 against 0.875)

@@ -165,6 +165,40 @@ class PartialSums:
         return total.to(torch.bfloat16)
 
 
+class AttentionPartials:
+    """An attention output that has not been added up yet: what :func:`attention_mfma` leaves per
+    key range when it is told to (``leave_partials``): ``part_o`` fp32 ``[tokens * heads, parts,
+    head_dim]`` and ``part_ml`` fp32 ``[tokens * heads, parts, 2]`` (maximum in the base-2 domain,
+    sum of exponentials).  It stands where the bf16 ``[tokens, heads * head_dim]`` output stands,
+    for a consumer that adds the ranges up itself (:func:`gemv_merged`)."""
+
+    def __init__(self, part_o: torch.Tensor, part_ml: torch.Tensor, tokens: int, heads: int):
+        if part_o.dim() != 3 or part_o.dtype != torch.float32 or part_o.shape[0] != tokens * heads \
+                or part_ml.shape != (tokens * heads, part_o.shape[1], 2) or part_ml.dtype != torch.float32:
+            raise KernelError("AttentionPartials: fp32 [tokens * heads, parts, head_dim] and [tokens * heads, parts, 2] needed")
+        self.part_o, self.part_ml, self.tokens, self.heads = part_o, part_ml, tokens, heads
+
+    @property
+    def parts(self) -> int:
+        return self.part_o.shape[1]
+
+    @property
+    def head_dim(self) -> int:
+        return self.part_o.shape[2]
+
+    @property
+    def shape(self):
+        return (self.tokens, self.heads * self.head_dim)
+
+    @property
+    def dtype(self):
+        return torch.bfloat16
+
+    @property
+    def device(self):
+        return self.part_o.device
+
+
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
             delta=None, row_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out = rmsnorm(x) * weight.  With ``delta`` (a tensor like x, or :class:`PartialSums`): x +=
@@ -436,7 +470,7 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
                    scale: float, window: int = 0, splits: int = 1, keys_per_split: int = 0,
                    row_tiles: int = 1, pair: bool = False,
                    item_meta: Optional[torch.Tensor] = None, covers_all_rows: bool = True,
-                   keep_cached: bool = False, waves: int = 1) -> torch.Tensor:
+                   keep_cached: bool = False, waves: int = 1, leave_partials: bool = False):
     """bf16 matrix-core attention over the paged cache.  Items are (entry, first query row) pairs
     of ``16 * row_tiles`` query rows each, row = token_in_step * (nq / nkv) + head_in_group.
     With ``pair`` one wavefront takes item i and item n-1-i of the list (give the list ordered by
@@ -449,10 +483,14 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
     short contexts that are still in the memory-side cache when the next step reads them.
     ``waves`` (1, 2 or 4; items of one row tile, head sizes up to 128): so many of the ``splits``
     key ranges go to the wavefronts of one workgroup, which adds their results up itself; only
-    ``splits // waves`` partial results per row are left for the merge (none: no merge launch)."""
+    ``splits // waves`` partial results per row are left for the merge (none: no merge launch).
+    ``leave_partials`` (the items cover every row of the step): where more than one partial result
+    a row is left they are not merged into ``out`` but returned as :class:`AttentionPartials`."""
     tokens = out.shape[0]
     if out.dtype != torch.bfloat16 or q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16:
         raise KernelError("attention_mfma: bfloat16 only")
+    if leave_partials and not covers_all_rows:
+        raise KernelError("attention_mfma: partial results can only be left for a launch that covers every row")
     if waves < 1 or splits % waves:
         raise KernelError(f"attention_mfma: {waves} wavefronts per item do not divide {splits} key ranges")
     if out.shape != (tokens, num_q_heads * head_dim):
@@ -471,8 +509,9 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
     if splits // waves > 1:
         part_o = torch.empty((tokens * num_q_heads, splits // waves, head_dim), dtype=torch.float32, device=out.device)
         part_ml = torch.empty((tokens * num_q_heads, splits // waves, 2), dtype=torch.float32, device=out.device)
+    left = leave_partials and part_o is not None
     check(hip_lib().kva_attention_mfma(
-        _dev(out, "out"), _opt(part_o, "part_o"), _opt(part_ml, "part_ml"),
+        None if left else _dev(out, "out"), _opt(part_o, "part_o"), _opt(part_ml, "part_ml"),
         _dev(q, "q", contiguous=False), q_row_stride, _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
         _dev(block_table, "block_table", torch.int32), block_table.shape[1],
         _opt(item_meta, "item_meta", torch.int32),
@@ -482,7 +521,7 @@ def attention_mfma(q: torch.Tensor, q_row_stride: int, out: torch.Tensor, k_cach
         num_kv_heads, head_dim, k_cache.shape[3], float(scale), int(window), int(splits),
         int(keys_per_split), 1 if pair else 0, 1 if covers_all_rows else 0, 1 if keep_cached else 0,
         int(waves), _stream()), "attention_mfma")
-    return out
+    return AttentionPartials(part_o, part_ml, tokens, num_q_heads) if left else out
 
 
 def attention_mfma_rope_supported(head_dim: int, page_size: int, group: int) -> bool:
@@ -899,6 +938,41 @@ def gemv(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor], swiglu: 
     return out
 
 
+def gemv_merged_supported(m: int, n: int, k: int, head_dim: int, parts: int) -> bool:
+    """Whether :func:`gemv_merged` takes ``m`` tokens of ``k / head_dim`` heads with ``parts``
+    partial results each."""
+    return bool(hip_lib().kva_gemv_merged_supported(int(m), int(n), int(k), int(head_dim), int(parts)))
+
+
+def gemv_merge_max_parts() -> int:
+    return int(hip_lib().kva_gemv_merge_max_parts())
+
+
+def gemv_merged(x: AttentionPartials, w: torch.Tensor, hidden: torch.Tensor, next_weight: Optional[torch.Tensor],
+                scaled_out: torch.Tensor, sumsq_out: torch.Tensor) -> torch.Tensor:
+    """:func:`gemv` with its residual epilogue over an attention output that is still in partial
+    results per key range: the kernel adds them up (as the merge kernel would, rounded to bf16)
+    where it would have read the tokens."""
+    m, k = x.shape
+    n = w.shape[0]
+    if w.dim() != 2 or w.dtype != torch.bfloat16 or w.shape[1] != k or not w.is_contiguous():
+        raise KernelError(f"gemv_merged: partial results of {tuple(x.shape)} do not fit a row-major bf16 weight {tuple(w.shape)}")
+    if not gemv_merged_supported(m, n, k, x.head_dim, x.parts):
+        raise KernelError(f"gemv_merged: {m} tokens, weight {tuple(w.shape)}, heads of {x.head_dim}, {x.parts} partial results: not supported")
+    p_out = gemv_sumsq_parts(n, k)
+    if hidden.shape != (m, n) or hidden.dtype != torch.bfloat16 or scaled_out.shape != (m, n) \
+            or scaled_out.dtype != torch.bfloat16 or sumsq_out.shape != (m, p_out):
+        raise KernelError(f"gemv_merged: hidden / scaled_out [M, N] bf16 and sumsq_out [M, {p_out}] needed")
+    if next_weight is not None and next_weight.shape != (n,):
+        raise KernelError("gemv_merged: the next norm's weight must be [N]")
+    check(hip_lib().kva_gemv_merged(
+        _dev(x.part_o, "part_o", torch.float32), _dev(x.part_ml, "part_ml", torch.float32), x.parts, x.head_dim,
+        _dev(w, "w"), m, n, k, _dev(hidden, "hidden"), _opt(next_weight, "next_weight"),
+        1 if next_weight is not None and next_weight.dtype == torch.float32 else 0,
+        _dev(scaled_out, "scaled_out"), _dev(sumsq_out, "sumsq_out", torch.float32), _stream()), "gemv_merged")
+    return hidden
+
+
 def gemv_qkv_rope_supported(m: int, k: int, head_dim: int) -> bool:
     return bool(hip_lib().kva_gemv_qkv_rope_supported(int(m), int(k), int(head_dim)))
 
@@ -967,7 +1041,7 @@ KERNEL_CLASSES = {
     "attention_mfma_rope": "attention",
     "gemm_nt_f32": "gemm fp32", "gemm_vendor": "gemm (vendor library)",
     "gemm_skinny": "gemm (few rows)", "gemm_skinny_qkv_rope": "gemm (few rows)",
-    "gemv": "gemm (few rows)", "gemv_qkv_rope": "gemm (few rows)",
+    "gemv": "gemm (few rows)", "gemv_qkv_rope": "gemm (few rows)", "gemv_merged": "gemm (few rows)",
     "sample": "sampling", "mark_tokens": "sampling",
 }
 

@@ -142,8 +142,13 @@ class GQAAttention(Mixer):
         batch, kv = ctx.batch, ctx.kv
         qkv = self.qkv(x, batch, kv)
         out = torch.empty((x.shape[0], self.num_heads * self.head_dim), dtype=x.dtype, device=x.device)
-        attn_ops.paged_attention(qkv, out, kv, batch, self.num_heads, self.num_kv_heads,
-                                 self.head_dim, self.scale, self.window, rope=self.qkv.pending_rotation)
+        # an output projection that adds the key ranges' partial results up itself (one or two
+        # decoded tokens) is told so: the attention kernel may then leave them unmerged
+        max_parts = self.o.takes_attention_partials(x.shape[0], x.dtype, tail, self.head_dim) \
+            if self.qkv.pending_rotation is None else 0
+        out = attn_ops.paged_attention(qkv, out, kv, batch, self.num_heads, self.num_kv_heads,
+                                       self.head_dim, self.scale, self.window, rope=self.qkv.pending_rotation,
+                                       max_parts=max_parts)
         if tail is not None:
             fused = self.o.into_residual(out, tail)
             if fused is not None:

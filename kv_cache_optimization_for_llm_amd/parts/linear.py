@@ -34,6 +34,12 @@ class Linear:
                 self.tiled = K.TiledWeight(self.weight, halves)
 
     GEMV, FEW_ROWS = "gemv", "few_rows"
+    # The matrix-vector product adds an attention output's partial results up itself only for up to
+    # 2,048 inputs: beyond, the registers that hold them cost it more than the merge launch saved
+    # (decode steps of one / two requests at 700 keys, 8 layers of the 3B sizes, 3,072 inputs of heads
+    # of 128: 0.536 / 0.578 -> 0.537 / 0.609 ms; 8B sizes, 4,096 inputs: 0.862 / 0.906 -> 0.854 / 0.964;
+    # 1B sizes, 2,048 inputs of heads of 64, 16 layers: 0.688 / 0.769 -> 0.660 / 0.741).
+    MERGES_UP_TO_INPUTS = 2048
 
     def fused_kernel(self, rows: int, dtype, rotated: bool = False) -> Optional[str]:
         """The hand-written product that takes ``rows`` rows of ``dtype`` with a norm on its input
@@ -63,6 +69,14 @@ class Linear:
             return None
         return self.fused_kernel(rows, dtype)
 
+    def takes_attention_partials(self, rows: int, dtype, tail: Optional[BranchTail], head_dim: int) -> int:
+        """How many partial results a row (``ops.kernels.AttentionPartials``) :meth:`into_residual`
+        can add up itself for ``rows`` rows of heads of ``head_dim``; 0: none, it wants the output."""
+        if self.residual_kernel(rows, dtype, tail) != self.GEMV or self.in_features > self.MERGES_UP_TO_INPUTS:
+            return 0
+        most = K.gemv_merge_max_parts()
+        return most if K.gemv_merged_supported(rows, self.out_features, self.in_features, head_dim, most) else 0
+
     def into_residual(self, x, tail: BranchTail):
         """hidden += x @ W^T in place and the sum prepared for ``tail.norm`` (NormedRows); or, at
         17 to 64 rows of a matrix that the few-rows kernel does not take whole, the product as
@@ -79,13 +93,18 @@ class Linear:
         if isinstance(x, NormedRows):
             norm = dict(sumsq=x.sumsq, norm_width=x.width, eps=x.eps)
             x = x.scaled
+        if isinstance(x, K.AttentionPartials) and kernel != self.GEMV:
+            raise K.KernelError("Linear.into_residual: partial results were left for a product that cannot add them up")
         if kernel == self.GEMV:
             if isinstance(x, K.TiledRows):
                 x = x.to_rows()
             sumsq = torch.empty((rows, K.gemv_sumsq_parts(self.out_features, self.in_features)),
                                 dtype=torch.float32, device=x.device)
-            K.gemv(x, self.weight, None, hidden=tail.hidden, next_weight=next_w, scaled_out=scaled,
-                   sumsq_out=sumsq, **norm)
+            if isinstance(x, K.AttentionPartials):
+                K.gemv_merged(x, self.weight, tail.hidden, next_w, scaled, sumsq)
+            else:
+                K.gemv(x, self.weight, None, hidden=tail.hidden, next_weight=next_w, scaled_out=scaled,
+                       sumsq_out=sumsq, **norm)
         else:
             sumsq = torch.empty((rows, K.gemm_skinny_sumsq_parts(self.out_features)), dtype=torch.float32,
                                 device=x.device)

@@ -100,6 +100,30 @@ def test_many_requests_decoding_together(name, batch, model_dirs, gpu, monkeypat
     assert llm.engine.cache.free_seats == batch
 
 
+@pytest.mark.parametrize("lengths", [[520], [700, 530], [1030]])
+def test_one_or_two_requests_decode_without_a_merge_launch(lengths, sharp_model_dirs, gpu, monkeypatch):
+    """Model E (512 wide, heads of 64): from 512 keys on the attention kernel leaves the key ranges
+    of one or two decoded tokens as partial results - four ranges a workgroup - and the output
+    projection's matrix-vector kernel adds them up where it would have read the tokens.  On the
+    weights that spread attention over far keys, every pick against the plain model; eagerly and
+    from the decode graph."""
+    from kv_cache_optimization_for_llm_amd.ops import kernels as K
+    calls = []
+    inside = K.gemv_merged
+    monkeypatch.setattr(K, "gemv_merged", lambda x, *a, **k: (calls.append(x.parts), inside(x, *a, **k))[1])
+    cfg, W = plain.load_model_dir(sharp_model_dirs["E"])
+    prompts = prompts_for("E", lengths, seed=11)
+    llm = LLM(sharp_model_dirs["E"], EngineOptions(dtype="bfloat16", page_size=16, max_seqs=2, max_seq_len=1100),
+              ServeOptions(max_batch_tokens=2048))
+    got = llm.generate(prompts, max_new_tokens=12, ignore_eos=True)
+    for p, g in zip(prompts, got):
+        assert len(g) == 12
+        check_choices(cfg, W, p, g, "bfloat16")
+    assert calls and all(2 <= parts <= K.gemv_merge_max_parts() for parts in calls)
+    assert llm.engine.graphs.replays > 0
+    llm.engine.cache.check()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_temperature_sampling_and_penalty_follow_the_plain_sampler(dtype, model_dirs, gpu):
     cfg, W = plain.load_model_dir(model_dirs["B"])

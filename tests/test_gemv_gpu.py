@@ -200,3 +200,51 @@ def test_refusals(gpu):
     with pytest.raises(K.KernelError):
         K.gemv_qkv_rope(x[:1], rnd(4 * 6, 512).to(gpu), torch.empty((1, 12), dtype=torch.bfloat16, device=gpu), 2, 1, 6,
                         torch.zeros(1, dtype=torch.int32, device=gpu), None, None, None, None, None, 0)
+
+
+@pytest.mark.parametrize("m", [1, 2])
+@pytest.mark.parametrize("n, k, d, parts", [(2048, 2048, 64, 3), (515, 512, 64, 2), (96, 1536, 96, 4), (389, 3072, 128, 4),
+                                            (130, 4096, 128, 3), (77, 2560, 16, 2), (64, 3584, 8, 4), (40, 1024, 32, 3)])
+def test_product_over_an_attention_output_still_in_partial_results(m, n, k, d, parts, gpu):
+    """The residual-epilogue product whose input is what an attention kernel left per key range
+    (running maximum in the base-2 domain, sum of exponentials, unnormalised output) against the
+    ranges added up here and the ordinary product over that sum; one range of one head without a
+    key (maximum -inf, everything else zero), which must weigh nothing."""
+    heads = k // d
+    g = torch.Generator().manual_seed(n + k + parts + m)
+    part_o = torch.randn(m * heads, parts, d, generator=g)
+    ml = torch.stack([torch.randn(m * heads, parts, generator=g) * 3, torch.rand(m * heads, parts, generator=g) * 5 + 0.5], -1)
+    part_o[1, parts - 1] = 0.0
+    ml[1, parts - 1, 0], ml[1, parts - 1, 1] = float("-inf"), 0.0
+    wgt = torch.exp2(ml[..., 0] - ml[..., 0].max(-1, keepdim=True).values)           # [rows, parts]
+    merged = (part_o * wgt[..., None]).sum(1) / (ml[..., 1] * wgt).sum(-1, keepdim=True)
+    x = merged.reshape(m, k).to(torch.bfloat16)
+    w = rnd(n, k, scale=0.05, seed=1)
+    h0 = rnd(m, n, seed=2)
+    w_next = (1 + 0.1 * torch.randn(n, generator=torch.Generator().manual_seed(3))).to(torch.bfloat16)
+    p_out = K.gemv_sumsq_parts(n, k)
+    assert K.gemv_merged_supported(m, n, k, d, parts)
+    hidden_a, hidden_b = h0.clone().to(gpu), h0.clone().to(gpu)
+    scaled_a, scaled_b = (torch.empty((m, n), dtype=torch.bfloat16, device=gpu) for _ in range(2))
+    ss_a, ss_b = (torch.empty((m, p_out), device=gpu) for _ in range(2))
+    K.gemv_merged(K.AttentionPartials(part_o.to(gpu), ml.to(gpu), m, heads), w.to(gpu), hidden_a, w_next.to(gpu), scaled_a, ss_a)
+    K.gemv(x.to(gpu), w.to(gpu), None, hidden=hidden_b, next_weight=w_next.to(gpu), scaled_out=scaled_b, sumsq_out=ss_b)
+    want = (h0.float() + (x.double() @ w.double().t()).float())
+    scale = want.abs().max()
+    assert (hidden_a.cpu().float() - want).abs().max() <= 8e-3 * scale
+    # against the ordinary product: the same but for inputs that the two ways of adding up round differently
+    assert (hidden_a.float() - hidden_b.float()).abs().max() <= 8e-3 * scale
+    hf = hidden_a.cpu().float()
+    assert torch.allclose(ss_a.cpu().sum(-1), (hf * hf).sum(-1), rtol=1e-5)
+    assert torch.equal(scaled_a.cpu(), (hf * w_next.float()).to(torch.bfloat16))
+
+
+def test_what_the_merging_product_takes():
+    assert K.gemv_merge_max_parts() >= 4
+    assert K.gemv_merged_supported(1, 2048, 2048, 64, 2) and K.gemv_merged_supported(2, 4096, 4096, 128, 4)
+    assert not K.gemv_merged_supported(1, 2048, 2048, 64, 1)         # nothing to add up
+    assert not K.gemv_merged_supported(1, 2048, 2048, 64, K.gemv_merge_max_parts() + 1)
+    assert not K.gemv_merged_supported(1, 2048, 5120, 64, 2)         # K beyond 4,096
+    assert not K.gemv_merged_supported(1, 2048, 2048, 12, 2)         # heads of no multiple of 8
+    assert not K.gemv_merged_supported(1, 2048, 2048, 80, 2)         # heads that do not divide K
+    assert not K.gemv_merged_supported(3, 2048, 2048, 64, 2)

@@ -3,7 +3,7 @@ cache pool is made from leftover device memory."""
 import pytest
 
 from kv_cache_optimization_for_llm_amd.engine.engine import EngineError, pool_pages_from_memory
-from kv_cache_optimization_for_llm_amd.ops.attention import (choose_decode_ranges, choose_lds_splits, choose_splits,
+from kv_cache_optimization_for_llm_amd.ops.attention import (choose_decode_ranges, choose_left_ranges, choose_lds_splits, choose_splits,
                                                              use_lds_kernel)
 
 KERNEL_MAX_SPLITS = 256         # what the kernels and their merge take (kva_attention_max_splits)
@@ -153,3 +153,21 @@ def test_which_products_of_one_or_two_tokens_take_the_matrix_vector_kernel():
     # long rows cost a second token more than a first one
     assert use_gemv(1, 4096, 5120) and not use_gemv(2, 4096, 5120)
     assert use_gemv(1, 2048, 8192) and use_gemv(2, 2048, 8192)
+
+
+@pytest.mark.parametrize("context", [512, 513, 600, 768, 769, 1000, 1024, 1500, 2048])
+@pytest.mark.parametrize("items", [1, 2])
+def test_key_ranges_left_for_an_output_projection_that_adds_them_up(items, context, ):
+    ranges, per, waves = choose_left_ranges(items, context, 64, 4)
+    assert waves == 4 and ranges % 4 == 0 and 2 <= ranges // 4 <= 4          # what the consumer takes
+    assert per % 32 == 0 and per >= 64 and ranges * per >= context           # every key in a range
+    assert (ranges - 4) * per < context                                     # no workgroup without a key
+
+
+def test_where_no_key_ranges_are_left_to_the_output_projection():
+    assert choose_left_ranges(3, 768, 64, 4) is None            # the matrix-vector kernel takes two tokens
+    assert choose_left_ranges(1, 300, 64, 4) is None            # too short for two workgroups of four ranges
+    assert choose_left_ranges(1, 4096, 64, 4) is None           # too long for 16 ranges
+    assert choose_left_ranges(1, 768, 128, 4) is None           # measured at head sizes up to 64
+    assert choose_left_ranges(1, 768, 64, 1) is None and choose_left_ranges(1, 768, 64, 0) is None
+    assert choose_left_ranges(1, 768, 64, 2) == (8, 96, 4)
