@@ -47,7 +47,7 @@ class Runner:
             engine.cache, max_batch_tokens=min(options.max_batch_tokens, engine.max_batch_tokens),
             chunk_size=options.chunk_size,
             eos_token_ids=engine.spec.eos_token_ids, ignore_eos=options.ignore_eos,
-            reserve_policy=options.reserve_policy)
+            reserve_policy=options.reserve_policy, portion_multiple=engine.model.portion_multiple)
         self.sampler = Sampler(engine.vocab_size, engine.cache.max_seqs, engine.device,
                                seed=options.sampling_seed, repetition_penalty=options.repetition_penalty)
         self.scheduler.on_admit = self._on_admit

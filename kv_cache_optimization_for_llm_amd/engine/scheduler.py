@@ -139,14 +139,23 @@ def reservation_tokens(policy: str, prompt_len: int, max_new_tokens: int, max_se
 class Scheduler:
     def __init__(self, cache: CacheManager, *, max_batch_tokens: int = 3072, chunk_size: Optional[int] = None,
                  eos_token_ids: Sequence[int] = (), ignore_eos: bool = False,
-                 reserve_policy: str = "max"):
+                 reserve_policy: str = "max", portion_multiple: int = 1):
         if max_batch_tokens < 1:
             raise ValueError("max_batch_tokens must be at least 1")
+        if portion_multiple < 1 or portion_multiple > max_batch_tokens:
+            raise ValueError(f"portions that end on multiples of {portion_multiple} positions do not fit "
+                             f"steps of {max_batch_tokens} tokens")
         if reserve_policy not in RESERVE_POLICIES:
             raise ValueError(f"reservation policy {reserve_policy!r} is not one of {RESERVE_POLICIES}")
         self.cache = cache
         self.max_batch_tokens = int(max_batch_tokens)
         self.chunk_size = int(chunk_size) if chunk_size else self.max_batch_tokens
+        # every portion but a prompt's last ends at a multiple of this many positions (what the
+        # model's mixers ask for: parts.base.Mixer.portion_multiple)
+        self.portion_multiple = int(portion_multiple)
+        if self.chunk_size < self.portion_multiple:
+            raise ValueError(f"chunk_size {self.chunk_size} is smaller than the {self.portion_multiple} positions "
+                             f"a portion must be a multiple of")
         self.eos = frozenset(int(e) for e in eos_token_ids)
         self.ignore_eos = bool(ignore_eos)
         self.reserve_policy = reserve_policy
@@ -318,6 +327,8 @@ class Scheduler:
             nonlocal budget
             want = min(len(seq.prompt) - seq.computed, self.chunk_size, budget)
             n = fit_tokens(seq, want)
+            if self.portion_multiple > 1 and seq.computed + n < len(seq.prompt):
+                n = (seq.computed + n) // self.portion_multiple * self.portion_multiple - seq.computed
             if n <= 0:
                 return
             for i, x in enumerate(cache.pages_needed(seq.seat, seq.computed + n)):

@@ -80,6 +80,16 @@ class Model:
         self.head: Optional[Linear] = None
 
     # ---- what the cache manager has to provide
+    @property
+    def portion_multiple(self) -> int:
+        """Positions at whose multiples a prompt may be cut into portions: the least common
+        multiple of what the layers' mixers ask for."""
+        import math
+        m = 1
+        for block in self.blocks:
+            m = math.lcm(m, max(1, int(getattr(block.mixer, "portion_multiple", 1))))
+        return m
+
     def cache_requirements(self):
         """(groups, states): groups = [(KVCacheSpec, [cache slot ids])] for slots that need paged
         K/V, states = {cache slot id: StateSpec}."""

@@ -243,6 +243,10 @@ class PositionEncoding(Part):
 
 class Mixer(Part):
     fuses_tail = False      # True: forward(x, ctx, tail=None) accepts NormedRows and a BranchTail
+    # A mixer that can only take a prompt in portions that end on multiples of so many positions
+    # (a state it carries is updated in blocks, say) says so here; the scheduler then cuts every
+    # portion but a prompt's last at such a position.  Attention takes any cut: 1.
+    portion_multiple = 1
 
     def kv_cache_spec(self) -> Optional[KVCacheSpec]:
         return None

@@ -517,3 +517,36 @@ def test_admission_asks_each_group_what_a_prompt_needs():
         s.add(Request(i, list(range(8, 108)), 3))
     out, reasons, _, plans = run(s)
     assert reasons == {(i, 0): "length" for i in range(3)} and all(len(v) == 3 for v in out.values())
+
+
+@pytest.mark.parametrize("multiple, chunk, budget", [(8, 20, 50), (5, 5, 17), (16, 64, 40), (3, 100, 29)])
+def test_portions_end_where_the_mixers_can_be_cut(multiple, chunk, budget):
+    """A model whose mixers take a prompt only in portions that end on multiples of so many
+    positions: every portion but a prompt's last ends there, whatever the token budget and the
+    other requests leave, and every request still emits all its tokens."""
+    s = Scheduler(cache(pages=128), max_batch_tokens=budget, chunk_size=chunk, ignore_eos=True,
+                  portion_multiple=multiple)
+    lengths = [1, multiple - 1, multiple, multiple + 1, 61, 100, 37]
+    for i, n in enumerate(lengths):
+        s.add(Request(i, [8 + (j % 50) for j in range(n)], 6))
+    cuts = []
+
+    def watch(plan):
+        assert plan.num_tokens <= budget
+        for e in plan.entries:
+            if len(e.tokens) > 1 or e.start < len(e.seq.prompt):
+                end = e.start + len(e.tokens)
+                assert e.start % multiple == 0 and (end % multiple == 0 or end == len(e.seq.prompt)), (e.start, end)
+                cuts.append((e.seq.request.id, e.start, end))
+    out, reasons, _, _ = run(s, on_plan=watch)
+    assert all(len(out[(i, 0)]) == 6 and reasons[(i, 0)] == "length" for i in range(len(lengths)))
+    assert any(end % multiple == 0 and end < lengths[i] for i, _, end in cuts), "no prompt was cut at all"
+
+
+def test_a_portion_multiple_that_cannot_be_kept_is_refused():
+    with pytest.raises(ValueError):
+        Scheduler(cache(), max_batch_tokens=16, portion_multiple=32)
+    with pytest.raises(ValueError):
+        Scheduler(cache(), max_batch_tokens=64, chunk_size=8, portion_multiple=16)
+    with pytest.raises(ValueError):
+        Scheduler(cache(), max_batch_tokens=64, portion_multiple=0)

@@ -67,6 +67,21 @@ class ToyDecayMixer(Mixer):
         return (y @ self.w_out.t()).to(x.dtype)
 
 
+class ToyBlockwiseDecayMixer(ToyDecayMixer):
+    """The same recurrence by a mixer that can only be cut where a block of four positions ends (it
+    would update its state block by block): it says so, and records where it was cut."""
+    portion_multiple = 4
+    cuts = []
+
+    def forward(self, x, ctx: MixerContext):
+        b = ctx.batch
+        for e in range(b.num_entries):
+            n = int(b.h_entry_q_start[e + 1]) - int(b.h_entry_q_start[e])
+            if n > 1:
+                type(self).cuts.append((int(b.h_entry_start_pos[e]), n))
+        return super().forward(x, ctx)
+
+
 class ToyLatentMixer(Mixer):
     """Attention over one latent vector per token: c_t = W_c x_t, g_t = 1 + tanh(w_g . x_t) (kept in
     32-bit), q_t = W_q x_t; y_t = W_o sum_{s<=t} softmax_s(q_t . c_s / sqrt(w)) g_s c_s.  What it
@@ -177,8 +192,8 @@ def toy_config(kind, dtype="float32"):
 
 def toy_layer(c, i, mixer):
     p = f"blocks.{i}."
-    if mixer == "toy_decay":
-        mx = PartSpec("toy_decay", dict(prefix=p + "mix.", hidden_size=c["hidden_size"], state_size=c["state_size"]))
+    if mixer in ("toy_decay", "toy_blockwise_decay"):
+        mx = PartSpec(mixer, dict(prefix=p + "mix.", hidden_size=c["hidden_size"], state_size=c["state_size"]))
     elif mixer == "toy_latent":
         mx = PartSpec("toy_latent", dict(prefix=p + "lat.", hidden_size=c["hidden_size"], latent_size=c["latent_size"]))
     else:
@@ -265,6 +280,9 @@ def registered():
     register_architecture("ToySandwichLM", dict, sandwich_spec, replace=True)
     MIXERS.register("toy_decay", ToyDecayMixer, replace=True)
     MIXERS.register("toy_latent", ToyLatentMixer, replace=True)
+    MIXERS.register("toy_blockwise_decay", ToyBlockwiseDecayMixer, replace=True)
+    register_architecture("ToyBlockwiseLM", dict, toy_spec(
+        "ToyBlockwiseLM", ["toy_blockwise_decay", "gqa_attention"], [LayerCall(0, 0), LayerCall(1, 1)]), replace=True)
     register_architecture("ToyLatentLM", dict, toy_spec(
         "ToyLatentLM", ["toy_latent", "gqa_attention", "toy_latent"],
         [LayerCall(0, 0), LayerCall(1, 1), LayerCall(2, 2)]), replace=True)
@@ -281,6 +299,7 @@ def registered():
     yield
     MIXERS.unregister("toy_decay")
     MIXERS.unregister("toy_latent")
+    MIXERS.unregister("toy_blockwise_decay")
     BLOCKS.unregister("toy_sandwich")
     POSITION_ENCODINGS.unregister("toy_neighbour_rotary")
     FEED_FORWARDS.unregister("toy_routed")
@@ -496,6 +515,42 @@ def test_a_model_that_keeps_no_keys_at_all(tmp_path, gpu):
         assert len(out[rid]) == 6
     eng.cache.check()
     assert eng.cache.free_seats == 2
+
+
+def test_the_scheduler_cuts_prompts_where_a_mixer_says_it_can_be_cut(tmp_path, gpu):
+    """A model with a mixer that takes portions only up to multiples of four positions, beside an
+    attention layer that takes any cut: the serving loop asks the model and cuts prompts there
+    (token budget 23, portions of at most 10 tokens: 8 at a time), a prompt's last portion ends
+    where the prompt ends, and what is generated is what the same weights generate under the mixer
+    that takes any cut."""
+    from kv_cache_optimization_for_llm_amd.engine.runner import Runner, ServeOptions
+    c = toy_config("ToyBlockwiseLM", "float32")
+    d = write_random_model(str(tmp_path / "toy"), c, seed=23, gain=1.0)
+    c2 = dict(c, architectures=["ToyStateLM"])
+    d2 = write_random_model(str(tmp_path / "toy2"), c2, seed=23, gain=1.0)
+    rng = np.random.default_rng(9)
+    prompts = [[int(t) for t in rng.integers(0, 97, n)] for n in (3, 30, 17, 41)]
+    results = []
+    for folder in (d, d2):
+        eng = Engine(folder, EngineOptions(dtype="float32", max_seqs=3, max_seq_len=96, cache_tokens=512))
+        runner = Runner(eng, ServeOptions(ignore_eos=True, max_batch_tokens=23, chunk_size=10))
+        if folder == d:
+            assert eng.model.portion_multiple == 4 and runner.scheduler.portion_multiple == 4
+            ToyBlockwiseDecayMixer.cuts.clear()
+        else:
+            assert eng.model.portion_multiple == 1
+        ids = [runner.submit(p, 5) for p in prompts]
+        out = {i: [] for i in ids}
+        for ev in runner.run_until_idle():
+            if ev.kind == "token":
+                out[ev.request_id].append(ev.token)
+        results.append([out[i] for i in ids])
+        eng.cache.check()
+    assert results[0] == results[1] and all(len(g) == 5 for g in results[0])
+    cuts = ToyBlockwiseDecayMixer.cuts
+    lengths = {len(p) for p in prompts}
+    assert cuts and all(start % 4 == 0 and ((start + n) % 4 == 0 or start + n in lengths) for start, n in cuts), cuts
+    assert any((start + n) % 4 == 0 and n == 8 for start, n in cuts)
 
 
 @pytest.mark.parametrize("dtype, tol", [("float32", 3e-5), ("bfloat16", 2e-2)])
