@@ -82,8 +82,12 @@ constexpr int GV_WAVES = 4;          // wavefronts per workgroup
 // load, wait, add takes over, and that wait is for every load in flight, the rows of W included:
 // 0.8 us of the Q/K/V product's 5.5 when four were asked for here.
 constexpr int GV_NORM_LOADS = 8;
-// Partial results of key ranges per row that the merged form adds up (a lane holds 10 floats of each).
-constexpr int GV_MERGE_MAX_PARTS = 4;
+// Partial results of key ranges per row that the merged form adds up (a lane holds 10 floats of
+// each): up to 4 in one instance, up to 8 in another that exists for one token only - the registers
+// of eight cost the steps that need four 1.5-2 % (one / two requests at 768 keys 0.660 / 0.741 ->
+// 0.670 / 0.757 ms), and one request at 2,049-4,096 keys gains 3 % from them (0.720 -> 0.698 at 3,000).
+constexpr int GV_MERGE_PARTS = 4;
+constexpr int GV_MERGE_MAX_PARTS = 8;
 
 // KV: 16-byte vectors per lane and row (K = 512 KV); M: tokens; RB: rows a wavefront has in flight.
 // Row r of unit u: plain / residual: u RB + r.  SwiGLU (RB even): pair t = r / 2 of the unit is
@@ -97,12 +101,14 @@ constexpr int GV_MERGE_MAX_PARTS = 4;
 //
 // MERGED (residual epilogue, K up to 4,096): the token(s) are not read but made - the output
 // projection of an attention layer takes the partial results that the attention kernel left per
-// key range (at most GV_MERGE_MAX_PARTS a row) and adds them up itself, as the merge kernel would
+// key range (at most PARTS a row) and adds them up itself, as the merge kernel would
 // (weights 2^(m_s - max m), the sum divided by the weighted sum of the l_s, rounded to bf16), so
 // that one or two decoded tokens need no merge launch.  The wavefronts of a workgroup share the
 // work: wavefront w makes the columns of vectors c = w, w + GV_WAVES, ... and leaves them in LDS.
-template <int KV, int M, int RB, int EPI, bool MERGED = false>
+template <int KV, int M, int RB, int EPI, int PARTS = 0>
 __global__ void __launch_bounds__(64 * GV_WAVES) gemv_kernel(const GemvArgs a) {
+    constexpr bool MERGED = PARTS > 0;
+    constexpr int MAXP = MERGED ? PARTS : 1;       // partial results a row that a lane has room for
     const int lane = threadIdx.x & 63, wave_in_block = threadIdx.x >> 6;
     const int K = a.K;
     constexpr int PAIRS = RB / 2;
@@ -146,8 +152,8 @@ __global__ void __launch_bounds__(64 * GV_WAVES) gemv_kernel(const GemvArgs a) {
     // the token(s), kept packed: lane l owns columns (64 c + l) * 8 .. + 8
     uint4 xp[M][KV];
     constexpr int MINE = MERGED ? (KV + GV_WAVES - 1) / GV_WAVES : 1;     // vectors this wavefront makes per token
-    float2 pml[MINE][M][GV_MERGE_MAX_PARTS];
-    float4 pov[MINE][M][GV_MERGE_MAX_PARTS][2];
+    float2 pml[MINE][M][MAXP];
+    float4 pov[MINE][M][MAXP][2];
     if constexpr (MERGED) {
         const int heads = K / a.part_head_dim;
 #pragma unroll
@@ -159,7 +165,7 @@ __global__ void __launch_bounds__(64 * GV_WAVES) gemv_kernel(const GemvArgs a) {
             for (int m = 0; m < M; ++m) {
                 const size_t row = (size_t)m * heads + head;
 #pragma unroll
-                for (int sp = 0; sp < GV_MERGE_MAX_PARTS; ++sp) {
+                for (int sp = 0; sp < MAXP; ++sp) {
                     const int ss = min(sp, a.parts - 1);                      // masked where they are added
                     pml[i][m][sp] = reinterpret_cast<const float2 *>(a.part_ml)[row * a.parts + ss];
                     const float4 *po = reinterpret_cast<const float4 *>(a.part_o + (row * a.parts + ss) * a.part_head_dim + j0);
@@ -214,11 +220,11 @@ __global__ void __launch_bounds__(64 * GV_WAVES) gemv_kernel(const GemvArgs a) {
             for (int m = 0; m < M; ++m) {
                 float mx = -INFINITY;
 #pragma unroll
-                for (int sp = 0; sp < GV_MERGE_MAX_PARTS; ++sp)
+                for (int sp = 0; sp < MAXP; ++sp)
                     if (sp < a.parts) mx = fmaxf(mx, pml[i][m][sp].x);
                 float denom = 0.f, acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int sp = 0; sp < GV_MERGE_MAX_PARTS; ++sp) {
+                for (int sp = 0; sp < MAXP; ++sp) {
                     if (sp < a.parts) {
                         const float wgt = pml[i][m][sp].x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(pml[i][m][sp].x - mx);
                         denom += pml[i][m][sp].y * wgt;
@@ -423,8 +429,11 @@ int launch(const GemvArgs &a, hipStream_t stream) {
     if constexpr (EPI == GV_RESID) {
         if (a.part_o != nullptr) {
 #define GVP(KVV, RBB)                                                                                          \
-    if (a.M == 1) hipLaunchKernelGGL((gemv_kernel<KVV, 1, RBB, GV_RESID, true>), grid, block, 0, stream, a);  \
-    else hipLaunchKernelGGL((gemv_kernel<KVV, 2, RBB, GV_RESID, true>), grid, block, 0, stream, a)
+    if (a.M == 1 && a.parts > GV_MERGE_PARTS)                                                                  \
+        hipLaunchKernelGGL((gemv_kernel<KVV, 1, RBB, GV_RESID, GV_MERGE_MAX_PARTS>), grid, block, 0, stream, a); \
+    else if (a.M == 1)                                                                                         \
+        hipLaunchKernelGGL((gemv_kernel<KVV, 1, RBB, GV_RESID, GV_MERGE_PARTS>), grid, block, 0, stream, a);   \
+    else hipLaunchKernelGGL((gemv_kernel<KVV, 2, RBB, GV_RESID, GV_MERGE_PARTS>), grid, block, 0, stream, a)
             switch (kv) {
             case 1: GVP(1, 8); break;
             case 2: GVP(2, 8); break;
@@ -540,12 +549,12 @@ extern "C" int kva_gemv(void *Y, const void *X, const void *W, int M, int N, int
 }
 
 // Whether kva_gemv_merged takes these sizes: one or two tokens, K up to 4,096 with an instance,
-// heads of a multiple of 8 features that divide K, 2 to GV_MERGE_MAX_PARTS partial results a row.
+// heads of a multiple of 8 features that divide K, 2 to kva_gemv_merge_max_parts(M) partial results a row.
+extern "C" int kva_gemv_merge_max_parts(int M) { return M == 1 ? GV_MERGE_MAX_PARTS : GV_MERGE_PARTS; }
 extern "C" int kva_gemv_merged_supported(int M, int N, int K, int head_dim, int parts) {
     return (kva_gemv_supported(M, N, K) && K <= 4096 && head_dim >= 8 && head_dim % 8 == 0 && K % head_dim == 0 &&
-            parts >= 2 && parts <= GV_MERGE_MAX_PARTS) ? 1 : 0;
+            parts >= 2 && parts <= kva_gemv_merge_max_parts(M)) ? 1 : 0;
 }
-extern "C" int kva_gemv_merge_max_parts() { return GV_MERGE_MAX_PARTS; }
 
 // kva_gemv's mode 3 (hidden[M, N] += X W^T, the next norm prepared) with X = the attention output
 // of M decoded tokens given as what the attention kernel left per key range: part_o

@@ -212,17 +212,24 @@ def choose_decode_ranges(num_items: int, num_kv_heads: int, max_context: int, he
 # 0.681, two requests at 768 / 1,900 keys 0.769 / 0.783 -> 0.741 / 0.766.  Up to 2,048 keys (contexts are
 # rounded up to a power of two when a step is captured): with at most 4 partial results a row 4,096
 # keys are 16 ranges of 256, and one request at 3,000 / 8,000 keys went 0.719 / 0.741 -> 0.722 / 0.805.
+# With 8 partial results a row, which the consumer has room for with one token only, 2,049-4,096 keys are
+# 32 ranges of 128: one request at 3,000 keys 0.720 -> 0.698 (two: 0.797 -> 0.798; 8,000 keys: 0.742 -> 0.746).
 # Head sizes up to 64, where it was measured (at 128, with wider output projections: parts/linear.py).
 _LEFT_MAX_ITEMS = 2
 _LEFT_MIN_KEYS = 64
 _LEFT_MAX_CONTEXT = 2048
+_LEFT_PARTS_SHORT = 4             # up to 2,048 keys: at most 16 ranges
+_LEFT_MAX_CONTEXT_ONE = 4096      # one token, a consumer that takes 8 partial results: 32 ranges up to here
 
 
 def choose_left_ranges(num_items: int, max_context: int, head_dim: int, max_parts: int):
     """(key ranges, keys per range, 4) for decoded tokens whose consumer takes up to ``max_parts``
     partial results a row, or None where the ordinary choice stands."""
-    if num_items > _LEFT_MAX_ITEMS or head_dim > _SHARED_TUNED_HEAD_DIM or max_parts < 2 \
-            or max_context > _LEFT_MAX_CONTEXT:
+    if num_items > _LEFT_MAX_ITEMS or head_dim > _SHARED_TUNED_HEAD_DIM or max_parts < 2:
+        return None
+    if max_context <= _LEFT_MAX_CONTEXT:
+        max_parts = min(max_parts, _LEFT_PARTS_SHORT)
+    elif num_items > 1 or max_context > _LEFT_MAX_CONTEXT_ONE or max_parts <= _LEFT_PARTS_SHORT:
         return None
     # a multiple of four ranges whatever the context: the last ones may hold few keys or none (a
     # range without a key weighs nothing when the results are added up)

@@ -944,8 +944,9 @@ def gemv_merged_supported(m: int, n: int, k: int, head_dim: int, parts: int) -> 
     return bool(hip_lib().kva_gemv_merged_supported(int(m), int(n), int(k), int(head_dim), int(parts)))
 
 
-def gemv_merge_max_parts() -> int:
-    return int(hip_lib().kva_gemv_merge_max_parts())
+def gemv_merge_max_parts(m: int = 2) -> int:
+    """Partial results a row that :func:`gemv_merged` adds up for ``m`` tokens."""
+    return int(hip_lib().kva_gemv_merge_max_parts(int(m)))
 
 
 def gemv_merged(x: AttentionPartials, w: torch.Tensor, hidden: torch.Tensor, next_weight: Optional[torch.Tensor],

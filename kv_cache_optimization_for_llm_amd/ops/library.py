@@ -64,7 +64,7 @@ _HIP_SIGNATURES = {
     "kva_gemv": [P, P, P, I, I, I, I, I, I, P, I, I, F, P, P, I, P, P, P],
     "kva_gemv_supported": [I, I, I],
     "kva_gemv_merged_supported": [I, I, I, I, I],
-    "kva_gemv_merge_max_parts": [],
+    "kva_gemv_merge_max_parts": [I],
     "kva_gemv_merged": [P, P, I, I, P, I, I, I, P, P, I, P, P, P],
     "kva_gemv_sumsq_parts": [I, I],
     "kva_gemv_qkv_rope_supported": [I, I, I],

@@ -74,7 +74,7 @@ class Linear:
         can add up itself for ``rows`` rows of heads of ``head_dim``; 0: none, it wants the output."""
         if self.residual_kernel(rows, dtype, tail) != self.GEMV or self.in_features > self.MERGES_UP_TO_INPUTS:
             return 0
-        most = K.gemv_merge_max_parts()
+        most = K.gemv_merge_max_parts(rows)
         return most if K.gemv_merged_supported(rows, self.out_features, self.in_features, head_dim, most) else 0
 
     def into_residual(self, x, tail: BranchTail):

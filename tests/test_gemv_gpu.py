@@ -204,12 +204,16 @@ def test_refusals(gpu):
 
 @pytest.mark.parametrize("m", [1, 2])
 @pytest.mark.parametrize("n, k, d, parts", [(2048, 2048, 64, 3), (515, 512, 64, 2), (96, 1536, 96, 4), (389, 3072, 128, 4),
-                                            (130, 4096, 128, 3), (77, 2560, 16, 2), (64, 3584, 8, 4), (40, 1024, 32, 3)])
+                                            (130, 4096, 128, 3), (77, 2560, 16, 2), (64, 3584, 8, 4), (40, 1024, 32, 3),
+                                            (2048, 2048, 64, 8), (61, 512, 32, 5), (200, 4096, 64, 7)])
 def test_product_over_an_attention_output_still_in_partial_results(m, n, k, d, parts, gpu):
     """The residual-epilogue product whose input is what an attention kernel left per key range
     (running maximum in the base-2 domain, sum of exponentials, unnormalised output) against the
     ranges added up here and the ordinary product over that sum; one range of one head without a
     key (maximum -inf, everything else zero), which must weigh nothing."""
+    if parts > K.gemv_merge_max_parts(m):
+        assert m == 2 and not K.gemv_merged_supported(m, n, k, d, parts)       # more than four only for one token
+        return
     heads = k // d
     g = torch.Generator().manual_seed(n + k + parts + m)
     part_o = torch.randn(m * heads, parts, d, generator=g)
@@ -240,10 +244,11 @@ def test_product_over_an_attention_output_still_in_partial_results(m, n, k, d, p
 
 
 def test_what_the_merging_product_takes():
-    assert K.gemv_merge_max_parts() >= 4
+    assert K.gemv_merge_max_parts(1) >= K.gemv_merge_max_parts(2) >= 4
     assert K.gemv_merged_supported(1, 2048, 2048, 64, 2) and K.gemv_merged_supported(2, 4096, 4096, 128, 4)
     assert not K.gemv_merged_supported(1, 2048, 2048, 64, 1)         # nothing to add up
-    assert not K.gemv_merged_supported(1, 2048, 2048, 64, K.gemv_merge_max_parts() + 1)
+    assert not K.gemv_merged_supported(1, 2048, 2048, 64, K.gemv_merge_max_parts(1) + 1)
+    assert not K.gemv_merged_supported(2, 2048, 2048, 64, K.gemv_merge_max_parts(2) + 1)
     assert not K.gemv_merged_supported(1, 2048, 5120, 64, 2)         # K beyond 4,096
     assert not K.gemv_merged_supported(1, 2048, 2048, 12, 2)         # heads of no multiple of 8
     assert not K.gemv_merged_supported(1, 2048, 2048, 80, 2)         # heads that do not divide K
