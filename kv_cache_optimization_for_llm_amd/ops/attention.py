@@ -98,6 +98,15 @@ def _cut_keys(want: int, max_context: int, max_splits: int) -> tuple:
     return (splits, per) if splits > 1 else (1, 0)
 
 
+def _cut_keys_by_fours(want: int, max_context: int):
+    """``max_context`` keys in at most ``want`` (a multiple of four) ranges of a multiple of 32
+    keys, their number a multiple of four: the last three at most hold no key, never a whole
+    workgroup of four.  None below 8 ranges."""
+    per = ((max_context + want - 1) // want + 31) // 32 * 32
+    n = ((max_context + per - 1) // per + 3) // 4 * 4
+    return (n, per) if n >= 8 else None
+
+
 def choose_splits(num_items: int, num_kv_heads: int, max_context: int, max_splits: int = None,
                   decoding: bool = False, merged_by_fours: bool = False) -> tuple:
     """(splits, keys_per_split) for the matrix-core kernel; never more splits than the kernels
@@ -134,6 +143,8 @@ def choose_splits(num_items: int, num_kv_heads: int, max_context: int, max_split
 # read: 8 requests at 8,192 / 32,768 keys (16 ranges of 512 / 2,048 keys) 1.156 / 2.167 -> 1.135 /
 # 2.134 ms, one request at 8,192 keys (64 ranges) 0.755 -> 0.740; but 8 requests at 768 / 2,048 /
 # 4,096 keys 0.846 / 0.932 / 1.024 -> 0.852 / 0.942 / 1.037 and one request at 768 keys 0.688 -> 0.705.
+# (Eight requests at 2,048 / 4,096 keys were measured again after the kernels had changed, together with
+# three to fifteen requests: see _SHARED_FEW_FROM.)
 _SHARED_MAX_HEAD_DIM = 128
 # Head size 128 (8 layers of the 8B sizes, ms a step, one wavefront a range -> this rule): 24 / 32
 # requests at 768 keys 1.194 / 1.213 -> 1.147 / 1.177 and 24 at 8,448 keys 2.281 -> 2.161, but 48
@@ -169,6 +180,23 @@ _SHARED_MIN_SPLITS = 64             # ... or from this many ranges
 _SHARED_MANY = 16                   # (8 ranges in two workgroups of four: 16 requests at 8,192 keys 1.550 -> 1.561 ms)
 _SHARED_MIN_WORKGROUPS = 192
 _SHARED_FEW_BYTES_CONTEXT = 8192
+# Between 16 and 128 pairs (three to fifteen requests on 8 kv heads) at contexts above 2,048 keys, and from
+# 48 pairs on above 1,024: four ranges to a workgroup and one workgroup per compute unit at most (a
+# 257th waits for a unit to come free: 7 requests at 8,100 keys in 20 ranges, 280 workgroups, 1.134
+# -> 1.237 ms; in 16 ranges, 224 workgroups, 1.111).  Whole decode steps, a wavefront a range -> this,
+# 3 / 4 / 5 / 6 / 7 requests: at 8,100 keys 1.008 / 1.034 / 1.047 / 1.087 / 1.134 -> 0.962 / 1.010 / 1.047 /
+# 1.086 / 1.111 ms, at 4,000 keys 0.884 / 0.924 / 0.947 / 0.984 / 1.000 -> 0.880 / 0.908 / 0.927 / 0.971 /
+# 0.982, at 2,000 keys 0.844 / 0.855 / 0.874 / 0.900 / 0.915 -> 0.850 / 0.867 / 0.886 / 0.884 / 0.894 (so
+# from 6 requests there), at 768 keys 0.825 / 0.828 / 0.830 / 0.837 / 0.845 -> 0.836 / 0.848 / 0.847 /
+# 0.848 / 0.851 (so not there).  The same up to 127 pairs (8 / 10 / 12 / 14 requests: at 2,000 keys 0.927 /
+# 0.982 / 1.025 / 1.044 -> 0.906 / 0.970 / 0.998 / 1.026, at 4,000 keys 1.025 / 1.088 / 1.126 / 1.185 -> 1.001 /
+# 1.094 / 1.117 / 1.164, at 8,100 keys 12 / 14 requests 1.369 / 1.471 -> 1.359 / 1.445); at 128 pairs (16
+# requests) 1.079 -> 1.063 at 2,000 keys but 1.204 / 1.530 -> 1.215 / 1.538 at 4,000 / 8,100: not there.
+_COMPUTE_UNITS = 256
+_SHARED_FEW_FROM = 16
+_SHARED_FEW_BELOW = 128
+_SHARED_FEW_CONTEXT = 2048
+_SHARED_FEW_PAIRS_MID = 48
 
 
 def choose_decode_ranges(num_items: int, num_kv_heads: int, max_context: int, head_dim: int,
@@ -187,6 +215,13 @@ def choose_decode_ranges(num_items: int, num_kv_heads: int, max_context: int, he
         splits, per = _cut_keys(4, max_context, 4)
         if splits in (2, 4):
             return splits, per, splits
+    if not wide and _SHARED_FEW_FROM < pairs < _SHARED_FEW_BELOW and (
+            max_context > _SHARED_FEW_CONTEXT or (max_context > _SHARED_SHORT_CONTEXT and pairs >= _SHARED_FEW_PAIRS_MID)):
+        # three to fifteen requests: as many workgroups of four ranges as there are compute units, no more
+        parts = min(_COMPUTE_UNITS // pairs, max_context // _MIN_KEYS_PER_SPLIT_DECODE // 4)
+        cut = _cut_keys_by_fours(4 * parts, max_context) if parts >= 2 else None
+        if cut is not None:
+            return cut[0], cut[1], 4
     if head_dim <= _SHARED_MAX_HEAD_DIM and not wide:
         # many ranges, four to a workgroup - if that still leaves a workgroup for most compute units
         # (one request at 32,768 / 131,072 keys: 64 ranges in 128 workgroups 0.979 / 1.616 ms, 128

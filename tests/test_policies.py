@@ -43,7 +43,8 @@ def test_key_ranges_of_decoded_tokens_and_the_wavefronts_that_share_them(nkv, it
     splits, per, waves = choose_decode_ranges(items, nkv, context, head_dim, KERNEL_MAX_SPLITS)
     assert 1 <= splits <= KERNEL_MAX_SPLITS and waves in (1, 2, 4) and splits % waves == 0
     if splits > 1:
-        assert per % 32 == 0 and splits * per >= context and (splits - 1) * per < context
+        # every key in a range, and no workgroup (of `waves` neighbouring ranges) without a key
+        assert per % 32 == 0 and splits * per >= context and (splits - waves) * per < context
     if head_dim > 128:
         assert waves == 1
 
@@ -57,13 +58,23 @@ def test_where_decoded_tokens_need_no_merge_launch():
     assert choose_decode_ranges(20, 8, 100, 64, KERNEL_MAX_SPLITS) == (2, 64, 2)
     # many ranges share a workgroup only where the merge has much to read
     assert choose_decode_ranges(8, 8, 8192, 64, KERNEL_MAX_SPLITS) == (16, 512, 4)
-    assert choose_decode_ranges(8, 8, 4096, 64, KERNEL_MAX_SPLITS) == (16, 256, 1)
+    assert choose_decode_ranges(8, 8, 768, 64, KERNEL_MAX_SPLITS) == (4, 192, 4)
+    # three to fifteen requests above 2,048 keys (from six requests on above 1,024): four ranges to a
+    # workgroup, and no more workgroups than compute units
+    assert choose_decode_ranges(8, 8, 4096, 64, KERNEL_MAX_SPLITS) == (16, 256, 4)
+    assert choose_decode_ranges(3, 8, 8192, 64, KERNEL_MAX_SPLITS) == (40, 224, 4)
+    assert choose_decode_ranges(7, 8, 8192, 64, KERNEL_MAX_SPLITS) == (16, 512, 4)          # 224 workgroups, not 280
+    assert choose_decode_ranges(12, 8, 2048, 64, KERNEL_MAX_SPLITS) == (8, 256, 4)
+    assert choose_decode_ranges(5, 8, 2048, 64, KERNEL_MAX_SPLITS)[2] == 1 and choose_decode_ranges(6, 8, 2048, 64, KERNEL_MAX_SPLITS)[2] == 4
+    assert choose_decode_ranges(5, 8, 768, 64, KERNEL_MAX_SPLITS)[2] == 1
+    assert choose_decode_ranges(16, 8, 4096, 64, KERNEL_MAX_SPLITS) == (8, 512, 1)
+    assert choose_decode_ranges(5, 8, 8192, 128, KERNEL_MAX_SPLITS)[2] == 1                 # head size 128: not measured
     assert choose_decode_ranges(1, 8, 8192, 64, KERNEL_MAX_SPLITS) == (64, 128, 4)
     assert choose_decode_ranges(1, 8, 768, 64, KERNEL_MAX_SPLITS) == (12, 64, 1)
     # short contexts: four ranges from 8 requests of 8 kv heads on
     assert choose_decode_ranges(8, 8, 768, 64, KERNEL_MAX_SPLITS) == (4, 192, 4)
     assert choose_decode_ranges(7, 8, 768, 64, KERNEL_MAX_SPLITS)[2] == 1
-    assert choose_decode_ranges(8, 8, 2048, 64, KERNEL_MAX_SPLITS) == (16, 128, 1)
+    assert choose_decode_ranges(8, 8, 2048, 64, KERNEL_MAX_SPLITS) == (16, 128, 4)
     assert choose_decode_ranges(32, 8, 768, 256, KERNEL_MAX_SPLITS)[2] == 1               # head size 256: one wavefront
     # one request and a long context: twice the ranges the merge kernel is given otherwise, four to a
     # workgroup, so that there is still a workgroup for every compute unit
