@@ -199,6 +199,36 @@ _SHARED_FEW_CONTEXT = 2048
 _SHARED_FEW_PAIRS_MID = 48
 
 
+# Long contexts, 17 to 63 requests on 8 kv heads: a workgroup of four ranges per (request, kv head)
+# pair is 136-504 workgroups, and the step waits for the compute units that got one more than the
+# others (264 workgroups: 8 units stream two pairs' keys while 248 stream one).  Two or three
+# workgroups a pair even that out at the price of partial results and the merge kernel.  Whole
+# decode steps at 8,100 keys, ms, one / two / three workgroups a pair: 17 requests 1.872 / 2.004 /
+# 1.800, 24: 1.974 / 2.100 / 2.180, 33: 2.914 / 2.720 / 2.640, 40: 3.045 / 2.840 / 2.808, 48: 3.170 /
+# 3.136 / 3.190, 56: 3.404 / 3.560 / 3.630; at 4,000 keys 17: 1.425 / 1.522 / 1.454, 33: 1.997 / 1.944 /
+# 1.984, 40: 2.062 / 2.021 / 2.104, 48: 2.140 / 2.139 / 2.305.  What fits them: the share of compute
+# units' turns that are used, workgroups / (256 * turns), divided by a price of 1 / 1.25 / 1.4 (up to
+# 4,096 keys, where the rest of the step weighs more: 1 / 1.3 / 1.6); the largest wins.  Checked at
+# batch sizes that were not used for it, four ranges a pair -> this: 18 / 36 / 44 requests at 8,100 keys
+# 1.866 / 2.965 / 3.135 -> 1.823 / 2.716 / 2.938 ms (20: 1.893 -> 1.909), at 16,000 keys 18 / 20 / 36 / 44:
+# 2.761 / 2.828 / 4.920 / 5.312 -> 2.559 / 2.705 / 4.316 / 4.762, at 4,000 keys 36 / 44: 2.025 / 2.125 ->
+# 1.988 / 2.075; 22, 28 and 52 requests keep one workgroup a pair.
+_GROUP_PRICE_LONG = (1.0, 1.25, 1.4)
+_GROUP_PRICE = (1.0, 1.3, 1.6)
+
+
+def _workgroups_a_pair(pairs: int, max_context: int) -> int:
+    price = _GROUP_PRICE if max_context <= _SHARED_LONG_CONTEXT else _GROUP_PRICE_LONG
+    best, best_score = 1, 0.0
+    for groups, cost in enumerate(price, start=1):
+        workgroups = pairs * groups
+        turns = (workgroups + _COMPUTE_UNITS - 1) // _COMPUTE_UNITS
+        score = workgroups / (turns * _COMPUTE_UNITS) / cost
+        if score > best_score * 1.0001:
+            best, best_score = groups, score
+    return best
+
+
 def choose_decode_ranges(num_items: int, num_kv_heads: int, max_context: int, head_dim: int,
                          max_splits: int = None) -> tuple:
     """(key ranges, keys per range, wavefronts per workgroup) for decoded tokens."""
@@ -210,6 +240,11 @@ def choose_decode_ranges(num_items: int, num_kv_heads: int, max_context: int, he
     frm = _SHARED_FOUR_FROM_SHORT if max_context <= _SHARED_SHORT_CONTEXT else _SHARED_FOUR_FROM
     if wide and frm < _SHARED_FOUR_FROM_SHORT_WIDE:
         frm = _SHARED_FOUR_FROM_SHORT_WIDE
+    if not wide and _SHARED_FOUR_FROM < pairs < _SHARED_FOUR_BELOW and max_context >= _SHARED_LONG_CONTEXT:
+        groups = _workgroups_a_pair(pairs, max_context)
+        cut = _cut_keys_by_fours(4 * groups, max_context) if groups > 1 else None
+        if cut is not None:
+            return cut[0], cut[1], 4
     if head_dim <= _SHARED_MAX_HEAD_DIM and frm < pairs < below \
             and max_context >= 4 * _MIN_KEYS_PER_SPLIT_DECODE:
         splits, per = _cut_keys(4, max_context, 4)

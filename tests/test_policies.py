@@ -182,3 +182,18 @@ def test_where_no_key_ranges_are_left_to_the_output_projection():
     assert choose_left_ranges(1, 768, 128, 4) is None           # measured at head sizes up to 64
     assert choose_left_ranges(1, 768, 64, 1) is None and choose_left_ranges(1, 768, 64, 0) is None
     assert choose_left_ranges(1, 768, 64, 2) == (8, 96, 4)
+
+
+def test_workgroups_a_pair_at_long_contexts_even_out_the_compute_units():
+    """17 to 63 requests on 8 kv heads at 4,096 keys or more: one workgroup of four ranges a pair
+    where that fills the compute units' turns well (192, 448 of 256), two or three where it
+    leaves most units idle in the last turn (264, 320 of 512)."""
+    from kv_cache_optimization_for_llm_amd.ops.attention import _workgroups_a_pair
+    assert [_workgroups_a_pair(p, 8192) for p in (136, 160, 176, 192, 264, 320, 384, 448, 504)] == [3, 3, 1, 1, 3, 3, 2, 1, 1]
+    assert [_workgroups_a_pair(p, 4096) for p in (136, 192, 264, 320, 384, 448)] == [1, 1, 2, 2, 2, 1]
+    assert choose_decode_ranges(33, 8, 8192, 64, KERNEL_MAX_SPLITS) == (12, 704, 4)
+    assert choose_decode_ranges(48, 8, 8192, 64, KERNEL_MAX_SPLITS) == (8, 1024, 4)
+    assert choose_decode_ranges(56, 8, 8192, 64, KERNEL_MAX_SPLITS) == (4, 2048, 4)
+    assert choose_decode_ranges(40, 8, 4096, 64, KERNEL_MAX_SPLITS) == (8, 512, 4)
+    assert choose_decode_ranges(40, 8, 2048, 64, KERNEL_MAX_SPLITS) == (4, 512, 4)          # shorter contexts: as before
+    assert choose_decode_ranges(40, 8, 131072, 64, KERNEL_MAX_SPLITS) == (12, 10944, 4)
