@@ -213,6 +213,8 @@ _SHARED_FEW_PAIRS_MID = 48
 # 1.866 / 2.965 / 3.135 -> 1.823 / 2.716 / 2.938 ms (20: 1.893 -> 1.909), at 16,000 keys 18 / 20 / 36 / 44:
 # 2.761 / 2.828 / 4.920 / 5.312 -> 2.559 / 2.705 / 4.316 / 4.762, at 4,000 keys 36 / 44: 2.025 / 2.125 ->
 # 1.988 / 2.075; 22, 28 and 52 requests keep one workgroup a pair.
+# Below 4,096 keys one workgroup a pair stays: two / three at 768 keys took 33-56 requests from 1.22-1.35
+# to 1.28-1.45 / 1.30-1.52 ms, at 2,000 keys from 1.51-1.71 to 1.52-1.81 / 1.50-1.83.
 _GROUP_PRICE_LONG = (1.0, 1.25, 1.4)
 _GROUP_PRICE = (1.0, 1.3, 1.6)
 
