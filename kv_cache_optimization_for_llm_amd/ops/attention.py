@@ -215,6 +215,8 @@ _SHARED_FEW_PAIRS_MID = 48
 # 1.988 / 2.075; 22, 28 and 52 requests keep one workgroup a pair.
 # Below 4,096 keys one workgroup a pair stays: two / three at 768 keys took 33-56 requests from 1.22-1.35
 # to 1.28-1.45 / 1.30-1.52 ms, at 2,000 keys from 1.51-1.71 to 1.52-1.81 / 1.50-1.83.
+# From 512 pairs on (64 requests and more) two workgroups a pair at 8,100 keys: 72 / 104 requests 4.73 /
+# 6.12 -> 4.54 / 5.98 ms, 80 a tie, 64 / 88 / 120 slower by 2-3 %; at 4,000 keys nothing gained: one stays.
 _GROUP_PRICE_LONG = (1.0, 1.25, 1.4)
 _GROUP_PRICE = (1.0, 1.3, 1.6)
 
