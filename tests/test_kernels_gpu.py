@@ -650,6 +650,65 @@ def test_attention_of_one_decoded_token_over_a_very_long_context(nkv, ctx, gpu):
                          torch.tensor([ctx - 1], dtype=torch.int32, device=gpu), nq, nkv, d, 1 / 8.0, 0, 512, 256)
 
 
+@pytest.mark.parametrize("items, ctx", [(5, 5000), (12, 2500), (20, 4200), (36, 8300), (7, 8192), (3, 9000)])
+def test_several_decoded_tokens_over_long_contexts_with_the_ranges_the_policy_picks(items, ctx, gpu):
+    """3 to 63 requests with thousands of keys each (8 kv heads, heads of 64): the policy gives
+    every (request, kv head) pair one to ten workgroups of four neighbouring key ranges, some
+    ranges of the shorter requests hold no key, and more than one workgroup a pair goes through
+    the merge kernel.  Contexts differ per request; in each, one key at a place of its own is made
+    to dominate one head, so a range that is dropped, counted twice or given to the wrong request
+    shows.  Against every request's last row of plain attention."""
+    from kv_cache_optimization_for_llm_amd.ops.attention import choose_decode_ranges
+    nq, nkv, d, page = 16, 8, 64, 16
+    g = torch.Generator().manual_seed(items * 7 + ctx)
+    lens = [ctx] + [int(x) for x in torch.randint(ctx // 3, ctx + 1, (items - 1,), generator=g)]
+    bucket = 1 << (ctx - 1).bit_length()
+    splits, per, waves = choose_decode_ranges(items, nkv, bucket, d)
+    assert waves == 4 and splits % 4 == 0 and splits >= 8, "the shapes of this test are the ones that share workgroups"
+    pages_each = [(n + page - 1) // page for n in lens]
+    total = sum(pages_each)
+    perm = torch.randperm(total, generator=g)
+    kc = torch.zeros(total, nkv, page, d, dtype=torch.bfloat16)
+    vc = torch.zeros(total, nkv, d, page, dtype=torch.bfloat16)
+    table = torch.zeros(items, max(pages_each), dtype=torch.int32)
+    qkv = torch.zeros(items, (nq + 2 * nkv) * d, dtype=torch.bfloat16)
+    want = torch.empty(items, nq * d)
+    at = 0
+    for i, n in enumerate(lens):
+        k = torch.randn(n, nkv, d, generator=g) * 0.1
+        v = torch.randn(n, nkv, d, generator=g)
+        q = torch.randn(nq, d, generator=g) * 0.1
+        far = (n * (i + 1) // (items + 1)) // per * per           # the first key of some range, another one per request
+        k[far] = 0
+        k[far, i % nkv, 5] = 12.0
+        q[(i % nkv) * 2, 5] = 12.0
+        k, v, q = (t.to(torch.bfloat16) for t in (k, v, q))
+        mine = perm[at:at + pages_each[i]]
+        at += pages_each[i]
+        pad = pages_each[i] * page - n
+        kp = torch.cat([k, torch.zeros(pad, nkv, d, dtype=torch.bfloat16)]).view(-1, page, nkv, d)
+        vp = torch.cat([v, torch.zeros(pad, nkv, d, dtype=torch.bfloat16)]).view(-1, page, nkv, d)
+        kc[mine] = kp.permute(0, 2, 1, 3)
+        vc[mine] = vp.permute(0, 2, 3, 1)
+        table[i, :pages_each[i]] = mine.to(torch.int32)
+        qkv[i, :nq * d] = q.reshape(-1)
+        kf, vf = k.float().to(gpu), v.float().to(gpu)
+        for h in range(nq):
+            kh = h // (nq // nkv)
+            p = torch.softmax((kf[:, kh] @ q[h].float().to(gpu) / 8.0).double(), 0).float()
+            want[i, h * d:(h + 1) * d] = (p @ vf[:, kh]).cpu()
+        h = (i % nkv) * 2
+        assert (want[i, h * d:(h + 1) * d] - v[far, i % nkv].float()).abs().max() < 0.3       # that key dominates its head
+    out = torch.empty(items, nq * d, dtype=torch.bfloat16, device=gpu)
+    idx = torch.arange(items, dtype=torch.int32, device=gpu)
+    K.attention_mfma(qkv.to(gpu), qkv.shape[1], out, K.keys_to_pages(kc).to(gpu), vc.to(gpu), table.to(gpu),
+                     idx, torch.zeros(items, dtype=torch.int32, device=gpu), idx,
+                     torch.arange(items + 1, dtype=torch.int32, device=gpu),
+                     torch.tensor([n - 1 for n in lens], dtype=torch.int32, device=gpu), nq, nkv, d, 1 / 8.0, 0,
+                     splits, per, waves=waves)
+    close(out, want, torch.bfloat16, f"{items} requests of up to {ctx} keys in {splits} ranges of {per}", tol16=8e-3)
+
+
 def test_choose_splits():
     assert choose_splits(4096, 8, 2048) == (1, 0)                 # a big prompt fills the GPU by itself
     s, per = choose_splits(1, 8, 8192)
